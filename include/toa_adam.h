@@ -1,0 +1,150 @@
+/*
+ * toa_adam.h -- C ABI of the MI355X (gfx950) fused Adam operator library
+ * (libtoa_adam.so).
+ *
+ * This is the boundary a host binding attaches to: plain device pointers,
+ * element counts, the Python-level hyper-parameters as double, the step
+ * number as an unsigned 64-bit integer and an opaque HIP stream.  No torch
+ * types appear.  Each entry point replaces one device launcher of the
+ * reference (declared in /root/reference/include/adam_op/adam_op_impl_cuda.cuh,
+ * dispatched from /root/reference/src/adam_op/adam_op.cpp) with the tensors
+ * replaced by (pointer, n, dtype).
+ *
+ * Conventions
+ *   dtype     TOA_F32 or TOA_F64; all arrays of one call share it.
+ *   pointers  device memory on the CURRENT HIP device, contiguous, n elements
+ *             each.  Any alignment is accepted; 16-byte aligned pointers take
+ *             the 128-bit path.  In toa_adam_forward_inplace the three arrays
+ *             may alias one another completely (the reference's availability
+ *             probe does that with n = 1).
+ *   scalars   b1, b2, eps, eps_root arrive as double and are rounded to the
+ *             element type inside the library; the bias corrections
+ *             1/(1-b^count) etc. are formed in double first and then rounded,
+ *             exactly as the reference launchers do.
+ *   stream    a hipStream_t passed as void*; NULL is the device's null stream.
+ *             Calls only enqueue work; they never synchronise.
+ *   n == 0    is a successful no-op (no launch).
+ *   return    0 on success; a positive value is a hipError_t from the launch;
+ *             a negative value is one of the TOA_E* argument errors below.
+ *             toa_adam_error_string() names either kind.
+ *   threads   re-entrant; no global state except a per-device cache of the
+ *             compute-unit count.
+ */
+#ifndef TOA_ADAM_H
+#define TOA_ADAM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TOA_API __attribute__((visibility("default")))
+
+enum { TOA_F32 = 0, TOA_F64 = 1 };
+
+enum {
+    TOA_EDTYPE = -1, /* dtype is not TOA_F32 / TOA_F64            */
+    TOA_ENULL = -2,  /* a required pointer is NULL while n > 0    */
+    TOA_ESIZE = -3   /* a tensor is too large for the launch grid */
+};
+
+/* Library ABI version (bumped on any signature change). */
+TOA_API int toa_adam_abi_version(void);
+
+/* Human-readable name of a return code from any function below. */
+TOA_API const char *toa_adam_error_string(int code);
+
+/* ---- single-tensor entry points ---------------------------------------- */
+
+/* Fused in-place step: mu, nu and updates are read once and overwritten.
+ * Replaces adamForwardInplaceCUDA (adam_op_impl_cuda.cuh:26-33, called from
+ * adam_op.cpp:41-43; arithmetic contract adam_op_impl_cpu.cpp:32-91). */
+TOA_API int toa_adam_forward_inplace(int dtype, void *updates, void *mu, void *nu, size_t n, double b1,
+                             double b2, double eps, double eps_root, uint64_t count,
+                             void *stream);
+
+/* mu_out = b1*mu + (1-b1)*updates.  Replaces adamForwardMuCUDA
+ * (adam_op_impl_cuda.cuh:35-37, adam_op.cpp:56-58; adam_op_impl_cpu.cpp:93-125). */
+TOA_API int toa_adam_forward_mu(int dtype, const void *updates, const void *mu, size_t n, double b1,
+                        void *mu_out, void *stream);
+
+/* nu_out = b2*nu + (1-b2)*updates^2.  Replaces adamForwardNuCUDA
+ * (adam_op_impl_cuda.cuh:39-41, adam_op.cpp:71-73; adam_op_impl_cpu.cpp:127-160). */
+TOA_API int toa_adam_forward_nu(int dtype, const void *updates, const void *nu, size_t n, double b2,
+                        void *nu_out, void *stream);
+
+/* updates_out = mu_hat / (sqrt(nu_hat + eps_root) + eps).  Replaces
+ * adamForwardUpdatesCUDA (adam_op_impl_cuda.cuh:43-49, adam_op.cpp:90-92;
+ * adam_op_impl_cpu.cpp:162-209). */
+TOA_API int toa_adam_forward_updates(int dtype, const void *new_mu, const void *new_nu, size_t n,
+                             double b1, double b2, double eps, double eps_root, uint64_t count,
+                             void *updates_out, void *stream);
+
+/* dupdates_out = (1-b1)*dmu, dmu_out = b1*dmu.  Replaces adamBackwardMuCUDA
+ * (adam_op_impl_cuda.cuh:51-54, adam_op.cpp:106-108; adam_op_impl_cpu.cpp:211-245). */
+TOA_API int toa_adam_backward_mu(int dtype, const void *dmu, size_t n, double b1, void *dupdates_out,
+                         void *dmu_out, void *stream);
+
+/* dupdates_out = 2*(1-b2)*updates*dnu, dnu_out = b2*dnu.  Replaces
+ * adamBackwardNuCUDA (adam_op_impl_cuda.cuh:56-59, adam_op.cpp:122-124;
+ * adam_op_impl_cpu.cpp:247-284). */
+TOA_API int toa_adam_backward_nu(int dtype, const void *dnu, const void *updates, size_t n, double b2,
+                         void *dupdates_out, void *dnu_out, void *stream);
+
+/* Reference's hand-derived VJP of forward_updates; `updates` is the forward
+ * OUTPUT.  Replaces adamBackwardUpdatesCUDA (adam_op_impl_cuda.cuh:61-68,
+ * adam_op.cpp:142-145; adam_op_impl_cpu.cpp:286-347). */
+TOA_API int toa_adam_backward_updates(int dtype, const void *dupdates, const void *updates,
+                              const void *new_mu, size_t n, double b1, double b2,
+                              double eps_root, uint64_t count, void *dnew_mu_out,
+                              void *dnew_nu_out, void *stream);
+
+/* ---- multi-tensor entry points ------------------------------------------
+ * One call covers a whole list of tensors (a flattened pytree): the host loop
+ * the reference runs per leaf (/root/reference/torchopt/transform/
+ * scale_by_adam.py:325-332, 378-385) collapses into one launch per
+ * TOA_MT_MAX_TENSORS(...) tensors that share a step count.  The arrays of
+ * pointers, lengths and counts are HOST arrays of num_tensors entries; they
+ * are consumed before the call returns.  counts may be NULL when count_all
+ * applies to every tensor.  Zero-length tensors are skipped. */
+
+TOA_API int toa_adam_forward_inplace_multi(int dtype, size_t num_tensors, void *const *updates,
+                                   void *const *mu, void *const *nu, const size_t *n, double b1,
+                                   double b2, double eps, double eps_root,
+                                   const uint64_t *counts, uint64_t count_all, void *stream);
+
+TOA_API int toa_adam_forward_mu_multi(int dtype, size_t num_tensors, const void *const *updates,
+                              const void *const *mu, const size_t *n, double b1,
+                              void *const *mu_out, void *stream);
+
+TOA_API int toa_adam_forward_nu_multi(int dtype, size_t num_tensors, const void *const *updates,
+                              const void *const *nu, const size_t *n, double b2,
+                              void *const *nu_out, void *stream);
+
+TOA_API int toa_adam_forward_updates_multi(int dtype, size_t num_tensors, const void *const *new_mu,
+                                   const void *const *new_nu, const size_t *n, double b1,
+                                   double b2, double eps, double eps_root,
+                                   const uint64_t *counts, uint64_t count_all,
+                                   void *const *updates_out, void *stream);
+
+TOA_API int toa_adam_backward_mu_multi(int dtype, size_t num_tensors, const void *const *dmu,
+                               const size_t *n, double b1, void *const *dupdates_out,
+                               void *const *dmu_out, void *stream);
+
+TOA_API int toa_adam_backward_nu_multi(int dtype, size_t num_tensors, const void *const *dnu,
+                               const void *const *updates, const size_t *n, double b2,
+                               void *const *dupdates_out, void *const *dnu_out, void *stream);
+
+TOA_API int toa_adam_backward_updates_multi(int dtype, size_t num_tensors, const void *const *dupdates,
+                                    const void *const *updates, const void *const *new_mu,
+                                    const size_t *n, double b1, double b2, double eps_root,
+                                    const uint64_t *counts, uint64_t count_all,
+                                    void *const *dnew_mu_out, void *const *dnew_nu_out,
+                                    void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TOA_ADAM_H */

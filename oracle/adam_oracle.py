@@ -1,0 +1,138 @@
+"""ctypes front-end of the C oracle (liboracle_adam.so) on NumPy arrays.
+
+TEST INFRASTRUCTURE, NOT PRODUCT: only tests, the smoke check and the
+CPU-baseline leg of the benchmark may import this module.  The shipped operator
+(torchopt_amd) never does.
+
+`load_reference()` additionally loads, where it has been built, the reference's
+own compiled CPU op (oracle/_ref/_C*.so, built by `make -C oracle ref` from the
+sources under /root/reference) as a Python module exposing `adam_op.forward_`
+and friends on CPU torch tensors.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import glob
+import importlib.util
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, 'liboracle_adam.so')
+
+_SFX = {np.dtype(np.float32): 'f32', np.dtype(np.float64): 'f64'}
+_CT = {np.dtype(np.float32): ctypes.c_float, np.dtype(np.float64): ctypes.c_double}
+
+_lib = None
+
+
+def build(force: bool = False) -> str:
+    """Compile the C oracle (gcc, a second or two)."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.run(['make', '-C', _HERE, '--no-print-directory'], check=True,
+                   stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+        _lib.oracle_adam_threads_for.restype = ctypes.c_int
+        _lib.oracle_adam_threads_for.argtypes = [ctypes.c_size_t]
+    return _lib
+
+
+def _ptr(a: np.ndarray):
+    assert a.flags['C_CONTIGUOUS'] and a.dtype in _SFX
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _fn(name: str, dtype):
+    return getattr(lib(), f'oracle_adam_{name}_{_SFX[np.dtype(dtype)]}')
+
+
+_D = ctypes.c_double
+_U64 = ctypes.c_uint64
+_SZ = ctypes.c_size_t
+
+
+def host_scalars(b1, b2, eps_root, count):
+    out = (ctypes.c_double * 4)()
+    lib().oracle_adam_host_scalars(_D(b1), _D(b2), _D(eps_root), _U64(count), out)
+    return tuple(out)
+
+
+def threads_for(n: int) -> int:
+    return lib().oracle_adam_threads_for(n)
+
+
+def forward_inplace(updates, mu, nu, b1, b2, eps, eps_root, count):
+    """Mutates the three arrays, like `forward_`."""
+    _fn('forward_inplace', updates.dtype)(_ptr(updates), _ptr(mu), _ptr(nu), _SZ(updates.size),
+                                          _D(b1), _D(b2), _D(eps), _D(eps_root), _U64(count))
+    return updates, mu, nu
+
+
+def forward_mu(updates, mu, b1):
+    out = np.empty_like(mu)
+    _fn('forward_mu', updates.dtype)(_ptr(updates), _ptr(mu), _SZ(updates.size), _D(b1), _ptr(out))
+    return out
+
+
+def forward_nu(updates, nu, b2):
+    out = np.empty_like(nu)
+    _fn('forward_nu', updates.dtype)(_ptr(updates), _ptr(nu), _SZ(updates.size), _D(b2), _ptr(out))
+    return out
+
+
+def forward_updates(new_mu, new_nu, b1, b2, eps, eps_root, count):
+    out = np.empty_like(new_mu)
+    _fn('forward_updates', new_mu.dtype)(_ptr(new_mu), _ptr(new_nu), _SZ(new_mu.size), _D(b1),
+                                         _D(b2), _D(eps), _D(eps_root), _U64(count), _ptr(out))
+    return out
+
+
+def backward_mu(dmu, b1):
+    du, dm = np.empty_like(dmu), np.empty_like(dmu)
+    _fn('backward_mu', dmu.dtype)(_ptr(dmu), _SZ(dmu.size), _D(b1), _ptr(du), _ptr(dm))
+    return du, dm
+
+
+def backward_nu(dnu, updates, b2):
+    du, dn = np.empty_like(dnu), np.empty_like(dnu)
+    _fn('backward_nu', dnu.dtype)(_ptr(dnu), _ptr(updates), _SZ(dnu.size), _D(b2), _ptr(du),
+                                  _ptr(dn))
+    return du, dn
+
+
+def backward_updates(dupdates, updates, new_mu, b1, b2, eps_root, count):
+    dm, dn = np.empty_like(dupdates), np.empty_like(dupdates)
+    _fn('backward_updates', dupdates.dtype)(_ptr(dupdates), _ptr(updates), _ptr(new_mu),
+                                            _SZ(dupdates.size), _D(b1), _D(b2), _D(eps_root),
+                                            _U64(count), _ptr(dm), _ptr(dn))
+    return dm, dn
+
+
+def reference_path():
+    hits = sorted(glob.glob(os.path.join(_HERE, '_ref', '_C*.so')))
+    return hits[0] if hits else None
+
+
+def load_reference():
+    """Import the compiled reference CPU op, or return None if it was not built."""
+    path = reference_path()
+    if path is None:
+        return None
+    import torch  # noqa: F401  (libtorch must be loaded first)
+
+    spec = importlib.util.spec_from_file_location('_C', path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod

@@ -1,0 +1,308 @@
+"""The CPU oracle is pinned here, on CPU, before anything is compared with it on the GPU.
+
+Three independent statements of the arithmetic must agree bit for bit:
+  1. the golden vectors written by the reference's own compiled CPU op (tests/golden);
+  2. the plain-C restatement (oracle/adam_oracle.c) -- the oracle the GPU tests use;
+  3. the NumPy one-rounding-per-operation specification (oracle/adam_spec.py);
+and, where oracle/_ref has been built, 4. the compiled reference itself on fresh inputs.
+Closed forms and invariants that the mathematics fixes come last; each is chosen so that a
+plausible slip (dropped term, wrong sign, swapped operand, fused multiply-add, scalar rounded
+at the wrong point) breaks it.
+"""
+
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import pytest
+
+from conftest import assert_bit_equal, hyper_of, load_golden
+from oracle import adam_oracle as O
+from oracle import adam_spec as S
+
+DTYPES = [np.float32, np.float64]
+TAG = {np.float32: 'f32', np.float64: 'f64'}
+
+
+def _cases(dtype):
+    return sorted(load_golden(TAG[dtype]).items())
+
+
+def _ids(dtype):
+    return [f'{TAG[dtype]}-{name}' for name, _ in _cases(dtype)]
+
+
+ALL_CASES = [(dt, name, case) for dt in DTYPES for name, case in _cases(dt)]
+ALL_IDS = [f'{TAG[dt]}-{name}' for dt, name, _ in ALL_CASES]
+
+
+@pytest.mark.parametrize('dtype,name,case', ALL_CASES, ids=ALL_IDS)
+@pytest.mark.parametrize('impl', [O, S], ids=['c_oracle', 'numpy_spec'])
+def test_against_reference_golden(impl, dtype, name, case):
+    b1, b2, eps, eps_root, count = hyper_of(case)
+    u, mu, nu = case['updates'], case['mu'], case['nu']
+    with np.errstate(all='ignore'):
+        assert_bit_equal(impl.forward_mu(u, mu, b1), case['new_mu'], 'forward_mu')
+        assert_bit_equal(impl.forward_nu(u, nu, b2), case['new_nu'], 'forward_nu')
+        assert_bit_equal(
+            impl.forward_updates(case['new_mu'], case['new_nu'], b1, b2, eps, eps_root, count),
+            case['new_updates'], 'forward_updates')
+        iu, im, iv = impl.forward_inplace(u.copy(), mu.copy(), nu.copy(), b1, b2, eps, eps_root,
+                                          count)
+        assert_bit_equal(iu, case['inplace_updates'], 'forward_ updates')
+        assert_bit_equal(im, case['inplace_mu'], 'forward_ mu')
+        assert_bit_equal(iv, case['inplace_nu'], 'forward_ nu')
+        du, dm = impl.backward_mu(case['dmu'], b1)
+        assert_bit_equal(du, case['bmu_dupdates'], 'backward_mu dupdates')
+        assert_bit_equal(dm, case['bmu_dmu'], 'backward_mu dmu')
+        du, dn = impl.backward_nu(case['dnu'], u, b2)
+        assert_bit_equal(du, case['bnu_dupdates'], 'backward_nu dupdates')
+        assert_bit_equal(dn, case['bnu_dnu'], 'backward_nu dnu')
+        dm, dn = impl.backward_updates(case['dupdates'], case['new_updates'], case['new_mu'],
+                                       b1, b2, eps_root, count)
+        assert_bit_equal(dm, case['bup_dnew_mu'], 'backward_updates dnew_mu')
+        assert_bit_equal(dn, case['bup_dnew_nu'], 'backward_updates dnew_nu')
+
+
+@pytest.mark.parametrize('dtype', DTYPES, ids=['f32', 'f64'])
+def test_golden_internal_consistency(dtype):
+    """In the reference's own outputs the fused step equals the three split ops chained."""
+    for name, case in _cases(dtype):
+        assert_bit_equal(case['inplace_mu'], case['new_mu'], name)
+        assert_bit_equal(case['inplace_nu'], case['new_nu'], name)
+        assert_bit_equal(case['inplace_updates'], case['new_updates'], name)
+
+
+def _rand(dtype, n, seed):
+    rng = np.random.default_rng(seed)
+    return (rng.standard_normal(n).astype(dtype), (0.1 * rng.standard_normal(n)).astype(dtype),
+            np.abs(0.01 * rng.standard_normal(n)).astype(dtype))
+
+
+@pytest.mark.parametrize('dtype', DTYPES, ids=['f32', 'f64'])
+@pytest.mark.parametrize('n', [0, 1, 3, 999, 1000, 1001, 4097, 300_007])
+def test_c_oracle_equals_numpy_spec(dtype, n):
+    """Sizes on both sides of the serial/OpenMP switch; threads must not change a bit."""
+    u, mu, nu = _rand(dtype, n, 11 + n)
+    rng = np.random.default_rng(n)
+    d1, d2, d3 = (rng.standard_normal(n).astype(dtype) for _ in range(3))
+    for b1, b2, eps, eps_root, count in [(0.9, 0.999, 1e-8, 0.0, 1), (0.9, 0.999, 1e-8, 1e-8, 5),
+                                         (0.8, 0.95, 1e-6, 1e-10, 77)]:
+        su, sm, sv = S.forward_inplace(u, mu, nu, b1, b2, eps, eps_root, count)
+        ou, om, ov = O.forward_inplace(u.copy(), mu.copy(), nu.copy(), b1, b2, eps, eps_root,
+                                       count)
+        for a, b, w in ((ou, su, 'u'), (om, sm, 'mu'), (ov, sv, 'nu')):
+            assert_bit_equal(a, b, f'forward_ {w}')
+        assert_bit_equal(O.forward_mu(u, mu, b1), sm)
+        assert_bit_equal(O.forward_nu(u, nu, b2), sv)
+        assert_bit_equal(O.forward_updates(sm, sv, b1, b2, eps, eps_root, count), su)
+        for a, b in zip(O.backward_mu(d1, b1), S.backward_mu(d1, b1)):
+            assert_bit_equal(a, b, 'backward_mu')
+        for a, b in zip(O.backward_nu(d2, u, b2), S.backward_nu(d2, u, b2)):
+            assert_bit_equal(a, b, 'backward_nu')
+        sm0 = sm.copy()
+        if n:
+            sm0[::5] = 0
+        for a, b in zip(O.backward_updates(d3, su, sm0, b1, b2, eps_root, count),
+                        S.backward_updates(d3, su, sm0, b1, b2, eps_root, count)):
+            assert_bit_equal(a, b, 'backward_updates')
+
+
+@pytest.mark.parametrize('dtype', DTYPES, ids=['f32', 'f64'])
+def test_c_oracle_equals_compiled_reference(dtype):
+    """Fresh inputs, a size that gives the reference several OpenMP threads."""
+    ref = O.load_reference()
+    if ref is None:
+        pytest.skip('oracle/_ref not built (needs the reference sources; `make -C oracle ref`)')
+    import torch
+
+    n = 1_000_003
+    u, mu, nu = _rand(dtype, n, 5)
+    rng = np.random.default_rng(6)
+    d1, d2, d3 = (rng.standard_normal(n).astype(dtype) for _ in range(3))
+    tn = torch.from_numpy
+    op = ref.adam_op
+    for b1, b2, eps, eps_root, count in [(0.9, 0.999, 1e-8, 0.0, 10), (0.9, 0.999, 1e-8, 1e-8, 3)]:
+        ru, rm, rv = (x.copy() for x in (u, mu, nu))
+        op.forward_(tn(ru), tn(rm), tn(rv), b1, b2, eps, eps_root, count)
+        ou, om, ov = O.forward_inplace(u.copy(), mu.copy(), nu.copy(), b1, b2, eps, eps_root,
+                                       count)
+        assert_bit_equal(ou, ru), assert_bit_equal(om, rm), assert_bit_equal(ov, rv)
+        assert_bit_equal(O.forward_mu(u, mu, b1), op.forward_mu(tn(u), tn(mu), b1).numpy())
+        assert_bit_equal(O.forward_nu(u, nu, b2), op.forward_nu(tn(u), tn(nu), b2).numpy())
+        assert_bit_equal(O.forward_updates(rm, rv, b1, b2, eps, eps_root, count),
+                         op.forward_updates(tn(rm), tn(rv), b1, b2, eps, eps_root, count).numpy())
+        for a, b in zip(O.backward_mu(d1, b1), op.backward_mu(tn(d1), tn(u), tn(mu), b1)):
+            assert_bit_equal(a, b.numpy())
+        for a, b in zip(O.backward_nu(d2, u, b2), op.backward_nu(tn(d2), tn(u), tn(nu), b2)):
+            assert_bit_equal(a, b.numpy())
+        rm0 = rm.copy()
+        rm0[::9] = 0
+        for a, b in zip(O.backward_updates(d3, ru, rm0, b1, b2, eps_root, count),
+                        op.backward_updates(tn(d3), tn(ru), tn(rm0), tn(rv), b1, b2, eps_root,
+                                            count)):
+            assert_bit_equal(a, b.numpy())
+
+
+# ---------------------------------------------------------------------------------------------
+# What the mathematics fixes
+# ---------------------------------------------------------------------------------------------
+
+
+def test_host_scalars_closed_form():
+    for b1, b2, er, c in [(0.9, 0.999, 0.0, 1), (0.9, 0.999, 1e-8, 5), (0.5, 0.25, 0.0, 3)]:
+        c1, c2, p1, q2 = O.host_scalars(b1, b2, er, c)
+        assert c1 == 1.0 / (1.0 - math.pow(b1, c))
+        assert c2 == 1.0 / (1.0 - math.pow(b2, c))
+        assert p1 == 1.0 - math.pow(b1, c)
+        assert q2 == 1.0 / (1.0 - math.pow(b2, c) + er)
+    # exactly representable: b = 0.5, count = 3 -> 1/(1 - 1/8) and 7/8
+    c1, _, p1, _ = O.host_scalars(0.5, 0.5, 0.0, 3)
+    assert p1 == 0.875 and c1 == 1.0 / 0.875
+    assert S.host_scalars(0.9, 0.999, 1e-8, 1000) == O.host_scalars(0.9, 0.999, 1e-8, 1000)
+
+
+def test_fp32_one_minus_beta_is_formed_in_float():
+    """1.0f - 0.999f is 9.9998713e-4, not float(1 - 0.999) = 1.00000005e-3: with nu = 0 the
+    new nu is exactly that factor times g*g (g = 1)."""
+    one = np.ones(4, np.float32)
+    zero = np.zeros(4, np.float32)
+    out = O.forward_nu(one, zero, 0.999)
+    want = np.float32(1) - np.float32(0.999)
+    assert out[0] == want and out[0] != np.float32(1.0 - 0.999)
+    out = O.forward_mu(one, zero, 0.9)
+    assert out[0] == np.float32(1) - np.float32(0.9) and out[0] != np.float32(1.0 - 0.9)
+
+
+def test_no_fused_multiply_add():
+    """b1*m + (1-b1)*g with b1 = 0.5: choose m, g whose products are inexact in float so that a
+    fused multiply-add (one rounding) and mul-then-add (two roundings) differ."""
+    rng = np.random.default_rng(3)
+    m = rng.standard_normal(4096).astype(np.float32)
+    g = (-m * np.float32(1 + 2 ** -12)).astype(np.float32)  # near-cancellation
+    b1 = 0.7
+    out = O.forward_mu(g, m, b1)
+    beta = np.float32(b1)
+    two_step = (beta * m) + ((np.float32(1) - beta) * g)
+    fused = (np.float64(beta) * m.astype(np.float64)
+             + np.float64(np.float32(1) - beta) * g.astype(np.float64)).astype(np.float32)
+    assert_bit_equal(out, two_step)
+    assert np.any(two_step != fused)  # the case does discriminate
+
+
+@pytest.mark.parametrize('dtype', DTYPES, ids=['f32', 'f64'])
+def test_first_step_from_zero_state_is_sign(dtype):
+    """count = 1, mu = nu = 0, eps_root = 0: update = g / (|g| + eps) ~ sign(g)."""
+    g = np.array([3.0, -2.0, 0.5, -1e-3, 1e3], dtype)
+    z = np.zeros_like(g)
+    u, m, v = O.forward_inplace(g.copy(), z.copy(), z.copy(), 0.9, 0.999, 1e-8, 0.0, 1)
+    tol = 8 * np.finfo(dtype).eps
+    # in float, 1.0f - 0.999f is off from 0.001 by 1.3e-5 relative, and c2 = 1000 undoes it only
+    # in exact arithmetic: the step is sign(g) to half of that
+    np.testing.assert_allclose(u, g / (np.abs(g) + dtype(1e-8)),
+                               rtol=1e-5 if dtype == np.float32 else tol)
+    np.testing.assert_allclose(m, (1 - 0.9) * g, rtol=tol)
+    np.testing.assert_allclose(v, (1 - 0.999) * g * g, rtol=2e-5 if dtype == np.float32 else tol)
+
+
+@pytest.mark.parametrize('dtype', DTYPES, ids=['f32', 'f64'])
+def test_forward_matches_high_precision_formula(dtype):
+    """Against the textbook formula evaluated in extended precision."""
+    u, mu, nu = _rand(dtype, 2000, 21)
+    b1, b2, eps, er, c = 0.9, 0.999, 1e-8, 1e-8, 7
+    ou, om, ov = O.forward_inplace(u.copy(), mu.copy(), nu.copy(), b1, b2, eps, er, c)
+    L = np.longdouble
+    beta1, beta2 = L(dtype(b1)), L(dtype(b2))
+    m1 = beta1 * L(mu) + (1 - beta1) * L(u)
+    v1 = beta2 * L(nu) + (1 - beta2) * L(u) * L(u)
+    up = (m1 / (1 - L(b1) ** c)) / (np.sqrt(v1 / (1 - L(b2) ** c) + L(er)) + L(eps))
+    e = np.finfo(dtype).eps
+    # cancellation in m1 costs absolute, not relative, accuracy
+    np.testing.assert_allclose(om.astype(L), m1, rtol=0, atol=4 * e * (np.abs(mu).max() + 1))
+    np.testing.assert_allclose(ov.astype(L), v1, rtol=8 * e)
+    np.testing.assert_allclose(ou.astype(L), up, rtol=0, atol=64 * e * np.abs(up).max())
+
+
+@pytest.mark.parametrize('dtype', DTYPES, ids=['f32', 'f64'])
+def test_backward_mu_nu_are_the_analytic_vjps(dtype):
+    """d(new_mu)/d(updates) = 1-b1, d/d(mu) = b1; d(new_nu)/d(updates) = 2(1-b2)g, d/d(nu) = b2
+    -- checked against central differences of the oracle's own forward in float64."""
+    rng = np.random.default_rng(5)
+    n = 64
+    g, m, v = _rand(np.float64, n, 9)
+    ct = rng.standard_normal(n)
+    h = 1e-6
+    fd_g = (O.forward_mu(g + h, m, 0.9) - O.forward_mu(g - h, m, 0.9)) / (2 * h) * ct
+    fd_m = (O.forward_mu(g, m + h, 0.9) - O.forward_mu(g, m - h, 0.9)) / (2 * h) * ct
+    du, dm = O.backward_mu(ct.astype(dtype), 0.9)
+    tol = 1e-5 if dtype == np.float32 else 1e-8
+    np.testing.assert_allclose(du, fd_g, rtol=tol, atol=tol)
+    np.testing.assert_allclose(dm, fd_m, rtol=tol, atol=tol)
+    fd_g = (O.forward_nu(g + h, v, 0.999) - O.forward_nu(g - h, v, 0.999)) / (2 * h) * ct
+    fd_v = (O.forward_nu(g, v + h, 0.999) - O.forward_nu(g, v - h, 0.999)) / (2 * h) * ct
+    du, dv = O.backward_nu(ct.astype(dtype), g.astype(dtype), 0.999)
+    np.testing.assert_allclose(du, fd_g, rtol=10 * tol, atol=10 * tol)
+    np.testing.assert_allclose(dv, fd_v, rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize('dtype', DTYPES, ids=['f32', 'f64'])
+def test_backward_updates_structure(dtype):
+    """The reference's backward of forward_updates is a hand-derived formula, not the exact
+    derivative; what is fixed: dnew_mu * new_mu == dupdates * updates (it is d*u/m), the exact
+    derivative is recovered when eps = eps_root = 0, zeros of new_mu give exact +0 and NaN does
+    not take the zero branch."""
+    rng = np.random.default_rng(8)
+    n = 512
+    b1, b2, c = 0.9, 0.999, 4
+    m1 = (0.1 * rng.standard_normal(n)).astype(dtype)
+    v1 = np.abs(0.01 * rng.standard_normal(n)).astype(dtype) + dtype(1e-4)
+    d = rng.standard_normal(n).astype(dtype)
+    u = O.forward_updates(m1, v1, b1, b2, 0.0, 0.0, c)
+    dm, dv = O.backward_updates(d, u, m1, b1, b2, 0.0, c)
+    e = np.finfo(dtype).eps
+    np.testing.assert_allclose(dm * m1, d * u, rtol=8 * e)
+    # exact derivative of u = (m c1) / sqrt(v c2):  du/dm = u/m,  du/dv = -u / (2 v)
+    np.testing.assert_allclose(dm, d * (u / m1), rtol=8 * e)
+    np.testing.assert_allclose(dv, -d * u / (2 * v1), rtol=64 * e)
+    m0 = m1.copy()
+    m0[:4] = [0.0, -0.0, np.nan, 1.0]
+    with np.errstate(all='ignore'):
+        dm, dv = O.backward_updates(d, u, m0, b1, b2, 0.0, c)
+    for out in (dm, dv):
+        assert out[0] == 0 and not np.signbit(out[0])
+        assert out[1] == 0 and not np.signbit(out[1])
+        assert np.isnan(out[2])
+
+
+def test_fp32_backward_updates_tail_runs_in_double():
+    """Pick values where rounding the tail products in float (instead of one final rounding
+    from double) changes the result; the oracle must match the double-tail evaluation."""
+    rng = np.random.default_rng(12)
+    n = 4096
+    d = rng.standard_normal(n).astype(np.float32)
+    u = rng.standard_normal(n).astype(np.float32)
+    m1 = (0.1 * rng.standard_normal(n)).astype(np.float32) + np.float32(0.5)
+    b1, b2, er, c = 0.9, 0.999, 1e-8, 5
+    _, dv = O.backward_updates(d, u, m1, b1, b2, er, c)
+    _, _, p1, q2 = O.host_scalars(b1, b2, er, c)
+    p1, q2 = np.float32(p1), np.float32(q2)
+    r = u / m1
+    den = r * p1
+    head = ((-d) * u) * den
+    in_double = (((head.astype(np.float64) * 0.5) * np.float64(q2))
+                 * den.astype(np.float64)).astype(np.float32)
+    in_float = ((head * np.float32(0.5)) * q2) * den
+    assert_bit_equal(dv, in_double)
+    assert np.any(in_double != in_float)
+
+
+def test_thread_policy():
+    """min(n/1000, nprocs) threads, serial up to and including n = 1000
+    (/root/reference/src/adam_op/adam_op_impl_cpu.cpp:30, 43-46)."""
+    import os
+
+    assert O.threads_for(0) == 1 and O.threads_for(1000) == 1
+    assert O.threads_for(1001) == 1
+    assert O.threads_for(2000) == min(2, os.cpu_count())
+    assert O.threads_for(10 ** 9) >= 1

@@ -1,0 +1,14 @@
+"""MI355X-native fused Adam operator: a drop-in for TorchOpt's accelerated Adam op.
+
+    from torchopt_amd._C import adam_op                    # the 7-function native surface
+    from torchopt_amd.accelerated_op import AdamOp         # the per-leaf callable
+    from torchopt_amd import accelerated_op_available
+"""
+
+from torchopt_amd import accelerated_op
+from torchopt_amd.accelerated_op import AdamOp
+from torchopt_amd.accelerated_op import is_available as accelerated_op_available
+
+__version__ = '0.1.0'
+
+__all__ = ['AdamOp', 'accelerated_op', 'accelerated_op_available']

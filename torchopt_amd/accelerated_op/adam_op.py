@@ -1,0 +1,107 @@
+"""``AdamOp``: the callable the Adam transformation applies to every leaf.
+
+Counterpart of /root/reference/torchopt/accelerated_op/adam_op.py:33-181, bound to
+``torchopt_amd._C.adam_op`` (hand-written gfx950 kernels) and to nothing else: there is no
+pure-PyTorch fallback module behind it.
+
+Contract kept from the reference:
+  * ``AdamOp(b1, b2, eps, *, eps_root, inplace)(mu, nu, updates, count)`` returns
+    ``(new_mu, new_nu, new_updates)``; ``updates is None`` returns ``(mu, nu, None)``
+    untouched (:148-149);
+  * ``inplace=True`` runs the fused ``forward_`` which overwrites all three tensors (:156-166);
+  * ``inplace=False`` chains three autograd Functions -- ``MuOp``, ``NuOp``, ``UpdatesOp`` --
+    whose backward passes call ``backward_mu`` / ``backward_nu`` / ``backward_updates`` with
+    the tensors the reference saves (:36-121), so outer-loop gradients flow through the step;
+  * non-tensor arguments (decay rates, the hyper-parameter tuple) get ``None`` gradients.
+"""
+
+from __future__ import annotations
+
+from typing import Any
+
+import torch
+
+from torchopt_amd._C import adam_op
+
+
+class AdamOp:
+    """Fused Adam scaling of one leaf: moments update plus bias-corrected step direction."""
+
+    class MuOp(torch.autograd.Function):
+        """First moment: ``new_mu = b1*mu + (1-b1)*updates``."""
+
+        @staticmethod
+        def forward(ctx: Any, updates: torch.Tensor, mu: torch.Tensor, b1: float) -> torch.Tensor:
+            ctx.save_for_backward(updates, mu)
+            ctx.b1 = b1
+            return adam_op.forward_mu(updates, mu, b1)
+
+        @staticmethod
+        def backward(ctx: Any, dmu: torch.Tensor):
+            updates, mu = ctx.saved_tensors
+            dupdates, dmu_in = adam_op.backward_mu(dmu, updates, mu, ctx.b1)
+            return dupdates, dmu_in, None
+
+    class NuOp(torch.autograd.Function):
+        """Second raw moment: ``new_nu = b2*nu + (1-b2)*updates**2``."""
+
+        @staticmethod
+        def forward(ctx: Any, updates: torch.Tensor, nu: torch.Tensor, b2: float) -> torch.Tensor:
+            ctx.save_for_backward(updates, nu)
+            ctx.b2 = b2
+            return adam_op.forward_nu(updates, nu, b2)
+
+        @staticmethod
+        def backward(ctx: Any, dnu: torch.Tensor):
+            updates, nu = ctx.saved_tensors
+            dupdates, dnu_in = adam_op.backward_nu(dnu, updates, nu, ctx.b2)
+            return dupdates, dnu_in, None
+
+    class UpdatesOp(torch.autograd.Function):
+        """Step direction ``mu_hat / (sqrt(nu_hat + eps_root) + eps)``; its backward is the
+        reference's hand-derived formula, which needs the forward output."""
+
+        @staticmethod
+        def forward(ctx: Any, new_mu: torch.Tensor, new_nu: torch.Tensor, hyper: tuple):
+            b1, b2, eps, eps_root, count = hyper
+            new_updates = adam_op.forward_updates(new_mu, new_nu, b1, b2, eps, eps_root, count)
+            ctx.save_for_backward(new_updates, new_mu, new_nu)
+            ctx.hyper = hyper
+            return new_updates
+
+        @staticmethod
+        def backward(ctx: Any, dupdates: torch.Tensor):
+            new_updates, new_mu, new_nu = ctx.saved_tensors
+            b1, b2, _eps, eps_root, count = ctx.hyper
+            dnew_mu, dnew_nu = adam_op.backward_updates(
+                dupdates, new_updates, new_mu, new_nu, b1, b2, eps_root, count)
+            return dnew_mu, dnew_nu, None
+
+    def __init__(
+        self,
+        b1: float = 0.9,
+        b2: float = 0.999,
+        eps: float = 1e-8,
+        *,
+        eps_root: float = 0.0,
+        inplace: bool = True,
+    ) -> None:
+        self.b1 = b1
+        self.b2 = b2
+        self.eps = eps
+        self.eps_root = eps_root
+        self.inplace = inplace
+
+    def __call__(self, mu, nu, updates, count):
+        if updates is None:
+            return mu, nu, None
+        if self.inplace:
+            # forward_ hands back [updates, mu, nu]; callers want (mu, nu, updates)
+            new_updates, new_mu, new_nu = adam_op.forward_(
+                updates, mu, nu, self.b1, self.b2, self.eps, self.eps_root, count)
+            return new_mu, new_nu, new_updates
+        new_mu = self.MuOp.apply(updates, mu, self.b1)
+        new_nu = self.NuOp.apply(updates, nu, self.b2)
+        hyper = (self.b1, self.b2, self.eps, self.eps_root, count)
+        new_updates = self.UpdatesOp.apply(new_mu, new_nu, hyper)
+        return new_mu, new_nu, new_updates

@@ -1,0 +1,375 @@
+// Device code of the fused Adam operator for gfx950 (MI355X, CDNA4).
+//
+// Every op here is a pure streaming pass: a handful of flops per element
+// against 12-48 bytes of HBM traffic, so the kernels are shaped for memory
+// throughput and nothing else:
+//   * 128-bit accesses (4 x f32 or 2 x f64 per lane); one wave instruction
+//     covers 1 KiB of contiguous memory;
+//   * a tile is kBlock * UNROLL vectors per stream; a lane issues all of its
+//     loads for a tile (UNROLL per input stream) before the first use, so a
+//     64-wide wave keeps UNROLL * NIN KiB in flight;
+//   * a bounded grid of workgroups walks the tiles with a grid stride, so at
+//     any moment the chip touches one moving window of each stream;
+//   * streams are touched once, so loads and stores carry the non-temporal
+//     hint.
+//
+// Arithmetic follows /root/reference/src/adam_op/adam_op_impl_cpu.cpp to the
+// rounding: every product and sum is rounded on its own (build with
+// -ffp-contract=off), (1-b) is formed in the element type, bias corrections
+// are pre-rounded reciprocals that multiply, sqrt and divide are the
+// correctly rounded ones, and the tail of backward_updates runs in double.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace toa {
+
+constexpr int kBlock = 256;  // 4 waves of 64
+
+template <typename T>
+struct Vec;
+template <>
+struct Vec<float> {
+    typedef float type __attribute__((ext_vector_type(4)));
+    static constexpr int N = 4;
+};
+template <>
+struct Vec<double> {
+    typedef double type __attribute__((ext_vector_type(2)));
+    static constexpr int N = 2;
+};
+
+template <bool NT, typename V>
+__device__ __forceinline__ V ld(const V *p) {
+    if constexpr (NT) return __builtin_nontemporal_load(p);
+    return *p;
+}
+template <bool NT, typename V>
+__device__ __forceinline__ void st(V *p, V v) {
+    if constexpr (NT)
+        __builtin_nontemporal_store(v, p);
+    else
+        *p = v;
+}
+
+__device__ __forceinline__ float toa_sqrt(float x) { return sqrtf(x); }
+__device__ __forceinline__ double toa_sqrt(double x) { return sqrt(x); }
+
+// ---------------------------------------------------------------------------
+// Element-wise ops.  Pointer slots: inputs first, then outputs; an in-place op
+// writes output j back to input slot out_slot(j).
+// ---------------------------------------------------------------------------
+
+// adam_op_impl_cpu.cpp:47-61.  Slots: 0 updates, 1 mu, 2 nu.
+template <typename T>
+struct ForwardInplace {
+    static constexpr int NIN = 3, NOUT = 3, NPTR = 3;
+    // outputs are produced as (mu', nu', updates') and stored in that order
+    __device__ static constexpr int out_slot(int j) { return j == 0 ? 1 : (j == 1 ? 2 : 0); }
+    T b1, b2, c1, c2, eps, eps_root;
+    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
+        const T g = in[0], m = in[1], v = in[2];
+        const T m1 = b1 * m + (1 - b1) * g;
+        const T v1 = b2 * v + (1 - b2) * g * g;
+        const T mh = m1 * c1;
+        const T vh = v1 * c2;
+        out[0] = m1;
+        out[1] = v1;
+        out[2] = mh / (toa_sqrt(vh + eps_root) + eps);
+    }
+};
+
+// adam_op_impl_cpu.cpp:103-108.  Slots: 0 updates, 1 mu, 2 mu_out.
+template <typename T>
+struct ForwardMu {
+    static constexpr int NIN = 2, NOUT = 1, NPTR = 3;
+    __device__ static constexpr int out_slot(int j) { return NIN + j; }
+    T b1;
+    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
+        out[0] = b1 * in[1] + (1 - b1) * in[0];
+    }
+};
+
+// adam_op_impl_cpu.cpp:137-143.  Slots: 0 updates, 1 nu, 2 nu_out.
+template <typename T>
+struct ForwardNu {
+    static constexpr int NIN = 2, NOUT = 1, NPTR = 3;
+    __device__ static constexpr int out_slot(int j) { return NIN + j; }
+    T b2;
+    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
+        const T g = in[0];
+        out[0] = b2 * in[1] + (1 - b2) * g * g;
+    }
+};
+
+// adam_op_impl_cpu.cpp:175-181.  Slots: 0 new_mu, 1 new_nu, 2 updates_out.
+template <typename T>
+struct ForwardUpdates {
+    static constexpr int NIN = 2, NOUT = 1, NPTR = 3;
+    __device__ static constexpr int out_slot(int j) { return NIN + j; }
+    T c1, c2, eps, eps_root;
+    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
+        const T mh = in[0] * c1;
+        const T vh = in[1] * c2;
+        out[0] = mh / (toa_sqrt(vh + eps_root) + eps);
+    }
+};
+
+// adam_op_impl_cpu.cpp:220-226.  Slots: 0 dmu, 1 dupdates_out, 2 dmu_out.
+template <typename T>
+struct BackwardMu {
+    static constexpr int NIN = 1, NOUT = 2, NPTR = 3;
+    __device__ static constexpr int out_slot(int j) { return NIN + j; }
+    T b1;
+    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
+        out[0] = (1 - b1) * in[0];
+        out[1] = b1 * in[0];
+    }
+};
+
+// adam_op_impl_cpu.cpp:257-264.  Slots: 0 dnu, 1 updates, 2 dupdates_out, 3 dnu_out.
+template <typename T>
+struct BackwardNu {
+    static constexpr int NIN = 2, NOUT = 2, NPTR = 4;
+    __device__ static constexpr int out_slot(int j) { return NIN + j; }
+    T b2;
+    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
+        out[0] = 2 * (1 - b2) * in[1] * in[0];
+        out[1] = b2 * in[0];
+    }
+};
+
+// adam_op_impl_cpu.cpp:298-316.  Slots: 0 dupdates, 1 updates, 2 new_mu,
+// 3 dnew_mu_out, 4 dnew_nu_out.  p1 = 1 - b1^count, q2 = 1/(1 - b2^count + eps_root).
+template <typename T>
+struct BackwardUpdates {
+    static constexpr int NIN = 3, NOUT = 2, NPTR = 5;
+    __device__ static constexpr int out_slot(int j) { return NIN + j; }
+    T p1, q2;
+    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
+        const T d = in[0], u = in[1], m1 = in[2];
+        const T r = u / m1;
+        const T den = r * p1;
+        const T dm = d * r;
+        // two products in T, then the double literal 0.5 lifts the rest to double
+        const T dn = static_cast<T>(-d * u * den * 0.5 * q2 * den);
+        const bool zero = (m1 == 0);  // +0 and -0, not NaN
+        out[0] = zero ? T(0) : dm;
+        out[1] = zero ? T(0) : dn;
+    }
+};
+
+// ---------------------------------------------------------------------------
+// Tile processing.  A tile is kBlock * UNROLL vectors (TILE = that * Vec<T>::N
+// elements) of one tensor.
+// ---------------------------------------------------------------------------
+
+template <typename T, int UNROLL>
+struct Tile {
+    static constexpr int VN = Vec<T>::N;
+    static constexpr int VECS = kBlock * UNROLL;
+    static constexpr int ELEMS = VECS * VN;
+};
+
+template <typename T, class Op>
+struct TensorPtrs {
+    T *p[Op::NPTR];
+};
+
+// All pointers 16-byte aligned, whole tile inside the tensor.
+template <typename T, class Op, int UNROLL, bool NT>
+__device__ __forceinline__ void tile_full(const Op &op, const TensorPtrs<T, Op> &tp,
+                                          size_t vec_base) {
+    using V = typename Vec<T>::type;
+    constexpr int VN = Vec<T>::N;
+    V in[Op::NIN][UNROLL];
+    const size_t v0 = vec_base + threadIdx.x;
+#pragma unroll
+    for (int k = 0; k < UNROLL; ++k)
+#pragma unroll
+        for (int i = 0; i < Op::NIN; ++i)
+            in[i][k] = ld<NT>(reinterpret_cast<const V *>(tp.p[i]) + v0 + (size_t)k * kBlock);
+
+    V out[Op::NOUT][UNROLL];
+#pragma unroll
+    for (int k = 0; k < UNROLL; ++k)
+#pragma unroll
+        for (int e = 0; e < VN; ++e) {
+            T a[Op::NIN], r[Op::NOUT];
+#pragma unroll
+            for (int i = 0; i < Op::NIN; ++i) a[i] = in[i][k][e];
+            op(a, r);
+#pragma unroll
+            for (int j = 0; j < Op::NOUT; ++j) out[j][k][e] = r[j];
+        }
+
+#pragma unroll
+    for (int k = 0; k < UNROLL; ++k)
+#pragma unroll
+        for (int j = 0; j < Op::NOUT; ++j)
+            st<NT>(reinterpret_cast<V *>(tp.p[Op::out_slot(j)]) + v0 + (size_t)k * kBlock,
+                   out[j][k]);
+}
+
+// All pointers 16-byte aligned, tile cut short by the end of the tensor:
+// `rem` (< Tile::ELEMS) elements remain from element index `base`.
+template <typename T, class Op, int UNROLL>
+__device__ __forceinline__ void tile_partial(const Op &op, const TensorPtrs<T, Op> &tp,
+                                             size_t base, uint32_t rem) {
+    using V = typename Vec<T>::type;
+    constexpr int VN = Vec<T>::N;
+    const uint32_t nvec = rem / VN;
+    const size_t vbase = base / VN;  // base is a multiple of Tile::ELEMS
+    for (uint32_t v = threadIdx.x; v < nvec; v += kBlock) {
+        V in[Op::NIN], out[Op::NOUT];
+#pragma unroll
+        for (int i = 0; i < Op::NIN; ++i) in[i] = reinterpret_cast<const V *>(tp.p[i])[vbase + v];
+#pragma unroll
+        for (int e = 0; e < VN; ++e) {
+            T a[Op::NIN], r[Op::NOUT];
+#pragma unroll
+            for (int i = 0; i < Op::NIN; ++i) a[i] = in[i][e];
+            op(a, r);
+#pragma unroll
+            for (int j = 0; j < Op::NOUT; ++j) out[j][e] = r[j];
+        }
+#pragma unroll
+        for (int j = 0; j < Op::NOUT; ++j)
+            reinterpret_cast<V *>(tp.p[Op::out_slot(j)])[vbase + v] = out[j];
+    }
+    // the last rem % VN elements, one lane each
+    const uint32_t done = nvec * VN;
+    if (threadIdx.x < rem - done) {
+        const size_t i0 = base + done + threadIdx.x;
+        T a[Op::NIN], r[Op::NOUT];
+#pragma unroll
+        for (int i = 0; i < Op::NIN; ++i) a[i] = tp.p[i][i0];
+        op(a, r);
+#pragma unroll
+        for (int j = 0; j < Op::NOUT; ++j) tp.p[Op::out_slot(j)][i0] = r[j];
+    }
+}
+
+// Some pointer is not 16-byte aligned: element-wise accesses, still coalesced
+// (consecutive lanes touch consecutive elements).
+template <typename T, class Op, int UNROLL>
+__device__ __forceinline__ void tile_unaligned(const Op &op, const TensorPtrs<T, Op> &tp,
+                                               size_t base, uint32_t cnt) {
+    constexpr int STEPS = 4;
+    for (uint32_t e0 = 0; e0 < cnt; e0 += kBlock * STEPS) {
+        T a[STEPS][Op::NIN];
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+            const uint32_t e = e0 + s * kBlock + threadIdx.x;
+            if (e < cnt) {
+#pragma unroll
+                for (int i = 0; i < Op::NIN; ++i) a[s][i] = tp.p[i][base + e];
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+            const uint32_t e = e0 + s * kBlock + threadIdx.x;
+            if (e < cnt) {
+                T r[Op::NOUT];
+                op(a[s], r);
+#pragma unroll
+                for (int j = 0; j < Op::NOUT; ++j) tp.p[Op::out_slot(j)][base + e] = r[j];
+            }
+        }
+    }
+}
+
+template <typename T, class Op>
+__device__ __forceinline__ bool all_aligned16(const TensorPtrs<T, Op> &tp) {
+    uintptr_t bits = 0;
+#pragma unroll
+    for (int i = 0; i < Op::NPTR; ++i) bits |= reinterpret_cast<uintptr_t>(tp.p[i]);
+    return (bits & 15u) == 0;
+}
+
+template <typename T, class Op, int UNROLL, bool NT>
+__device__ __forceinline__ void process_tile(const Op &op, const TensorPtrs<T, Op> &tp, size_t n,
+                                             size_t tile, bool aligned) {
+    using TL = Tile<T, UNROLL>;
+    const size_t base = tile * TL::ELEMS;
+    const size_t left = n - base;
+    if (aligned) {
+        if (left >= (size_t)TL::ELEMS)
+            tile_full<T, Op, UNROLL, NT>(op, tp, tile * TL::VECS);
+        else
+            tile_partial<T, Op, UNROLL>(op, tp, base, (uint32_t)left);
+    } else {
+        const uint32_t cnt = left >= (size_t)TL::ELEMS ? (uint32_t)TL::ELEMS : (uint32_t)left;
+        tile_unaligned<T, Op, UNROLL>(op, tp, base, cnt);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Single-tensor kernel: workgroups stride over the tensor's tiles.
+// ---------------------------------------------------------------------------
+template <typename T, class Op, int UNROLL, bool NT>
+__global__ __launch_bounds__(kBlock) void stream_kernel(const Op op, const TensorPtrs<T, Op> tp,
+                                                        const size_t n, const size_t num_tiles) {
+    const bool aligned = all_aligned16<T, Op>(tp);
+    for (size_t tile = blockIdx.x; tile < num_tiles; tile += gridDim.x)
+        process_tile<T, Op, UNROLL, NT>(op, tp, n, tile, aligned);
+}
+
+// ---------------------------------------------------------------------------
+// Multi-tensor kernel.  The per-tensor table travels in the kernel-argument
+// segment (no device allocation, no upload, capturable in a HIP graph):
+// pointer slots, element counts and an exclusive prefix sum of tile counts.
+// A workgroup maps a global tile id to (tensor, local tile) with a binary
+// search over the prefix sums; every value involved is wave-uniform, so the
+// search runs on the scalar unit against the scalar cache.
+// ---------------------------------------------------------------------------
+// Bytes of kernel-argument space given to the table.  With the op's scalars
+// (at most 48 bytes) and the 256 bytes of implicit arguments the whole segment
+// stays under the 4 KiB HIP allows.
+constexpr int kKernargBudget = 3712;
+
+template <class Op>
+struct MultiCap {
+    // per tensor: NPTR pointers, one 64-bit length, one 32-bit tile prefix
+    static constexpr int kPerTensor = 8 * Op::NPTR + 8 + 4;
+    static constexpr int MAX = (kKernargBudget - 8) / kPerTensor;
+};
+
+template <typename T, class Op>
+struct MultiTable {
+    static constexpr int MAX = MultiCap<Op>::MAX;
+    T *p[Op::NPTR][MAX];
+    uint64_t n[MAX];
+    uint32_t tile_start[MAX + 1];  // tile_start[num] == total tiles
+    uint32_t num;
+};
+
+template <typename T, class Op, int UNROLL, bool NT>
+__global__ __launch_bounds__(kBlock) void multi_stream_kernel(const Op op,
+                                                              const MultiTable<T, Op> tab) {
+    const uint32_t total = tab.tile_start[tab.num];
+    uint32_t t = 0;
+    for (uint32_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+        if (tile >= tab.tile_start[t + 1]) {
+            // largest t with tile_start[t] <= tile
+            uint32_t lo = t + 1, hi = tab.num - 1;
+            while (lo < hi) {
+                const uint32_t mid = (lo + hi + 1) >> 1;
+                if (tab.tile_start[mid] <= tile)
+                    lo = mid;
+                else
+                    hi = mid - 1;
+            }
+            t = lo;
+        }
+        TensorPtrs<T, Op> tp;
+#pragma unroll
+        for (int i = 0; i < Op::NPTR; ++i) tp.p[i] = tab.p[i][t];
+        const bool aligned = all_aligned16<T, Op>(tp);
+        process_tile<T, Op, UNROLL, NT>(op, tp, (size_t)tab.n[t], (size_t)(tile - tab.tile_start[t]),
+                                        aligned);
+    }
+}
+
+}  // namespace toa

@@ -1,0 +1,340 @@
+// Host side of libtoa_adam.so: the C ABI declared in include/toa_adam.h.
+//
+// Each entry point rounds the Python-level scalars the way the reference
+// launchers do (/root/reference/src/adam_op/adam_op_impl_cpu.cpp:73-84,
+// 191-206, 328-343: powers, differences and reciprocals in double, then one
+// cast to the element type), picks a grid and enqueues one kernel on the
+// caller's stream.  Nothing here allocates, copies or synchronises.
+#include "toa_adam.h"
+
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cmath>
+#include <vector>
+
+#include "adam_kernels.hpp"
+
+namespace {
+
+using namespace toa;
+
+// Launch shape of the streaming kernels (see adam_kernels.hpp).
+constexpr int kUnroll = 4;          // 16-byte loads in flight per lane per input stream
+constexpr bool kNonTemporal = true; // streams are touched once
+constexpr int kBlocksPerCU = 8;     // resident workgroups the grid is capped at, per CU
+
+constexpr int kMaxDevices = 64;
+std::atomic<int> g_cu_count[kMaxDevices];
+
+int cu_count() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+    int n = g_cu_count[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+            n <= 0)
+            n = 256;
+        g_cu_count[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
+unsigned grid_for(size_t num_tiles) {
+    const size_t cap = (size_t)cu_count() * kBlocksPerCU;
+    return (unsigned)(num_tiles < cap ? num_tiles : cap);
+}
+
+struct HostScalars {
+    double c1, c2, p1, q2;
+};
+
+// adam_op_impl_cpu.cpp:73-74 (c1, c2), :328-329 (p1, q2); std::pow(double, size_t)
+// promotes the exponent to double.
+HostScalars host_scalars(double b1, double b2, double eps_root, uint64_t count) {
+    const double pb1 = std::pow(b1, (double)count);
+    const double pb2 = std::pow(b2, (double)count);
+    return {1 / (1 - pb1), 1 / (1 - pb2), 1 - pb1, 1 / (1 - pb2 + eps_root)};
+}
+
+template <typename T, class Op>
+int launch_single(const Op &op, T *const (&ptrs)[Op::NPTR], size_t n, void *stream) {
+    if (n == 0) return 0;
+    TensorPtrs<T, Op> tp;
+    for (int i = 0; i < Op::NPTR; ++i) {
+        if (ptrs[i] == nullptr) return TOA_ENULL;
+        tp.p[i] = ptrs[i];
+    }
+    constexpr size_t tile = Tile<T, kUnroll>::ELEMS;
+    const size_t num_tiles = (n + tile - 1) / tile;
+    hipLaunchKernelGGL((stream_kernel<T, Op, kUnroll, kNonTemporal>), dim3(grid_for(num_tiles)),
+                       dim3(kBlock), 0, (hipStream_t)stream, op, tp, n, num_tiles);
+    return (int)hipGetLastError();
+}
+
+// Launch one op over a list of tensors.  `make_op(count)` builds the op's
+// scalars for one step number; tensors are batched per distinct count and per
+// kernel-argument table capacity.
+template <typename T, class Op, class MakeOp>
+int launch_multi(MakeOp make_op, size_t num, const void *const *const (&lists)[Op::NPTR],
+                 const size_t *n, const uint64_t *counts, uint64_t count_all, void *stream) {
+    using Table = MultiTable<T, Op>;
+    constexpr size_t tile = Tile<T, kUnroll>::ELEMS;
+    if (num == 0) return 0;
+    if (n == nullptr) return TOA_ENULL;
+    for (int i = 0; i < Op::NPTR; ++i)
+        if (lists[i] == nullptr) return TOA_ENULL;
+
+    // validate everything before the first launch
+    for (size_t k = 0; k < num; ++k) {
+        if (n[k] == 0) continue;
+        for (int i = 0; i < Op::NPTR; ++i)
+            if (lists[i][k] == nullptr) return TOA_ENULL;
+        if ((n[k] + tile - 1) / tile > 0x7fffffffu) return TOA_ESIZE;
+    }
+
+    std::vector<uint64_t> distinct;
+    if (counts == nullptr) {
+        distinct.push_back(count_all);
+    } else {
+        for (size_t k = 0; k < num; ++k) {
+            if (n[k] == 0) continue;
+            bool seen = false;
+            for (uint64_t c : distinct) seen |= (c == counts[k]);
+            if (!seen) distinct.push_back(counts[k]);
+        }
+    }
+
+    Table tab;
+    for (uint64_t c : distinct) {
+        const Op op = make_op(c);
+        tab.num = 0;
+        tab.tile_start[0] = 0;
+        auto flush = [&]() -> int {
+            if (tab.num == 0) return 0;
+            const uint32_t total = tab.tile_start[tab.num];
+            hipLaunchKernelGGL((multi_stream_kernel<T, Op, kUnroll, kNonTemporal>),
+                               dim3(grid_for(total)), dim3(kBlock), 0, (hipStream_t)stream, op,
+                               tab);
+            tab.num = 0;
+            return (int)hipGetLastError();
+        };
+        for (size_t k = 0; k < num; ++k) {
+            if (n[k] == 0 || (counts != nullptr && counts[k] != c)) continue;
+            const uint64_t tiles = (n[k] + tile - 1) / tile;
+            if (tab.num == (uint32_t)Table::MAX ||
+                (uint64_t)tab.tile_start[tab.num] + tiles > 0xffffffffu) {
+                if (int rc = flush()) return rc;
+            }
+            const uint32_t t = tab.num;
+            for (int i = 0; i < Op::NPTR; ++i)
+                tab.p[i][t] = static_cast<T *>(const_cast<void *>(lists[i][k]));
+            tab.n[t] = n[k];
+            tab.tile_start[t + 1] = tab.tile_start[t] + (uint32_t)tiles;
+            tab.num = t + 1;
+        }
+        if (int rc = flush()) return rc;
+    }
+    return 0;
+}
+
+template <typename T>
+T *mut(const void *p) {
+    return static_cast<T *>(const_cast<void *>(p));
+}
+
+#define TOA_DISPATCH(dtype, ...)                  \
+    switch (dtype) {                              \
+        case TOA_F32: {                           \
+            using T = float;                      \
+            return __VA_ARGS__();                 \
+        }                                         \
+        case TOA_F64: {                           \
+            using T = double;                     \
+            return __VA_ARGS__();                 \
+        }                                         \
+        default:                                  \
+            return TOA_EDTYPE;                    \
+    }
+
+}  // namespace
+
+extern "C" {
+
+int toa_adam_abi_version(void) { return 1; }
+
+const char *toa_adam_error_string(int code) {
+    switch (code) {
+        case 0: return "success";
+        case TOA_EDTYPE: return "toa_adam: unsupported dtype (expected TOA_F32 or TOA_F64)";
+        case TOA_ENULL: return "toa_adam: null pointer for a non-empty tensor";
+        case TOA_ESIZE: return "toa_adam: tensor too large for one launch";
+        default: return code > 0 ? hipGetErrorString((hipError_t)code) : "toa_adam: unknown error";
+    }
+}
+
+int toa_adam_forward_inplace(int dtype, void *updates, void *mu, void *nu, size_t n, double b1,
+                             double b2, double eps, double eps_root, uint64_t count,
+                             void *stream) {
+    const HostScalars s = host_scalars(b1, b2, eps_root, count);
+    TOA_DISPATCH(dtype, [&] {
+        const ForwardInplace<T> op{(T)b1, (T)b2, (T)s.c1, (T)s.c2, (T)eps, (T)eps_root};
+        T *const p[3] = {(T *)updates, (T *)mu, (T *)nu};
+        return launch_single<T>(op, p, n, stream);
+    });
+}
+
+int toa_adam_forward_mu(int dtype, const void *updates, const void *mu, size_t n, double b1,
+                        void *mu_out, void *stream) {
+    TOA_DISPATCH(dtype, [&] {
+        const ForwardMu<T> op{(T)b1};
+        T *const p[3] = {mut<T>(updates), mut<T>(mu), (T *)mu_out};
+        return launch_single<T>(op, p, n, stream);
+    });
+}
+
+int toa_adam_forward_nu(int dtype, const void *updates, const void *nu, size_t n, double b2,
+                        void *nu_out, void *stream) {
+    TOA_DISPATCH(dtype, [&] {
+        const ForwardNu<T> op{(T)b2};
+        T *const p[3] = {mut<T>(updates), mut<T>(nu), (T *)nu_out};
+        return launch_single<T>(op, p, n, stream);
+    });
+}
+
+int toa_adam_forward_updates(int dtype, const void *new_mu, const void *new_nu, size_t n,
+                             double b1, double b2, double eps, double eps_root, uint64_t count,
+                             void *updates_out, void *stream) {
+    const HostScalars s = host_scalars(b1, b2, eps_root, count);
+    TOA_DISPATCH(dtype, [&] {
+        const ForwardUpdates<T> op{(T)s.c1, (T)s.c2, (T)eps, (T)eps_root};
+        T *const p[3] = {mut<T>(new_mu), mut<T>(new_nu), (T *)updates_out};
+        return launch_single<T>(op, p, n, stream);
+    });
+}
+
+int toa_adam_backward_mu(int dtype, const void *dmu, size_t n, double b1, void *dupdates_out,
+                         void *dmu_out, void *stream) {
+    TOA_DISPATCH(dtype, [&] {
+        const BackwardMu<T> op{(T)b1};
+        T *const p[3] = {mut<T>(dmu), (T *)dupdates_out, (T *)dmu_out};
+        return launch_single<T>(op, p, n, stream);
+    });
+}
+
+int toa_adam_backward_nu(int dtype, const void *dnu, const void *updates, size_t n, double b2,
+                         void *dupdates_out, void *dnu_out, void *stream) {
+    TOA_DISPATCH(dtype, [&] {
+        const BackwardNu<T> op{(T)b2};
+        T *const p[4] = {mut<T>(dnu), mut<T>(updates), (T *)dupdates_out, (T *)dnu_out};
+        return launch_single<T>(op, p, n, stream);
+    });
+}
+
+int toa_adam_backward_updates(int dtype, const void *dupdates, const void *updates,
+                              const void *new_mu, size_t n, double b1, double b2,
+                              double eps_root, uint64_t count, void *dnew_mu_out,
+                              void *dnew_nu_out, void *stream) {
+    const HostScalars s = host_scalars(b1, b2, eps_root, count);
+    TOA_DISPATCH(dtype, [&] {
+        const BackwardUpdates<T> op{(T)s.p1, (T)s.q2};
+        T *const p[5] = {mut<T>(dupdates), mut<T>(updates), mut<T>(new_mu), (T *)dnew_mu_out,
+                         (T *)dnew_nu_out};
+        return launch_single<T>(op, p, n, stream);
+    });
+}
+
+// ---- multi-tensor -----------------------------------------------------------
+
+#define CPP(x) reinterpret_cast<const void *const *>(x)
+
+int toa_adam_forward_inplace_multi(int dtype, size_t num_tensors, void *const *updates,
+                                   void *const *mu, void *const *nu, const size_t *n, double b1,
+                                   double b2, double eps, double eps_root,
+                                   const uint64_t *counts, uint64_t count_all, void *stream) {
+    TOA_DISPATCH(dtype, [&] {
+        const void *const *const lists[3] = {CPP(updates), CPP(mu), CPP(nu)};
+        auto make = [&](uint64_t c) {
+            const HostScalars s = host_scalars(b1, b2, eps_root, c);
+            return ForwardInplace<T>{(T)b1, (T)b2, (T)s.c1, (T)s.c2, (T)eps, (T)eps_root};
+        };
+        return launch_multi<T, ForwardInplace<T>>(make, num_tensors, lists, n, counts, count_all,
+                                                  stream);
+    });
+}
+
+int toa_adam_forward_mu_multi(int dtype, size_t num_tensors, const void *const *updates,
+                              const void *const *mu, const size_t *n, double b1,
+                              void *const *mu_out, void *stream) {
+    TOA_DISPATCH(dtype, [&] {
+        const void *const *const lists[3] = {updates, mu, CPP(mu_out)};
+        auto make = [&](uint64_t) { return ForwardMu<T>{(T)b1}; };
+        return launch_multi<T, ForwardMu<T>>(make, num_tensors, lists, n, nullptr, 0, stream);
+    });
+}
+
+int toa_adam_forward_nu_multi(int dtype, size_t num_tensors, const void *const *updates,
+                              const void *const *nu, const size_t *n, double b2,
+                              void *const *nu_out, void *stream) {
+    TOA_DISPATCH(dtype, [&] {
+        const void *const *const lists[3] = {updates, nu, CPP(nu_out)};
+        auto make = [&](uint64_t) { return ForwardNu<T>{(T)b2}; };
+        return launch_multi<T, ForwardNu<T>>(make, num_tensors, lists, n, nullptr, 0, stream);
+    });
+}
+
+int toa_adam_forward_updates_multi(int dtype, size_t num_tensors, const void *const *new_mu,
+                                   const void *const *new_nu, const size_t *n, double b1,
+                                   double b2, double eps, double eps_root,
+                                   const uint64_t *counts, uint64_t count_all,
+                                   void *const *updates_out, void *stream) {
+    TOA_DISPATCH(dtype, [&] {
+        const void *const *const lists[3] = {new_mu, new_nu, CPP(updates_out)};
+        auto make = [&](uint64_t c) {
+            const HostScalars s = host_scalars(b1, b2, eps_root, c);
+            return ForwardUpdates<T>{(T)s.c1, (T)s.c2, (T)eps, (T)eps_root};
+        };
+        return launch_multi<T, ForwardUpdates<T>>(make, num_tensors, lists, n, counts, count_all,
+                                                  stream);
+    });
+}
+
+int toa_adam_backward_mu_multi(int dtype, size_t num_tensors, const void *const *dmu,
+                               const size_t *n, double b1, void *const *dupdates_out,
+                               void *const *dmu_out, void *stream) {
+    TOA_DISPATCH(dtype, [&] {
+        const void *const *const lists[3] = {dmu, CPP(dupdates_out), CPP(dmu_out)};
+        auto make = [&](uint64_t) { return BackwardMu<T>{(T)b1}; };
+        return launch_multi<T, BackwardMu<T>>(make, num_tensors, lists, n, nullptr, 0, stream);
+    });
+}
+
+int toa_adam_backward_nu_multi(int dtype, size_t num_tensors, const void *const *dnu,
+                               const void *const *updates, const size_t *n, double b2,
+                               void *const *dupdates_out, void *const *dnu_out, void *stream) {
+    TOA_DISPATCH(dtype, [&] {
+        const void *const *const lists[4] = {dnu, updates, CPP(dupdates_out), CPP(dnu_out)};
+        auto make = [&](uint64_t) { return BackwardNu<T>{(T)b2}; };
+        return launch_multi<T, BackwardNu<T>>(make, num_tensors, lists, n, nullptr, 0, stream);
+    });
+}
+
+int toa_adam_backward_updates_multi(int dtype, size_t num_tensors, const void *const *dupdates,
+                                    const void *const *updates, const void *const *new_mu,
+                                    const size_t *n, double b1, double b2, double eps_root,
+                                    const uint64_t *counts, uint64_t count_all,
+                                    void *const *dnew_mu_out, void *const *dnew_nu_out,
+                                    void *stream) {
+    TOA_DISPATCH(dtype, [&] {
+        const void *const *const lists[5] = {dupdates, updates, new_mu, CPP(dnew_mu_out),
+                                             CPP(dnew_nu_out)};
+        auto make = [&](uint64_t c) {
+            const HostScalars s = host_scalars(b1, b2, eps_root, c);
+            return BackwardUpdates<T>{(T)s.p1, (T)s.q2};
+        };
+        return launch_multi<T, BackwardUpdates<T>>(make, num_tensors, lists, n, counts,
+                                                   count_all, stream);
+    });
+}
+
+}  // extern "C"
