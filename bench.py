@@ -1,0 +1,295 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused Adam operator on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config {0,2,3,4}]
+
+A "step" is one pass of the hot path over one batch of synthetic state that is already
+resident in HBM: for the default workload (config 2) one fused in-place `forward_` over three
+float32 arrays of 268 435 456 elements (1 GiB each), launched through the C ABI of
+libtoa_adam.so on PyTorch's current stream.  W untimed steps, then exactly K timed steps
+bracketed by `torch.cuda.synchronize()`; one JSON line on stdout.
+
+Beside the headline `value` (elements per second) the line carries
+  roofline      achieved HBM bandwidth of the kernel: algorithmic bytes per launch (24 B per
+                float32 element for forward_) over the average launch duration, measured with
+                events on the launch stream across the timed region, against 8 TB/s;
+  cpu_baseline  the reference's CPU op (or this repo's bit-identical C port of it) timed on the
+                host's cores on a bounded sample of the same workload.
+
+Everything on one GPU: `--gpus N` with N > 1 is refused.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+REPO = os.path.dirname(os.path.abspath(__file__))
+if REPO not in sys.path:
+    sys.path.insert(0, REPO)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published peak HBM3E bandwidth
+
+# Algorithmic bytes per element: every operand array is read or written exactly once.
+BYTES_PER_ELEM = {  # op -> number of arrays streamed (multiply by the element size)
+    'forward_': 6, 'forward_mu': 3, 'forward_nu': 3, 'forward_updates': 3,
+    'backward_mu': 3, 'backward_nu': 4, 'backward_updates': 5,
+}
+
+# HBM bytes per launch of the config-2 kernel as counted by rocprofv3 --pmc (FETCH_SIZE and
+# WRITE_SIZE, each scaled by what the same counter reads for a plain copy of known size);
+# see profiles/.  None until measured for the current kernel.
+MEASURED_TRAFFIC_BYTES = {2: None}
+
+B1, B2, EPS = 0.9, 0.999, 1e-8
+
+
+# ----------------------------------------------------------------------------- workloads
+
+
+def maml_shapes():
+    """Config 1: MAML-style conv net, 10 tensors, 32 645 elements."""
+    return ([(32, 3, 3, 3)] + [(32, 32, 3, 3)] * 3 + [(32,)] * 4 + [(5, 800), (5,)])
+
+
+def gpt2_medium_shapes():
+    """Config 4: GPT-2-medium parameter list (24 layers, d=1024), embeddings last."""
+    shapes = []
+    for _ in range(24):
+        shapes += [(3072, 1024), (3072,), (1024, 1024), (1024,), (4096, 1024), (4096,),
+                   (1024, 4096), (1024,), (1024,), (1024,), (1024,), (1024,)]
+    shapes += [(50257, 1024), (1024, 1024)]
+    return shapes
+
+
+def numel(shape):
+    n = 1
+    for s in shape:
+        n *= s
+    return n
+
+
+CONFIGS = {
+    0: dict(name='config0: fused forward_ in place, 1 048 576 float32 elements, count=10',
+            dtype='f32', n=1 << 20, eps_root=0.0, count=10),
+    2: dict(name='config2: fused forward_ in place, 268 435 456 float32 elements '
+                 '(1 GiB per state array), count=1000',
+            dtype='f32', n=1 << 28, eps_root=0.0, count=1000),
+    3: dict(name='config3: fused forward_ in place, 67 108 864 float64 elements, count=3',
+            dtype='f64', n=1 << 26, eps_root=1e-8, count=3),
+    4: dict(name='config4: multi-tensor forward_ in place over the GPT-2-medium parameter list '
+                 '(float32), count=1',
+            dtype='f32', shapes=gpt2_medium_shapes(), eps_root=0.0, count=1),
+}
+
+
+# ----------------------------------------------------------------------------- GPU side
+
+
+def make_state(torch, n, dtype, seed):
+    """updates ~ N(0,1), mu ~ 0.1 N(0,1), nu ~ |0.01 N(0,1)|, generated on the GPU."""
+    g = torch.Generator(device='cuda')
+    g.manual_seed(seed)
+    u = torch.randn(n, device='cuda', dtype=dtype, generator=g)
+    mu = torch.randn(n, device='cuda', dtype=dtype, generator=g).mul_(0.1)
+    nu = torch.randn(n, device='cuda', dtype=dtype, generator=g).mul_(0.01).abs_()
+    return u, mu, nu
+
+
+def run_gpu(cfg_id, steps, warmup):
+    import torch
+
+    from torchopt_amd import _lib
+
+    if not torch.cuda.is_available():
+        raise SystemExit('bench.py needs a GPU: the fused Adam op has no CPU path')
+    lib = _lib.load()
+    cfg = CONFIGS[cfg_id]
+    dtype = torch.float32 if cfg['dtype'] == 'f32' else torch.float64
+    code = _lib.TOA_F32 if cfg['dtype'] == 'f32' else _lib.TOA_F64
+    esize = 4 if cfg['dtype'] == 'f32' else 8
+    stream = torch.cuda.current_stream()
+    sptr = stream.cuda_stream
+    eps_root, count = cfg['eps_root'], cfg['count']
+
+    if 'shapes' in cfg:
+        import ctypes
+
+        sizes = [numel(s) for s in cfg['shapes']]
+        total = sum(sizes)
+        tensors = [make_state(torch, n, dtype, 1000 * cfg_id + k) for k, n in enumerate(sizes)]
+        num = len(sizes)
+        pu = (ctypes.c_void_p * num)(*[t[0].data_ptr() for t in tensors])
+        pm = (ctypes.c_void_p * num)(*[t[1].data_ptr() for t in tensors])
+        pv = (ctypes.c_void_p * num)(*[t[2].data_ptr() for t in tensors])
+        ns = (ctypes.c_size_t * num)(*sizes)
+
+        def step():
+            rc = lib.toa_adam_forward_inplace_multi(code, num, pu, pm, pv, ns, B1, B2, EPS,
+                                                    eps_root, None, count, sptr)
+            if rc:
+                raise RuntimeError(lib.toa_adam_error_string(rc).decode())
+        extra = {'tensors': num}
+    else:
+        total = cfg['n']
+        u, mu, nu = make_state(torch, total, dtype, 1000 * cfg_id)
+        pu, pm, pv = u.data_ptr(), mu.data_ptr(), nu.data_ptr()
+
+        def step():
+            rc = lib.toa_adam_forward_inplace(code, pu, pm, pv, total, B1, B2, EPS, eps_root,
+                                              count, sptr)
+            if rc:
+                raise RuntimeError(lib.toa_adam_error_string(rc).decode())
+        extra = {}
+
+    for _ in range(warmup):
+        step()
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev0.record(stream)
+    for _ in range(steps):
+        step()
+    ev1.record(stream)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+
+    wall_ms = (t1 - t0) * 1e3 / steps
+    kern_ms = ev0.elapsed_time(ev1) / steps  # stream time per launch (launches are back to back)
+    alg_bytes = BYTES_PER_ELEM['forward_'] * esize * total
+    achieved = alg_bytes / (kern_ms * 1e-3) / 1e9
+    traffic = MEASURED_TRAFFIC_BYTES.get(cfg_id)
+    return {
+        'elements': total,
+        'ms_per_step': wall_ms,
+        'value': total / (wall_ms * 1e-3),
+        'roofline': {
+            'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
+            'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': traffic,
+            'kernel_ms': round(kern_ms, 5), 'algorithmic_bytes_per_launch': alg_bytes,
+            'bytes_per_element': BYTES_PER_ELEM['forward_'] * esize,
+        },
+        'extra': extra,
+        'device': torch.cuda.get_device_name(0),
+    }
+
+
+# ----------------------------------------------------------------------------- CPU baseline
+
+
+def run_cpu_baseline(cfg_id, budget_s=12.0):
+    """Time the reference CPU op (oracle/_ref, where built) or the C port on a bounded sample.
+
+    Only this leg touches `oracle/`; it is the reported baseline, never the measured product.
+    """
+    import numpy as np
+
+    from oracle import adam_oracle
+
+    cfg = CONFIGS[cfg_id]
+    np_dtype = np.float32 if cfg['dtype'] == 'f32' else np.float64
+    full = cfg['n'] if 'n' in cfg else sum(numel(s) for s in cfg['shapes'])
+    n = min(full, 1 << 26)
+
+    # the box's CPU share, not every core the machine shows
+    share = int(os.environ.get('OMP_NUM_THREADS', '16') or 16)
+    try:
+        avail = sorted(os.sched_getaffinity(0))
+        cores = max(1, min(share, len(avail)))
+        os.sched_setaffinity(0, set(avail[:cores]))
+    except (AttributeError, OSError):
+        cores = max(1, min(share, os.cpu_count() or 1))
+
+    rng = np.random.default_rng(1000 * cfg_id)
+    block = 1 << 20
+    reps = (n + block - 1) // block
+    u = np.tile(rng.standard_normal(block).astype(np_dtype), reps)[:n].copy()
+    mu = np.tile((0.1 * rng.standard_normal(block)).astype(np_dtype), reps)[:n].copy()
+    nu = np.tile(np.abs(0.01 * rng.standard_normal(block)).astype(np_dtype), reps)[:n].copy()
+
+    ref = None
+    try:
+        ref = adam_oracle.load_reference()
+    except Exception as exc:  # noqa: BLE001
+        print(f'[bench] compiled reference not usable ({exc}); timing the C port',
+              file=sys.stderr)
+    if ref is not None:
+        import torch
+
+        tu, tm, tv = torch.from_numpy(u), torch.from_numpy(mu), torch.from_numpy(nu)
+
+        def one():
+            ref.adam_op.forward_(tu, tm, tv, B1, B2, EPS, cfg['eps_root'], cfg['count'])
+        kind = 'reference'
+    else:
+        def one():
+            adam_oracle.forward_inplace(u, mu, nu, B1, B2, EPS, cfg['eps_root'], cfg['count'])
+        kind = 'port'
+
+    one()  # warm-up (threads, page faults)
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 25):
+        t0 = time.perf_counter()
+        one()
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    esize = np.dtype(np_dtype).itemsize
+    return {
+        'value': n / med, 'unit': 'elements/s', 'cores': cores, 'kind': kind,
+        'sample': f'{n} of {full} elements ({cfg["dtype"]}), forward_ in place, '
+                  f'median of {len(times)} passes after 1 warm-up',
+        'gb_per_s': round(BYTES_PER_ELEM['forward_'] * esize * n / med / 1e9, 2),
+    }
+
+
+# ----------------------------------------------------------------------------- main
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__.split('\n')[0])
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=50)
+    ap.add_argument('--warmup', type=int, default=10)
+    ap.add_argument('--config', type=int, default=2, choices=sorted(CONFIGS))
+    ap.add_argument('--no-cpu-baseline', action='store_true')
+    args = ap.parse_args(argv)
+
+    if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
+        print('bench.py: this build measures one GPU only (the op needs no exchange between '
+              'GPUs; each would run the same kernel on its shard). Run with --gpus 1.',
+              file=sys.stderr)
+        return 2
+
+    gpu = run_gpu(args.config, args.steps, args.warmup)
+    cfg = CONFIGS[args.config]
+    line = {
+        'metric': 'adam_forward_inplace_elements_per_s',
+        'value': gpu['value'],
+        'unit': 'elements/s',
+        'n_gpus': 1,
+        'steps': args.steps,
+        'warmup': args.warmup,
+        'ms_per_step': gpu['ms_per_step'],
+        'higher_is_better': True,
+        'scaling': 'weak',
+        'vs_baseline': None,
+        'dtype': cfg['dtype'],
+        'data': 'synthetic',
+        'config': {'workload': cfg['name'], 'elements': gpu['elements'], 'b1': B1, 'b2': B2,
+                   'eps': EPS, 'eps_root': cfg['eps_root'], 'count': cfg['count'],
+                   'device': gpu['device'], **gpu['extra']},
+        'roofline': gpu['roofline'],
+    }
+    if not args.no_cpu_baseline:
+        line['cpu_baseline'] = run_cpu_baseline(args.config)
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == '__main__':
+    sys.exit(main())

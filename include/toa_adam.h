@@ -27,8 +27,7 @@
  *   return    0 on success; a positive value is a hipError_t from the launch;
  *             a negative value is one of the TOA_E* argument errors below.
  *             toa_adam_error_string() names either kind.
- *   threads   re-entrant; no global state except a per-device cache of the
- *             compute-unit count.
+ *   threads   re-entrant; the only global state is the residency knob below.
  */
 #ifndef TOA_ADAM_H
 #define TOA_ADAM_H
@@ -52,6 +51,15 @@ enum {
 
 /* Library ABI version (bumped on any signature change). */
 TOA_API int toa_adam_abi_version(void);
+
+/* Tuning knob: how many single-wave workgroups of these kernels may be resident
+ * on one compute unit.  The kernels are HBM-bound and run fastest with a bounded
+ * number of bytes in flight; each op has its own measured default (13 for the
+ * in-place step, 24-32 for the out-of-place ops).  1..32 overrides the default
+ * of every op, anything else restores the per-op defaults.  The environment
+ * variable TOA_ADAM_WAVES_PER_CU sets the initial override.  Returns the
+ * previous override (0 = none).  No counterpart in the reference. */
+TOA_API int toa_adam_set_waves_per_cu(int waves);
 
 /* Human-readable name of a return code from any function below. */
 TOA_API const char *toa_adam_error_string(int code);

@@ -1,0 +1,173 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports every symbol the
+public header declares, the ctypes table agrees with the header, argument errors come back as
+codes before any device work, and the Python surface refuses what it cannot serve instead of
+computing it somewhere else."""
+
+from __future__ import annotations
+
+import ctypes
+import inspect
+import os
+import re
+
+import pytest
+import torch
+
+from conftest import REPO
+from torchopt_amd import AdamOp, _lib, accelerated_op_available
+from torchopt_amd._C import adam_op
+
+HEADER = os.path.join(REPO, 'include', 'toa_adam.h')
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+    decls = re.findall(r'TOA_API\s+(?:const\s+char\s*\*|int)\s*(\w+)\s*\(([^;]*?)\)\s*;', text,
+                       flags=re.S)
+    return {name: [a.strip() for a in args.split(',')] if args.strip() != 'void' else []
+            for name, args in decls}
+
+
+def test_header_declares_the_expected_surface():
+    names = set(declared_functions())
+    singles = {'forward_inplace', 'forward_mu', 'forward_nu', 'forward_updates', 'backward_mu',
+               'backward_nu', 'backward_updates'}
+    want = {f'toa_adam_{s}' for s in singles} | {f'toa_adam_{s}_multi' for s in singles}
+    want |= {'toa_adam_abi_version', 'toa_adam_error_string', 'toa_adam_set_waves_per_cu'}
+    assert names == want
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared_functions():
+        assert hasattr(lib, name), f'{name} declared in include/toa_adam.h but not exported'
+
+
+def test_ctypes_table_matches_header_arity():
+    decl = declared_functions()
+    for name, argtypes in _lib.SIGNATURES.items():
+        assert name in decl
+        assert len(argtypes) == len(decl[name]), (name, len(argtypes), decl[name])
+    assert set(_lib.SIGNATURES) | {'toa_adam_abi_version', 'toa_adam_error_string'} == set(decl)
+
+
+def test_abi_version_and_error_strings():
+    lib = _lib.load()
+    assert lib.toa_adam_abi_version() == _lib.ABI_VERSION
+    assert lib.toa_adam_error_string(0) == b'success'
+    for code in (-1, -2, -3):
+        assert b'toa_adam' in lib.toa_adam_error_string(code)
+    with pytest.raises(RuntimeError, match='unsupported dtype'):
+        _lib.check(-1, 'x')
+
+
+def test_argument_errors_need_no_device():
+    """Bad dtype and empty inputs return before any HIP call."""
+    lib = _lib.load()
+    assert lib.toa_adam_forward_inplace(5, None, None, None, 0, 0.9, 0.999, 1e-8, 0.0, 1, None) == -1
+    assert lib.toa_adam_forward_inplace(0, None, None, None, 0, 0.9, 0.999, 1e-8, 0.0, 1, None) == 0
+    assert lib.toa_adam_forward_inplace(0, None, None, None, 8, 0.9, 0.999, 1e-8, 0.0, 1, None) == -2
+    assert lib.toa_adam_backward_updates(1, None, None, None, 0, 0.9, 0.999, 0.0, 1, None, None,
+                                         None) == 0
+    assert lib.toa_adam_forward_inplace_multi(0, 0, None, None, None, None, 0.9, 0.999, 1e-8, 0.0,
+                                              None, 1, None) == 0
+    assert lib.toa_adam_forward_inplace_multi(3, 2, None, None, None, None, 0.9, 0.999, 1e-8, 0.0,
+                                              None, 1, None) == -1
+    assert lib.toa_adam_forward_inplace_multi(0, 2, None, None, None, None, 0.9, 0.999, 1e-8, 0.0,
+                                              None, 1, None) == -2
+
+
+def test_waves_knob_round_trip():
+    lib = _lib.load()
+    first = lib.toa_adam_set_waves_per_cu(16)
+    assert lib.toa_adam_set_waves_per_cu(99) == 16  # out of range restores the per-op defaults
+    assert lib.toa_adam_set_waves_per_cu(first) == 0
+
+
+def test_python_surface_names_and_keywords():
+    """The seven functions and their keyword names as the reference registers them
+    (/root/reference/src/adam_op/adam_op.cpp:157-214)."""
+    want = {
+        'forward_': ['updates', 'mu', 'nu', 'b1', 'b2', 'eps', 'eps_root', 'count'],
+        'forward_mu': ['updates', 'mu', 'b1'],
+        'forward_nu': ['updates', 'nu', 'b2'],
+        'forward_updates': ['new_mu', 'new_nu', 'b1', 'b2', 'eps', 'eps_root', 'count'],
+        'backward_mu': ['dmu', 'updates', 'mu', 'b1'],
+        'backward_nu': ['dnu', 'updates', 'nu', 'b1'],
+        'backward_updates': ['dupdates', 'updates', 'new_mu', 'new_nu', 'b1', 'b2', 'eps_root',
+                             'count'],
+    }
+    for name, params in want.items():
+        assert list(inspect.signature(getattr(adam_op, name)).parameters) == params
+
+
+def test_cpu_and_meta_tensors_are_refused_not_computed():
+    """No CPU path hides behind the op: other devices raise the reference's own error."""
+    a = torch.ones(4)
+    for fn, args in [
+        (adam_op.forward_, (a, a.clone(), a.clone(), 0.9, 0.999, 1e-8, 0.0, 1)),
+        (adam_op.forward_mu, (a, a, 0.9)),
+        (adam_op.forward_nu, (a, a, 0.999)),
+        (adam_op.forward_updates, (a, a, 0.9, 0.999, 1e-8, 0.0, 1)),
+        (adam_op.backward_mu, (a, a, a, 0.9)),
+        (adam_op.backward_nu, (a, a, a, 0.999)),
+        (adam_op.backward_updates, (a, a, a, a, 0.9, 0.999, 0.0, 1)),
+        (adam_op.forward_multi_, ([a], [a.clone()], [a.clone()], 0.9, 0.999, 1e-8, 0.0, 1)),
+    ]:
+        with pytest.raises(RuntimeError, match='Not implemented'):
+            fn(*args)
+    m = torch.ones(4, device='meta')
+    with pytest.raises(RuntimeError, match='Not implemented'):
+        adam_op.forward_mu(m, m, 0.9)
+    assert torch.equal(a, torch.ones(4))  # untouched
+
+
+def test_availability_probe_semantics():
+    """tests/test_accelerated_op.py:36-40 of the reference: `meta` is never available; here the
+    CPU is not served either, and `cuda` follows the machine."""
+    assert not accelerated_op_available('meta')
+    assert not accelerated_op_available(torch.device('meta'))
+    assert not accelerated_op_available('cpu')
+    assert not accelerated_op_available(['cpu', 'meta'])
+    if not torch.cuda.is_available():
+        assert not accelerated_op_available()
+        assert not accelerated_op_available('cuda')
+        assert not accelerated_op_available('cuda:0')
+        assert not accelerated_op_available(0)
+        assert not accelerated_op_available(['cuda', 'cpu'])
+
+
+def test_adam_op_passes_none_updates_through():
+    """accelerated_op/adam_op.py:148-149 of the reference."""
+    mu, nu = torch.ones(3), torch.ones(3)
+    for inplace in (True, False):
+        r = AdamOp(inplace=inplace)(mu, nu, None, 1)
+        assert r[0] is mu and r[1] is nu and r[2] is None
+
+
+def test_adam_op_defaults_and_function_classes():
+    op = AdamOp()
+    assert (op.b1, op.b2, op.eps, op.eps_root, op.inplace) == (0.9, 0.999, 1e-8, 0.0, True)
+    with pytest.raises(TypeError):
+        AdamOp(0.9, 0.999, 1e-8, 0.0)  # eps_root and inplace are keyword-only
+    for cls in (AdamOp.MuOp, AdamOp.NuOp, AdamOp.UpdatesOp):
+        assert issubclass(cls, torch.autograd.Function)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, '_lib', None)
+    monkeypatch.setattr(_lib, 'LIB_PATH', str(tmp_path / 'libtoa_adam.so'))
+    with pytest.raises(ImportError, match='no fallback'):
+        _lib.load()
+
+
+def test_product_never_imports_the_oracle():
+    """The oracle is test infrastructure; nothing under torchopt_amd/ may reference it."""
+    pkg = os.path.join(REPO, 'torchopt_amd')
+    for root, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith(('.py', '.hip', '.hpp', '.h')):
+                text = open(os.path.join(root, f)).read()
+                assert not re.search(r'^\s*(from|import)\s+oracle\b', text, flags=re.M), f
+                assert 'liboracle' not in text and 'adam_oracle' not in text, f

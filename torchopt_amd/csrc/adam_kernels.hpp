@@ -2,16 +2,23 @@
 //
 // Every op here is a pure streaming pass: a handful of flops per element
 // against 12-48 bytes of HBM traffic, so the kernels are shaped for memory
-// throughput and nothing else:
-//   * 128-bit accesses (4 x f32 or 2 x f64 per lane); one wave instruction
+// throughput and nothing else.  What measurement on MI355X settled:
+//   * 128-bit accesses (4 x f32 or 2 x f64 per lane): one wave instruction
 //     covers 1 KiB of contiguous memory;
-//   * a tile is kBlock * UNROLL vectors per stream; a lane issues all of its
-//     loads for a tile (UNROLL per input stream) before the first use, so a
-//     64-wide wave keeps UNROLL * NIN KiB in flight;
-//   * a bounded grid of workgroups walks the tiles with a grid stride, so at
-//     any moment the chip touches one moving window of each stream;
-//   * streams are touched once, so loads and stores carry the non-temporal
-//     hint.
+//   * a workgroup is ONE wavefront and handles ONE tile (1 KiB of every
+//     stream).  The grid has one workgroup per tile, so the hardware
+//     dispatcher hands out tiles in address order and the set of tiles in
+//     flight is one compact window that slides through each array -- DRAM
+//     pages and the TLB see a sequential stream even though thousands of
+//     waves run at once.  Coarser tiles, contiguous per-workgroup chunks and
+//     persistent grid-stride grids all measured 5-20 % slower on the
+//     read-modify-write stream;
+//   * residency is capped per op (kWavesPerCU, enforced through a dynamic-LDS
+//     reservation made at launch): more bytes in flight than the memory
+//     system needs only lengthens queues and widens the window.  The in-place
+//     step peaks at 13 waves per CU, the out-of-place ops at 24-32;
+//   * every array is touched once, so loads and stores carry the
+//     non-temporal hint (worth ~10 %).
 //
 // Arithmetic follows /root/reference/src/adam_op/adam_op_impl_cpu.cpp to the
 // rounding: every product and sum is rounded on its own (build with
@@ -25,7 +32,7 @@
 
 namespace toa {
 
-constexpr int kBlock = 256;  // 4 waves of 64
+constexpr int kBlock = 64;  // one wavefront per workgroup
 
 template <typename T>
 struct Vec;
@@ -58,13 +65,15 @@ __device__ __forceinline__ double toa_sqrt(double x) { return sqrt(x); }
 
 // ---------------------------------------------------------------------------
 // Element-wise ops.  Pointer slots: inputs first, then outputs; an in-place op
-// writes output j back to input slot out_slot(j).
+// writes output j back to input slot out_slot(j).  kWavesPerCU is the measured
+// best number of resident single-wave workgroups per compute unit.
 // ---------------------------------------------------------------------------
 
 // adam_op_impl_cpu.cpp:47-61.  Slots: 0 updates, 1 mu, 2 nu.
 template <typename T>
 struct ForwardInplace {
     static constexpr int NIN = 3, NOUT = 3, NPTR = 3;
+    static constexpr int kWavesPerCU = 13;  // read-modify-write: a tight window wins
     // outputs are produced as (mu', nu', updates') and stored in that order
     __device__ static constexpr int out_slot(int j) { return j == 0 ? 1 : (j == 1 ? 2 : 0); }
     T b1, b2, c1, c2, eps, eps_root;
@@ -84,6 +93,7 @@ struct ForwardInplace {
 template <typename T>
 struct ForwardMu {
     static constexpr int NIN = 2, NOUT = 1, NPTR = 3;
+    static constexpr int kWavesPerCU = 24;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T b1;
     __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
@@ -95,6 +105,7 @@ struct ForwardMu {
 template <typename T>
 struct ForwardNu {
     static constexpr int NIN = 2, NOUT = 1, NPTR = 3;
+    static constexpr int kWavesPerCU = 24;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T b2;
     __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
@@ -107,6 +118,7 @@ struct ForwardNu {
 template <typename T>
 struct ForwardUpdates {
     static constexpr int NIN = 2, NOUT = 1, NPTR = 3;
+    static constexpr int kWavesPerCU = 32;  // sqrt and divide: needs the waves to hide ALU time
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T c1, c2, eps, eps_root;
     __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
@@ -120,6 +132,7 @@ struct ForwardUpdates {
 template <typename T>
 struct BackwardMu {
     static constexpr int NIN = 1, NOUT = 2, NPTR = 3;
+    static constexpr int kWavesPerCU = 24;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T b1;
     __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
@@ -132,6 +145,7 @@ struct BackwardMu {
 template <typename T>
 struct BackwardNu {
     static constexpr int NIN = 2, NOUT = 2, NPTR = 4;
+    static constexpr int kWavesPerCU = 24;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T b2;
     __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
@@ -145,6 +159,7 @@ struct BackwardNu {
 template <typename T>
 struct BackwardUpdates {
     static constexpr int NIN = 3, NOUT = 2, NPTR = 5;
+    static constexpr int kWavesPerCU = 24;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T p1, q2;
     __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
@@ -161,8 +176,8 @@ struct BackwardUpdates {
 };
 
 // ---------------------------------------------------------------------------
-// Tile processing.  A tile is kBlock * UNROLL vectors (TILE = that * Vec<T>::N
-// elements) of one tensor.
+// Tile processing.  A tile is kBlock * UNROLL vectors (that * Vec<T>::N
+// elements) of one tensor; the library instantiates UNROLL = 1.
 // ---------------------------------------------------------------------------
 
 template <typename T, int UNROLL>
@@ -306,7 +321,8 @@ __device__ __forceinline__ void process_tile(const Op &op, const TensorPtrs<T, O
 }
 
 // ---------------------------------------------------------------------------
-// Single-tensor kernel: workgroups stride over the tensor's tiles.
+// Single-tensor kernel: one workgroup per tile (the stride loop only runs more
+// than once for tensors beyond the grid limit).
 // ---------------------------------------------------------------------------
 template <typename T, class Op, int UNROLL, bool NT>
 __global__ __launch_bounds__(kBlock) void stream_kernel(const Op op, const TensorPtrs<T, Op> tp,

@@ -11,6 +11,7 @@
 
 #include <atomic>
 #include <cmath>
+#include <cstdlib>
 #include <vector>
 
 #include "adam_kernels.hpp"
@@ -20,29 +21,42 @@ namespace {
 using namespace toa;
 
 // Launch shape of the streaming kernels (see adam_kernels.hpp).
-constexpr int kUnroll = 4;          // 16-byte loads in flight per lane per input stream
-constexpr bool kNonTemporal = true; // streams are touched once
-constexpr int kBlocksPerCU = 8;     // resident workgroups the grid is capped at, per CU
+constexpr int kUnroll = 1;           // one 16-byte access per lane per stream
+constexpr bool kNonTemporal = true;  // every array is touched once
+constexpr unsigned kMaxGrid = 1u << 25;  // workgroups per launch; larger tensors stride
+constexpr int kLdsPerCU = 160 * 1024;    // gfx950
 
-constexpr int kMaxDevices = 64;
-std::atomic<int> g_cu_count[kMaxDevices];
+// Global override of the per-op resident-wave cap: -1 = not yet initialised,
+// 0 = use each op's own kWavesPerCU, 1..32 = that many for every op.  Set by
+// toa_adam_set_waves_per_cu() or, initially, by the environment variable
+// TOA_ADAM_WAVES_PER_CU (read once).
+std::atomic<int> g_waves_override{-1};
 
-int cu_count() {
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
-    int n = g_cu_count[dev].load(std::memory_order_relaxed);
-    if (n == 0) {
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-            n <= 0)
-            n = 256;
-        g_cu_count[dev].store(n, std::memory_order_relaxed);
+int waves_override() {
+    int w = g_waves_override.load(std::memory_order_relaxed);
+    if (w < 0) {
+        w = 0;
+        if (const char *env = std::getenv("TOA_ADAM_WAVES_PER_CU")) {
+            const int v = std::atoi(env);
+            if (v >= 1 && v <= 32) w = v;
+        }
+        g_waves_override.store(w, std::memory_order_relaxed);
     }
-    return n;
+    return w;
+}
+
+// Dynamic LDS bytes that let exactly `waves` single-wave workgroups fit on a CU.
+// The kernels never touch LDS; the reservation only bounds residency.
+template <class Op>
+unsigned lds_reservation() {
+    const int o = waves_override();
+    const int w = o ? o : Op::kWavesPerCU;
+    if (w >= 32) return 0;  // 32 waves per CU is the hardware limit anyway
+    return (unsigned)((kLdsPerCU / w) & ~1023);
 }
 
 unsigned grid_for(size_t num_tiles) {
-    const size_t cap = (size_t)cu_count() * kBlocksPerCU;
-    return (unsigned)(num_tiles < cap ? num_tiles : cap);
+    return (unsigned)(num_tiles < kMaxGrid ? num_tiles : kMaxGrid);
 }
 
 struct HostScalars {
@@ -68,7 +82,8 @@ int launch_single(const Op &op, T *const (&ptrs)[Op::NPTR], size_t n, void *stre
     constexpr size_t tile = Tile<T, kUnroll>::ELEMS;
     const size_t num_tiles = (n + tile - 1) / tile;
     hipLaunchKernelGGL((stream_kernel<T, Op, kUnroll, kNonTemporal>), dim3(grid_for(num_tiles)),
-                       dim3(kBlock), 0, (hipStream_t)stream, op, tp, n, num_tiles);
+                       dim3(kBlock), lds_reservation<Op>(), (hipStream_t)stream, op, tp, n,
+                       num_tiles);
     return (int)hipGetLastError();
 }
 
@@ -114,8 +129,8 @@ int launch_multi(MakeOp make_op, size_t num, const void *const *const (&lists)[O
             if (tab.num == 0) return 0;
             const uint32_t total = tab.tile_start[tab.num];
             hipLaunchKernelGGL((multi_stream_kernel<T, Op, kUnroll, kNonTemporal>),
-                               dim3(grid_for(total)), dim3(kBlock), 0, (hipStream_t)stream, op,
-                               tab);
+                               dim3(grid_for(total)), dim3(kBlock), lds_reservation<Op>(),
+                               (hipStream_t)stream, op, tab);
             tab.num = 0;
             return (int)hipGetLastError();
         };
@@ -162,6 +177,12 @@ T *mut(const void *p) {
 extern "C" {
 
 int toa_adam_abi_version(void) { return 1; }
+
+int toa_adam_set_waves_per_cu(int waves) {
+    const int prev = waves_override();
+    g_waves_override.store(waves >= 1 && waves <= 32 ? waves : 0, std::memory_order_relaxed);
+    return prev;
+}
 
 const char *toa_adam_error_string(int code) {
     switch (code) {
