@@ -39,10 +39,11 @@ BYTES_PER_ELEM = {  # op -> number of arrays streamed (multiply by the element s
     'backward_mu': 3, 'backward_nu': 4, 'backward_updates': 5,
 }
 
-# HBM bytes per launch of the config-2 kernel as counted by rocprofv3 --pmc (FETCH_SIZE and
-# WRITE_SIZE, each scaled by what the same counter reads for a plain copy of known size);
-# see profiles/.  None until measured for the current kernel.
-MEASURED_TRAFFIC_BYTES = {2: None}
+# HBM bytes per step as counted by rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE in separate runs,
+# each scaled by what the same counter reads for a plain 1 GiB copy: x1.99996 and x1.0); the
+# commands and raw readings are in profiles/*pmc_traffic*.md.  Not measured live: a counter run
+# serialises the kernels, so it cannot share a process with the timed region.
+MEASURED_TRAFFIC_BYTES = {2: 6442485175, 4: 8516628944}
 
 B1, B2, EPS = 0.9, 0.999, 1e-8
 
@@ -120,7 +121,21 @@ def run_gpu(cfg_id, steps, warmup):
 
         sizes = [numel(s) for s in cfg['shapes']]
         total = sum(sizes)
-        tensors = [make_state(torch, n, dtype, 1000 * cfg_id + k) for k, n in enumerate(sizes)]
+        # Allocation order as the Adam transformation produces it: the gradients of the whole
+        # tree, then mu for every leaf, then nu for every leaf (init_fn maps zeros_like over
+        # the tree once per moment, /root/reference/torchopt/transform/scale_by_adam.py:401-414),
+        # so the three arrays of one leaf lie far apart.
+        gens = []
+        for k in range(len(sizes)):
+            g = torch.Generator(device='cuda')
+            g.manual_seed(1000 * cfg_id + k)
+            gens.append(g)
+        us = [torch.randn(n, device='cuda', dtype=dtype, generator=g) for n, g in zip(sizes, gens)]
+        ms = [torch.randn(n, device='cuda', dtype=dtype, generator=g).mul_(0.1)
+              for n, g in zip(sizes, gens)]
+        vs = [torch.randn(n, device='cuda', dtype=dtype, generator=g).mul_(0.01).abs_()
+              for n, g in zip(sizes, gens)]
+        tensors = list(zip(us, ms, vs))
         num = len(sizes)
         pu = (ctypes.c_void_p * num)(*[t[0].data_ptr() for t in tensors])
         pm = (ctypes.c_void_p * num)(*[t[1].data_ptr() for t in tensors])
@@ -257,6 +272,10 @@ def main(argv=None):
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--config', type=int, default=2, choices=sorted(CONFIGS))
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--pmc-calibration', action='store_true',
+                    help='after the timed region also run 5 plain device copies of 1 GiB, so a '
+                         'rocprofv3 --pmc run holds a kernel of known traffic to scale '
+                         'FETCH_SIZE / WRITE_SIZE by')
     args = ap.parse_args(argv)
 
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
@@ -267,6 +286,15 @@ def main(argv=None):
 
     gpu = run_gpu(args.config, args.steps, args.warmup)
     cfg = CONFIGS[args.config]
+    if args.pmc_calibration:
+        import torch
+
+        src = torch.ones(1 << 28, device='cuda')
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
     line = {
         'metric': 'adam_forward_inplace_elements_per_s',
         'value': gpu['value'],

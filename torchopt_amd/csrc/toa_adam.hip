@@ -25,6 +25,9 @@ constexpr int kUnroll = 1;           // one 16-byte access per lane per stream
 constexpr bool kNonTemporal = true;  // every array is touched once
 constexpr unsigned kMaxGrid = 1u << 25;  // workgroups per launch; larger tensors stride
 constexpr int kLdsPerCU = 160 * 1024;    // gfx950
+// The multi-tensor kernel spends three dependent scalar loads finding its tensor
+// before any memory traffic starts; a few more resident waves cover that.
+constexpr int kMultiExtraWaves = 4;
 
 // Global override of the per-op resident-wave cap: -1 = not yet initialised,
 // 0 = use each op's own kWavesPerCU, 1..32 = that many for every op.  Set by
@@ -48,9 +51,9 @@ int waves_override() {
 // Dynamic LDS bytes that let exactly `waves` single-wave workgroups fit on a CU.
 // The kernels never touch LDS; the reservation only bounds residency.
 template <class Op>
-unsigned lds_reservation() {
+unsigned lds_reservation(int extra_waves = 0) {
     const int o = waves_override();
-    const int w = o ? o : Op::kWavesPerCU;
+    const int w = o ? o : Op::kWavesPerCU + extra_waves;
     if (w >= 32) return 0;  // 32 waves per CU is the hardware limit anyway
     return (unsigned)((kLdsPerCU / w) & ~1023);
 }
@@ -91,17 +94,18 @@ int launch_single(const Op &op, T *const (&ptrs)[Op::NPTR], size_t n, void *stre
 // scalars for one step number; tensors are batched per distinct count and per
 // kernel-argument table capacity.
 template <typename T, class Op, class MakeOp>
-int launch_multi(MakeOp make_op, size_t num, const void *const *const (&lists)[Op::NPTR],
+int launch_multi(MakeOp make_op, size_t num_tensors,
+                 const void *const *const (&lists)[Op::NPTR],
                  const size_t *n, const uint64_t *counts, uint64_t count_all, void *stream) {
     using Table = MultiTable<T, Op>;
     constexpr size_t tile = Tile<T, kUnroll>::ELEMS;
-    if (num == 0) return 0;
+    if (num_tensors == 0) return 0;
     if (n == nullptr) return TOA_ENULL;
     for (int i = 0; i < Op::NPTR; ++i)
         if (lists[i] == nullptr) return TOA_ENULL;
 
     // validate everything before the first launch
-    for (size_t k = 0; k < num; ++k) {
+    for (size_t k = 0; k < num_tensors; ++k) {
         if (n[k] == 0) continue;
         for (int i = 0; i < Op::NPTR; ++i)
             if (lists[i][k] == nullptr) return TOA_ENULL;
@@ -112,7 +116,7 @@ int launch_multi(MakeOp make_op, size_t num, const void *const *const (&lists)[O
     if (counts == nullptr) {
         distinct.push_back(count_all);
     } else {
-        for (size_t k = 0; k < num; ++k) {
+        for (size_t k = 0; k < num_tensors; ++k) {
             if (n[k] == 0) continue;
             bool seen = false;
             for (uint64_t c : distinct) seen |= (c == counts[k]);
@@ -121,32 +125,41 @@ int launch_multi(MakeOp make_op, size_t num, const void *const *const (&lists)[O
     }
 
     Table tab;
+    uint32_t num = 0;       // tensors in the table being filled
+    uint32_t next_tile = 0; // tiles in the table being filled
+    auto reset = [&]() {
+        num = 0;
+        next_tile = 0;
+        for (int g = 0; g < kMaxGroups; ++g) tab.coarse[g] = kNoTile;
+        for (int g = 0; g < Table::GROUPS; ++g)
+            for (int i = 0; i < kGroup; ++i) tab.group[g].start[i] = kNoTile;
+    };
     for (uint64_t c : distinct) {
         const Op op = make_op(c);
-        tab.num = 0;
-        tab.tile_start[0] = 0;
+        reset();
         auto flush = [&]() -> int {
-            if (tab.num == 0) return 0;
-            const uint32_t total = tab.tile_start[tab.num];
+            if (num == 0) return 0;
+            tab.total = next_tile;
             hipLaunchKernelGGL((multi_stream_kernel<T, Op, kUnroll, kNonTemporal>),
-                               dim3(grid_for(total)), dim3(kBlock), lds_reservation<Op>(),
-                               (hipStream_t)stream, op, tab);
-            tab.num = 0;
+                               dim3(grid_for(next_tile)), dim3(kBlock),
+                               lds_reservation<Op>(kMultiExtraWaves), (hipStream_t)stream, op,
+                               tab);
+            reset();
             return (int)hipGetLastError();
         };
-        for (size_t k = 0; k < num; ++k) {
+        for (size_t k = 0; k < num_tensors; ++k) {
             if (n[k] == 0 || (counts != nullptr && counts[k] != c)) continue;
             const uint64_t tiles = (n[k] + tile - 1) / tile;
-            if (tab.num == (uint32_t)Table::MAX ||
-                (uint64_t)tab.tile_start[tab.num] + tiles > 0xffffffffu) {
+            if (num == (uint32_t)Table::MAX || (uint64_t)next_tile + tiles >= kNoTile) {
                 if (int rc = flush()) return rc;
             }
-            const uint32_t t = tab.num;
             for (int i = 0; i < Op::NPTR; ++i)
-                tab.p[i][t] = static_cast<T *>(const_cast<void *>(lists[i][k]));
-            tab.n[t] = n[k];
-            tab.tile_start[t + 1] = tab.tile_start[t] + (uint32_t)tiles;
-            tab.num = t + 1;
+                tab.rec[num].p[i] = static_cast<T *>(const_cast<void *>(lists[i][k]));
+            tab.rec[num].n = n[k];
+            tab.group[num / kGroup].start[num % kGroup] = next_tile;
+            if (num % kGroup == 0 && num > 0) tab.coarse[num / kGroup - 1] = next_tile;
+            next_tile += (uint32_t)tiles;
+            ++num;
         }
         if (int rc = flush()) return rc;
     }
