@@ -1,0 +1,233 @@
+"""`scale_by_accelerated_adam` and `MultiAdamOp` on the GPU: tree handling, count bookkeeping,
+in-place and differentiable branches, against the CPU oracle leaf by leaf, against the per-leaf
+`AdamOp`, and against `torch.optim.Adam` as the library routine the whole chain reduces to."""
+
+from __future__ import annotations
+
+import collections
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import assert_bit_equal
+from oracle import adam_oracle as O
+from torchopt_amd import AdamOp, MultiAdamOp
+from torchopt_amd.transform import scale_by_accelerated_adam
+from torchopt_amd.transform.scale_by_adam import _host_value
+
+import bench
+
+pytestmark = pytest.mark.gpu
+
+B1, B2, EPS = 0.9, 0.999, 1e-8
+Point = collections.namedtuple('Point', 'w b')
+
+
+@pytest.fixture(scope='module', autouse=True)
+def _gpu():
+    assert torch.cuda.is_available(), 'these tests need a GPU; there is no fallback path'
+    yield
+    torch.cuda.synchronize()
+
+
+def host(t):
+    return t.detach().cpu().numpy()
+
+
+def dev(a):
+    return torch.as_tensor(np.array(a)).cuda()  # keeps 0-dim leaves 0-dim
+
+
+def make_tree(dtype, seed):
+    rng = np.random.default_rng(seed)
+    r = lambda *s: np.asarray(rng.standard_normal(s), dtype=dtype)  # noqa: E731
+    return {'conv': Point(r(8, 3, 3, 3), r(8)), 'skip': None, 'head': [r(5, 40), r(5)],
+            'scalar': r()}
+
+
+def tree_leaves(tree):
+    return [tree['conv'].w, tree['conv'].b, tree['head'][0], tree['head'][1], tree['scalar']]
+
+
+def to_dev(tree):
+    return {'conv': Point(dev(tree['conv'].w), dev(tree['conv'].b)), 'skip': None,
+            'head': [dev(tree['head'][0]), dev(tree['head'][1])], 'scalar': dev(tree['scalar'])}
+
+
+@pytest.mark.parametrize('dtype', [np.float32, np.float64], ids=['f32', 'f64'])
+def test_inplace_steps_on_a_nested_tree(dtype):
+    """Five optimizer steps; one leaf misses its gradient on steps 2 and 3, so its count lags."""
+    t = scale_by_accelerated_adam(B1, B2, EPS, eps_root=0.0)
+    params = to_dev(make_tree(dtype, 0))
+    state = t.init(params)
+    h_mu = [np.zeros_like(a) for a in tree_leaves(make_tree(dtype, 0))]
+    h_nu = [np.zeros_like(a) for a in h_mu]
+    h_count = [0] * 5
+    for step in range(1, 6):
+        h_grads = make_tree(dtype, 100 + step)
+        grads = to_dev(h_grads)
+        missing = step in (2, 3)
+        if missing:
+            grads['head'][1] = None
+        old_state = state
+        updates, state = t.update(grads, state, params=params, inplace=True)
+        # structure and identity: in place, the outputs are the inputs
+        assert isinstance(updates['conv'], Point) and updates['skip'] is None
+        assert updates['conv'].w is grads['conv'].w
+        assert state.mu['conv'].w is old_state.mu['conv'].w
+        if missing:
+            assert updates['head'][1] is None
+            assert state.count['head'][1] is old_state.count['head'][1]
+        for k, (g, got_u, got_m, got_v, got_c) in enumerate(zip(
+                tree_leaves(h_grads), tree_leaves(updates), tree_leaves(state.mu),
+                tree_leaves(state.nu), tree_leaves(state.count))):
+            if missing and k == 3:
+                pass
+            else:
+                h_count[k] += 1
+                g = np.ascontiguousarray(g).reshape(-1).copy()
+                O.forward_inplace(g, h_mu[k].reshape(-1), h_nu[k].reshape(-1), B1, B2, EPS, 0.0,
+                                  h_count[k])
+                assert_bit_equal(host(got_u).reshape(-1), g, f'step {step} leaf {k} updates')
+            assert_bit_equal(host(got_m), h_mu[k], f'step {step} leaf {k} mu')
+            assert_bit_equal(host(got_v), h_nu[k], f'step {step} leaf {k} nu')
+            assert got_c.dim() == 0 and got_c.dtype == torch.int64 and got_c.is_cuda
+            assert int(got_c) == h_count[k] == _host_value(got_c)
+    assert h_count == [5, 5, 5, 3, 5]
+
+
+def test_flat_variant_matches_tree_variant():
+    dtype = np.float32
+    sizes = [bench.numel(s) for s in bench.maml_shapes()]
+    rng = np.random.default_rng(3)
+    grads = [rng.standard_normal(n).astype(dtype) for n in sizes]
+    flat = scale_by_accelerated_adam.flat(B1, B2, EPS, 1e-8)
+    tree = scale_by_accelerated_adam(B1, B2, EPS, 1e-8)
+    p_flat = tuple(dev(g) for g in grads)
+    p_tree = {'p': [dev(g) for g in grads]}
+    s_flat, s_tree = flat.init(p_flat), tree.init(p_tree)
+    assert isinstance(s_flat.mu, tuple)
+    for _ in range(3):
+        u_flat, s_flat = flat.update(tuple(dev(g) for g in grads), s_flat, inplace=True)
+        u_tree, s_tree = tree.update({'p': [dev(g) for g in grads]}, s_tree, inplace=True)
+    assert isinstance(u_flat, tuple) and isinstance(s_flat.nu, tuple)
+    for a, b in zip(u_flat, u_tree['p']):
+        assert torch.equal(a, b)
+    for a, b in zip(s_flat.nu, s_tree.nu['p']):
+        assert torch.equal(a, b)
+
+
+def test_count_state_restored_from_elsewhere_is_read_once():
+    """Counts that did not come from this transformation (a loaded checkpoint) carry no host
+    mirror: they are read from the device, and the step uses their value."""
+    t = scale_by_accelerated_adam(B1, B2, EPS)
+    g = np.random.default_rng(1).standard_normal(1000).astype(np.float32)
+    state = t.init([dev(g)])
+    restored = state._replace(count=[torch.tensor(41, device='cuda')])
+    updates, new_state = t.update([dev(g)], restored, inplace=True)
+    assert int(new_state.count[0]) == 42
+    e = g.copy()
+    O.forward_inplace(e, np.zeros_like(g), np.zeros_like(g), B1, B2, EPS, 0.0, 42)
+    assert_bit_equal(host(updates[0]), e, 'count 42')
+
+
+def test_differentiable_branch_matches_per_leaf_adam_op():
+    """inplace=False: the list-level autograd Functions give the same values and the same
+    gradients as the reference-shaped per-leaf AdamOp, bit for bit."""
+    shapes = bench.maml_shapes()
+    rng = np.random.default_rng(11)
+    data = [[rng.standard_normal(s).astype(np.float32) for _ in range(3)] for s in shapes]
+    cots = [[rng.standard_normal(s).astype(np.float32) for _ in range(3)] for s in shapes]
+    count, eps_root = 5, 1e-8
+
+    def leaves():
+        return [[dev(a).requires_grad_(True) for a in (g, 0.1 * m, np.abs(0.01 * v))]
+                for g, m, v in data]
+
+    # per leaf
+    single = leaves()
+    op = AdamOp(B1, B2, EPS, eps_root=eps_root, inplace=False)
+    outs = [op(m, v, g, count) for g, m, v in single]
+    torch.autograd.backward([o for out in outs for o in out],
+                            [dev(c) for ct in cots for c in ct])
+    # whole list
+    multi = leaves()
+    mop = MultiAdamOp(B1, B2, EPS, eps_root=eps_root, inplace=False)
+    new_mu, new_nu, new_u = mop([x[1] for x in multi], [x[2] for x in multi],
+                                [x[0] for x in multi], count)
+    flat_out = [o for trio in zip(new_mu, new_nu, new_u) for o in trio]
+    assert all(o.requires_grad for o in flat_out)
+    torch.autograd.backward(flat_out, [dev(c) for ct in cots for c in ct])
+    for k in range(len(shapes)):
+        for a, b, what in zip(outs[k], (new_mu[k], new_nu[k], new_u[k]), ('mu', 'nu', 'updates')):
+            assert torch.equal(a, b), f'leaf {k} new {what}'
+        for a, b, what in zip(single[k], multi[k], ('updates', 'mu', 'nu')):
+            assert torch.equal(a.grad, b.grad), f'leaf {k} grad wrt {what}'
+
+
+def test_meta_step_through_the_transformation():
+    """A MAML-style inner step: params' = params - lr * adam(grad); the outer loss
+    differentiates through the update, the moments and the step."""
+    torch.manual_seed(0)
+    w = torch.randn(6, 4, device='cuda', dtype=torch.float64, requires_grad=True)
+    b = torch.randn(6, device='cuda', dtype=torch.float64, requires_grad=True)
+    x = torch.randn(16, 4, device='cuda', dtype=torch.float64)
+    y = torch.randn(16, 6, device='cuda', dtype=torch.float64)
+    t = scale_by_accelerated_adam(B1, B2, EPS, eps_root=1e-8, moment_requires_grad=True)
+    state = t.init((w, b))
+
+    def inner_loss(w_, b_):
+        return ((x @ w_.t() + b_ - y) ** 2).mean()
+
+    grads = torch.autograd.grad(inner_loss(w, b), (w, b), create_graph=True)
+    updates, state = t.update(grads, state, params=(w, b), inplace=False)
+    assert isinstance(updates, tuple) and updates[0].requires_grad
+    w1, b1 = w - 0.1 * updates[0], b - 0.1 * updates[1]
+    outer = inner_loss(w1, b1)
+    gw, gb = torch.autograd.grad(outer, (w, b))
+    assert torch.isfinite(gw).all() and torch.isfinite(gb).all() and gw.abs().sum() > 0
+    # same computation through the per-leaf reference-shaped op
+    op = AdamOp(B1, B2, EPS, eps_root=1e-8, inplace=False)
+    grads2 = torch.autograd.grad(inner_loss(w, b), (w, b), create_graph=True)
+    z = [torch.zeros_like(p, requires_grad=True) for p in (w, b)]
+    z2 = [torch.zeros_like(p, requires_grad=True) for p in (w, b)]
+    u2 = [op(m, v, g, 1)[2] for m, v, g in zip(z, z2, grads2)]
+    outer2 = inner_loss(w - 0.1 * u2[0], b - 0.1 * u2[1])
+    gw2, gb2 = torch.autograd.grad(outer2, (w, b))
+    # three gradient paths meet at w; their summation order may differ between the two graphs
+    torch.testing.assert_close(gw, gw2, rtol=1e-12, atol=1e-14)
+    torch.testing.assert_close(gb, gb2, rtol=1e-12, atol=1e-14)
+
+
+@pytest.mark.parametrize('inplace', [True, False])
+def test_chain_reduces_to_torch_optim_adam(inplace):
+    """With eps_root = 0 the chain scale_by_adam -> scale(-lr) -> apply is torch.optim.Adam;
+    the reference pins its accelerated path the same way, in float64, at 25x the default
+    tolerance (/root/reference/tests/test_alias.py:207-270, tests/helpers.py:202-229)."""
+    torch.manual_seed(1)
+    lr = 1e-2
+    model = torch.nn.Sequential(torch.nn.Linear(20, 32), torch.nn.Tanh(),
+                                torch.nn.Linear(32, 5)).to('cuda', torch.float64)
+    ref = torch.nn.Sequential(torch.nn.Linear(20, 32), torch.nn.Tanh(),
+                              torch.nn.Linear(32, 5)).to('cuda', torch.float64)
+    ref.load_state_dict(model.state_dict())
+    base = [p.detach().clone() for p in model.parameters()]
+    optim_ref = torch.optim.Adam(ref.parameters(), lr, betas=(B1, B2), eps=EPS)
+    t = scale_by_accelerated_adam(B1, B2, EPS, eps_root=0.0)
+    params = tuple(model.parameters())
+    state = t.init(params)
+    for step in range(5):
+        x = torch.randn(64, 20, device='cuda', dtype=torch.float64)
+        y = torch.randint(0, 5, (64,), device='cuda')
+        loss = torch.nn.functional.cross_entropy(model(x), y)
+        grads = torch.autograd.grad(loss, params)
+        updates, state = t.update(grads, state, params=params, inplace=inplace)
+        with torch.no_grad():
+            for p, u in zip(params, updates):
+                p.add_(u, alpha=-lr)
+        optim_ref.zero_grad()
+        torch.nn.functional.cross_entropy(ref(x), y).backward()
+        optim_ref.step()
+    for p, q, p0 in zip(model.parameters(), ref.parameters(), base):
+        torch.testing.assert_close(p - p0, q - p0, rtol=25 * 1e-7, atol=25 * 1e-7)

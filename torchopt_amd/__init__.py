@@ -6,9 +6,9 @@
 """
 
 from torchopt_amd import accelerated_op
-from torchopt_amd.accelerated_op import AdamOp
+from torchopt_amd.accelerated_op import AdamOp, MultiAdamOp
 from torchopt_amd.accelerated_op import is_available as accelerated_op_available
 
 __version__ = '0.1.0'
 
-__all__ = ['AdamOp', 'accelerated_op', 'accelerated_op_available']
+__all__ = ['AdamOp', 'MultiAdamOp', 'accelerated_op', 'accelerated_op_available']

@@ -7,9 +7,9 @@ from typing import Iterable, Union
 
 import torch
 
-from torchopt_amd.accelerated_op.adam_op import AdamOp
+from torchopt_amd.accelerated_op.adam_op import AdamOp, MultiAdamOp
 
-__all__ = ['AdamOp', 'is_available']
+__all__ = ['AdamOp', 'MultiAdamOp', 'is_available']
 
 Device = Union[torch.device, str, int]
 
