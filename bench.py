@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused Adam operator on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config {0,2,3,4}]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config {0,1,2,3,4}]
 
 A "step" is one pass of the hot path over one batch of synthetic state that is already
 resident in HBM: for the default workload (config 2) one fused in-place `forward_` over three
@@ -76,6 +76,9 @@ def numel(shape):
 CONFIGS = {
     0: dict(name='config0: fused forward_ in place, 1 048 576 float32 elements, count=10',
             dtype='f32', n=1 << 20, eps_root=0.0, count=10),
+    1: dict(name='config1: forward mu/nu/updates + backward updates/nu/mu over the MAML pytree '
+                 '(10 float32 tensors, 32 645 elements), six multi-tensor launches per step',
+            dtype='f32', shapes=maml_shapes(), eps_root=1e-8, count=5, differentiable=True),
     2: dict(name='config2: fused forward_ in place, 268 435 456 float32 elements '
                  '(1 GiB per state array), count=1000',
             dtype='f32', n=1 << 28, eps_root=0.0, count=1000),
@@ -116,7 +119,72 @@ def run_gpu(cfg_id, steps, warmup):
     sptr = stream.cuda_stream
     eps_root, count = cfg['eps_root'], cfg['count']
 
-    if 'shapes' in cfg:
+    bytes_per_elem = BYTES_PER_ELEM['forward_'] * esize
+    if cfg.get('differentiable'):
+        import ctypes
+
+        sizes = [numel(s) for s in cfg['shapes']]
+        total, num = sum(sizes), len(sizes)
+        g = torch.Generator(device='cuda')
+        g.manual_seed(1000 * cfg_id)
+
+        def fresh():
+            return [torch.randn(n, device='cuda', dtype=dtype, generator=g) for n in sizes]
+
+        def arr(ts):
+            return (ctypes.c_void_p * num)(*[t.data_ptr() for t in ts])
+
+        ups, mus, nus = fresh(), [t.mul_(0.1) for t in fresh()], [t.mul_(0.01).abs_() for t in fresh()]
+        d_u, d_m, d_v = fresh(), fresh(), fresh()
+        outs = [fresh() for _ in range(9)]  # new_mu, new_nu, new_u, 2 x 3 backward outputs
+        keep = (ups, mus, nus, d_u, d_m, d_v, outs)  # noqa: F841  (owns the device memory)
+        a_up, a_mu, a_nu, a_du, a_dm, a_dv = (arr(x) for x in (ups, mus, nus, d_u, d_m, d_v))
+        o = [arr(x) for x in outs]
+        ns = (ctypes.c_size_t * num)(*sizes)
+
+        def check(rc):
+            if rc:
+                raise RuntimeError(lib.toa_adam_error_string(rc).decode())
+
+        def step():
+            check(lib.toa_adam_forward_mu_multi(code, num, a_up, a_mu, ns, B1, o[0], sptr))
+            check(lib.toa_adam_forward_nu_multi(code, num, a_up, a_nu, ns, B2, o[1], sptr))
+            check(lib.toa_adam_forward_updates_multi(code, num, o[0], o[1], ns, B1, B2, EPS,
+                                                     eps_root, None, count, o[2], sptr))
+            check(lib.toa_adam_backward_updates_multi(code, num, a_du, o[2], o[0], ns, B1, B2,
+                                                      eps_root, None, count, o[3], o[4], sptr))
+            check(lib.toa_adam_backward_nu_multi(code, num, a_dv, a_up, ns, B2, o[5], o[6], sptr))
+            check(lib.toa_adam_backward_mu_multi(code, num, a_dm, ns, B1, o[7], o[8], sptr))
+
+        ptrs = [[t.data_ptr() for t in x] for x in (ups, mus, nus, d_u, d_m, d_v, *outs)]
+
+        def per_tensor_step():  # what the reference's per-leaf loop launches: 6 kernels per leaf
+            for k, n in enumerate(sizes):
+                p = [x[k] for x in ptrs]
+                lib.toa_adam_forward_mu(code, p[0], p[1], n, B1, p[6], sptr)
+                lib.toa_adam_forward_nu(code, p[0], p[2], n, B2, p[7], sptr)
+                lib.toa_adam_forward_updates(code, p[6], p[7], n, B1, B2, EPS, eps_root, count,
+                                             p[8], sptr)
+                lib.toa_adam_backward_updates(code, p[3], p[8], p[6], n, B1, B2, eps_root, count,
+                                              p[9], p[10], sptr)
+                lib.toa_adam_backward_nu(code, p[5], p[0], n, B2, p[11], p[12], sptr)
+                lib.toa_adam_backward_mu(code, p[4], n, B1, p[13], p[14], sptr)
+
+        for _ in range(warmup):
+            per_tensor_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            per_tensor_step()
+        torch.cuda.synchronize()
+        per_leaf_ms = (time.perf_counter() - t0) * 1e3 / steps
+        bytes_per_elem = sum(BYTES_PER_ELEM[k] for k in (
+            'forward_mu', 'forward_nu', 'forward_updates', 'backward_updates', 'backward_nu',
+            'backward_mu')) * esize
+        extra = {'tensors': num, 'launches_per_step': 6,
+                 'per_leaf_loop_ms_per_step': round(per_leaf_ms, 5),
+                 'per_leaf_loop_launches_per_step': 6 * num}
+    elif 'shapes' in cfg:
         import ctypes
 
         sizes = [numel(s) for s in cfg['shapes']]
@@ -175,7 +243,7 @@ def run_gpu(cfg_id, steps, warmup):
 
     wall_ms = (t1 - t0) * 1e3 / steps
     kern_ms = ev0.elapsed_time(ev1) / steps  # stream time per launch (launches are back to back)
-    alg_bytes = BYTES_PER_ELEM['forward_'] * esize * total
+    alg_bytes = bytes_per_elem * total
     achieved = alg_bytes / (kern_ms * 1e-3) / 1e9
     traffic = MEASURED_TRAFFIC_BYTES.get(cfg_id)
     return {
@@ -186,7 +254,7 @@ def run_gpu(cfg_id, steps, warmup):
             'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
             'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': traffic,
             'kernel_ms': round(kern_ms, 5), 'algorithmic_bytes_per_launch': alg_bytes,
-            'bytes_per_element': BYTES_PER_ELEM['forward_'] * esize,
+            'bytes_per_element': bytes_per_elem,
         },
         'extra': extra,
         'device': torch.cuda.get_device_name(0),
@@ -296,7 +364,8 @@ def main(argv=None):
         torch.cuda.synchronize()
         del src, dst
     line = {
-        'metric': 'adam_forward_inplace_elements_per_s',
+        'metric': ('adam_forward_backward_elements_per_s' if cfg.get('differentiable')
+                   else 'adam_forward_inplace_elements_per_s'),
         'value': gpu['value'],
         'unit': 'elements/s',
         'n_gpus': 1,

@@ -149,5 +149,41 @@ void oracle_adam_host_scalars(double b1, double b2, double eps_root, uint64_t co
         }                                                                                      \
     }
 
+/* The classic in-place optimizer step as the reference chain performs it, three
+ * passes restated as three statements per element (element-wise, so the order of
+ * passes and elements is immaterial):
+ *   1. [maximize] g = -g                 /root/reference/torchopt/alias/utils.py:148
+ *   2. Adam forward_ in place            adam_op_impl_cpu.cpp:32-91
+ *   3. updates *= -lr (scalar rounded to T)  /root/reference/torchopt/transform/scale.py:93-98
+ *   4. params += updates                 /root/reference/torchopt/update.py:71-74
+ * With write_updates == 0 the updates array is left as it was (the fused GPU
+ * step can skip that store); params, mu and nu are the same either way. */
+#define ORACLE_DEFINE_STEP(T, SFX, SQRT)                                                       \
+    void oracle_adam_fused_step_##SFX(T *params, T *updates, T *mu, T *nu, size_t n,           \
+                                      double b1_, double b2_, double eps_, double eps_root_,   \
+                                      uint64_t count, double lr_, int maximize,                \
+                                      int write_updates) {                                     \
+        double s[4];                                                                           \
+        oracle_adam_host_scalars(b1_, b2_, eps_root_, count, s);                               \
+        const T b1 = (T)b1_, b2 = (T)b2_, eps = (T)eps_, eps_root = (T)eps_root_;              \
+        const T c1 = (T)s[0], c2 = (T)s[1], neg_lr = (T)(-lr_);                                \
+        PAR_FOR(n)                                                                             \
+        for (size_t i = 0; i < n; ++i) {                                                       \
+            const T g = maximize ? -updates[i] : updates[i];                                   \
+            const T m1 = b1 * mu[i] + (1 - b1) * g;                                            \
+            const T v1 = b2 * nu[i] + (1 - b2) * g * g;                                        \
+            const T mh = m1 * c1;                                                              \
+            const T vh = v1 * c2;                                                              \
+            const T u1 = mh / (SQRT(vh + eps_root) + eps);                                     \
+            const T step = u1 * neg_lr;                                                        \
+            mu[i] = m1;                                                                        \
+            nu[i] = v1;                                                                        \
+            params[i] = params[i] + step;                                                      \
+            if (write_updates) updates[i] = step;                                              \
+        }                                                                                      \
+    }
+
 ORACLE_DEFINE(float, f32, sqrtf)
 ORACLE_DEFINE(double, f64, sqrt)
+ORACLE_DEFINE_STEP(float, f32, sqrtf)
+ORACLE_DEFINE_STEP(double, f64, sqrt)

@@ -17,8 +17,11 @@
  *   compiled CPU op on seeded and edge-case inputs (tests/golden fixtures,
  *   written by tests/golden/make_golden.py), and against an independent
  *   NumPy one-rounding-per-operation specification (oracle/adam_spec.py);
- *   plus closed forms in tests/test_oracle.py.  No function is "parity
- *   unpinned".
+ *   plus closed forms in tests/test_oracle.py;
+ *   oracle_adam_fused_step_*: bit-for-bit against the reference chain itself run
+ *   on CPU -- the compiled reference forward_ followed by the two torch calls the
+ *   reference makes (Tensor.mul_(-lr), Tensor.add_) -- in tests/test_oracle.py.
+ *   No function is "parity unpinned".
  */
 #ifndef ADAM_ORACLE_H
 #define ADAM_ORACLE_H
@@ -79,6 +82,16 @@ void oracle_adam_backward_updates_f64(const double *dupdates, const double *upda
                                       const double *new_mu, size_t n, double b1, double b2,
                                       double eps_root, uint64_t count, double *dnew_mu_out,
                                       double *dnew_nu_out);
+
+/* The reference chain's classic in-place step: [negate], Adam forward_, updates *= -lr,
+ * params += updates (alias/utils.py:148, adam_op_impl_cpu.cpp:32-91, transform/scale.py:93-98,
+ * update.py:71-74). */
+void oracle_adam_fused_step_f32(float *params, float *updates, float *mu, float *nu, size_t n,
+                                double b1, double b2, double eps, double eps_root,
+                                uint64_t count, double lr, int maximize, int write_updates);
+void oracle_adam_fused_step_f64(double *params, double *updates, double *mu, double *nu, size_t n,
+                                double b1, double b2, double eps, double eps_root,
+                                uint64_t count, double lr, int maximize, int write_updates);
 
 /* Host-side bias-correction scalars in double, before the cast to the element
  * type (adam_op_impl_cpu.cpp:73-74, 191-192, 328-329).

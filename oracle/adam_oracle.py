@@ -120,6 +120,17 @@ def backward_updates(dupdates, updates, new_mu, b1, b2, eps_root, count):
     return dm, dn
 
 
+def fused_step(params, updates, mu, nu, b1, b2, eps, eps_root, count, lr, maximize=False,
+               write_updates=True):
+    """Mutates params, mu, nu (and updates when write_updates), like the reference's classic
+    in-place chain: [negate], forward_, scale by -lr, apply."""
+    _fn('fused_step', params.dtype)(_ptr(params), _ptr(updates), _ptr(mu), _ptr(nu),
+                                    _SZ(params.size), _D(b1), _D(b2), _D(eps), _D(eps_root),
+                                    _U64(count), _D(lr), ctypes.c_int(int(maximize)),
+                                    ctypes.c_int(int(write_updates)))
+    return params, updates, mu, nu
+
+
 def reference_path():
     hits = sorted(glob.glob(os.path.join(_HERE, '_ref', '_C*.so')))
     return hits[0] if hits else None

@@ -1,0 +1,151 @@
+"""The one-pass optimizer step (Adam, scale by -lr, add to the parameters) against the CPU
+oracle of the reference's three-pass chain, against the unfused chain run on the GPU, and
+through the `FusedAdam` optimizer."""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import assert_bit_equal
+from oracle import adam_oracle as O
+from torchopt_amd import FusedAdam
+from torchopt_amd._C import adam_op
+from torchopt_amd.transform import scale_by_accelerated_adam
+
+pytestmark = pytest.mark.gpu
+
+B1, B2, EPS = 0.9, 0.999, 1e-8
+
+
+@pytest.fixture(scope='module', autouse=True)
+def _gpu():
+    assert torch.cuda.is_available(), 'these tests need a GPU; there is no fallback path'
+    yield
+    torch.cuda.synchronize()
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    return t.detach().cpu().numpy()
+
+
+def rand4(dtype, n, seed):
+    rng = np.random.default_rng(seed)
+    return (rng.standard_normal(n).astype(dtype), rng.standard_normal(n).astype(dtype),
+            (0.1 * rng.standard_normal(n)).astype(dtype),
+            np.abs(0.01 * rng.standard_normal(n)).astype(dtype))
+
+
+@pytest.mark.parametrize('dtype', [np.float32, np.float64], ids=['f32', 'f64'])
+@pytest.mark.parametrize('maximize', [False, True])
+@pytest.mark.parametrize('write_updates', [False, True])
+def test_single_tensor_against_oracle(dtype, maximize, write_updates):
+    for k, n in enumerate([1, 3, 255, 256, 257, 1025, 65537, (1 << 20) + 3]):
+        lr, count, eps_root = (1e-3, 1, 0.0) if k % 2 else (0.05, 1000, 1e-8)
+        p, g, m, v = rand4(dtype, n, 200 + n)
+        gp, gg, gm, gv = dev(p), dev(g), dev(m), dev(v)
+        r = adam_op.fused_step_(gp, gg, gm, gv, B1, B2, EPS, eps_root, count, lr,
+                                maximize=maximize, write_updates=write_updates)
+        assert r[0] is gp and r[1] is gg
+        O.fused_step(p, g, m, v, B1, B2, EPS, eps_root, count, lr, maximize, write_updates)
+        assert_bit_equal(host(gp), p, f'n={n} params')
+        assert_bit_equal(host(gm), m, f'n={n} mu')
+        assert_bit_equal(host(gv), v, f'n={n} nu')
+        assert_bit_equal(host(gg), g, f'n={n} updates (untouched unless write_updates)')
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float64], ids=['f32', 'f64'])
+def test_equals_the_unfused_chain_on_the_gpu(dtype):
+    """forward_ then Tensor.mul_(-lr) then Tensor.add_ -- the reference's three passes, with
+    PyTorch's own GPU kernels for the last two -- give the same bits as the one-pass step."""
+    n, lr, count = (1 << 22) + 5, 3e-4, 12
+    g = torch.Generator(device='cuda').manual_seed(5)
+    p = torch.randn(n, device='cuda', dtype=dtype, generator=g)
+    u = torch.randn(n, device='cuda', dtype=dtype, generator=g)
+    m = torch.randn(n, device='cuda', dtype=dtype, generator=g).mul_(0.1)
+    v = torch.randn(n, device='cuda', dtype=dtype, generator=g).mul_(0.01).abs_()
+    p2, u2, m2, v2 = p.clone(), u.clone(), m.clone(), v.clone()
+    adam_op.forward_(u, m, v, B1, B2, EPS, 0.0, count)
+    u.mul_(-lr)
+    p.add_(u)
+    adam_op.fused_step_(p2, u2, m2, v2, B1, B2, EPS, 0.0, count, lr, write_updates=True)
+    assert torch.equal(p, p2) and torch.equal(u, u2) and torch.equal(m, m2) and torch.equal(v, v2)
+
+
+def test_multi_tensor_with_ragged_members_and_counts():
+    sizes = [1000, 0, 17, 300_001, 256, 5] + [33] * 100  # crosses one kernel-argument table
+    counts = [(k % 3) + 1 for k in range(len(sizes))]
+    hs = [rand4(np.float32, n, 300 + k) for k, n in enumerate(sizes)]
+    ds = [[dev(a) for a in h] for h in hs]
+    r = adam_op.fused_step_multi_([d[0] for d in ds], [d[1] for d in ds], [d[2] for d in ds],
+                                  [d[3] for d in ds], B1, B2, EPS, 1e-8, counts, 0.01,
+                                  maximize=True, write_updates=False)
+    assert r[0][0] is ds[0][0]
+    for k, (h, d) in enumerate(zip(hs, ds)):
+        O.fused_step(h[0], h[1], h[2], h[3], B1, B2, EPS, 1e-8, counts[k], 0.01, True, False)
+        for j, what in enumerate(('params', 'updates', 'mu', 'nu')):
+            assert_bit_equal(host(d[j]), h[j], f'tensor {k} {what}')
+
+
+@pytest.mark.parametrize('maximize', [False, True])
+def test_fused_adam_equals_the_transformation_chain(maximize):
+    """FusedAdam.step() against scale_by_accelerated_adam -> mul_(-lr) -> add_ on clones, over
+    several steps with a parameter whose gradient is missing on some steps."""
+    torch.manual_seed(3)
+    lr = 2e-3
+    shapes = [(64, 32), (64,), (10, 64), (10,), ()]
+    params = [torch.randn(s, device='cuda', requires_grad=True) for s in shapes]
+    twins = [p.detach().clone() for p in params]
+    opt = FusedAdam(params, lr, eps_root=1e-8, maximize=maximize)
+    chain = scale_by_accelerated_adam(B1, B2, EPS, eps_root=1e-8)
+    state = chain.init(tuple(twins))
+    for step in range(6):
+        opt.zero_grad(set_to_none=True)
+        grads = [torch.randn(s, device='cuda') for s in shapes]
+        if step in (1, 4):
+            grads[3] = None
+        for p, g in zip(params, grads):
+            p.grad = None if g is None else g.clone()
+        opt.step()
+        # p.grad is left alone by the fused step
+        assert all(p.grad is None or torch.equal(p.grad, g) for p, g in zip(params, grads))
+        ups = tuple(None if g is None else (g.neg() if maximize else g.clone()) for g in grads)
+        ups, state = chain.update(ups, state, params=tuple(twins), inplace=True)
+        for t, u in zip(twins, ups):
+            if u is not None:
+                t.add_(u.mul_(-lr))
+        for k, (p, t) in enumerate(zip(params, twins)):
+            assert torch.equal(p.detach(), t), f'step {step} param {k}'
+    st = opt.state_dict()[0]
+    assert [int(c) for c in st.count] == [6, 6, 6, 4, 6]
+    for a, b in zip(st.mu, state.mu):
+        assert torch.equal(a, b)
+    # the state round-trips and can be handed to the transformation
+    opt.load_state_dict(opt.state_dict())
+    chain.update(tuple(torch.randn(s, device='cuda') for s in shapes), st, inplace=True)
+
+
+def test_fused_adam_tracks_torch_optim_adam():
+    torch.manual_seed(0)
+    net = torch.nn.Sequential(torch.nn.Linear(16, 32), torch.nn.ReLU(),
+                              torch.nn.Linear(32, 4)).to('cuda', torch.float64)
+    ref = torch.nn.Sequential(torch.nn.Linear(16, 32), torch.nn.ReLU(),
+                              torch.nn.Linear(32, 4)).to('cuda', torch.float64)
+    ref.load_state_dict(net.state_dict())
+    a = FusedAdam(net.parameters(), 1e-2)
+    b = torch.optim.Adam(ref.parameters(), 1e-2)
+    for _ in range(10):
+        x = torch.randn(32, 16, device='cuda', dtype=torch.float64)
+        y = torch.randn(32, 4, device='cuda', dtype=torch.float64)
+        for model, opt in ((net, a), (ref, b)):
+            opt.zero_grad()
+            loss = ((model(x) - y) ** 2).mean()
+            loss.backward()
+            opt.step()
+    for p, q in zip(net.parameters(), ref.parameters()):
+        torch.testing.assert_close(p, q, rtol=25e-7, atol=25e-7)

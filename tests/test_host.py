@@ -34,7 +34,8 @@ def test_header_declares_the_expected_surface():
     singles = {'forward_inplace', 'forward_mu', 'forward_nu', 'forward_updates', 'backward_mu',
                'backward_nu', 'backward_updates'}
     want = {f'toa_adam_{s}' for s in singles} | {f'toa_adam_{s}_multi' for s in singles}
-    want |= {'toa_adam_abi_version', 'toa_adam_error_string', 'toa_adam_set_waves_per_cu'}
+    want |= {'toa_adam_abi_version', 'toa_adam_error_string', 'toa_adam_set_waves_per_cu',
+             'toa_adam_fused_step', 'toa_adam_fused_step_multi'}
     assert names == want
 
 
@@ -153,6 +154,26 @@ def test_adam_op_defaults_and_function_classes():
         AdamOp(0.9, 0.999, 1e-8, 0.0)  # eps_root and inplace are keyword-only
     for cls in (AdamOp.MuOp, AdamOp.NuOp, AdamOp.UpdatesOp):
         assert issubclass(cls, torch.autograd.Function)
+
+
+def test_fused_adam_argument_validation():
+    from torchopt_amd import FusedAdam
+
+    p = [torch.ones(3)]
+    for kwargs in (dict(lr=-1.0), dict(eps=-1.0), dict(betas=(1.0, 0.9)), dict(betas=(0.9, 1.0)),
+                   dict(weight_decay=0.01), dict(lr=lambda c: 0.1)):
+        with pytest.raises(ValueError):
+            FusedAdam(p, **kwargs)
+    with pytest.raises(TypeError):
+        FusedAdam([1.0])
+    opt = FusedAdam(p)
+    assert opt.state_dict() == (None,)
+    opt.zero_grad()  # no grads yet: nothing to do
+    assert opt.step() is None  # no grads: nothing is launched, counts stay at zero
+    assert [int(c) for c in opt.state_dict()[0].count] == [0]
+    p[0].grad = torch.ones(3)
+    with pytest.raises(RuntimeError, match='Not implemented'):  # CPU parameters are refused
+        opt.step()
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

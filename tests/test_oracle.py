@@ -145,6 +145,52 @@ def test_c_oracle_equals_compiled_reference(dtype):
             assert_bit_equal(a, b.numpy())
 
 
+@pytest.mark.parametrize('dtype', DTYPES, ids=['f32', 'f64'])
+@pytest.mark.parametrize('maximize', [False, True])
+def test_fused_step_is_the_reference_chain(dtype, maximize):
+    """The classic in-place step of the reference is three passes: [neg_], forward_,
+    Tensor.mul_(-lr) (transform/scale.py:93-98) and Tensor.add_ (update.py:71-74).  Run exactly
+    those calls on CPU tensors -- forward_ from the compiled reference where it is built, else
+    from the pinned C oracle -- and compare the one-pass oracle with them."""
+    import torch
+
+    ref = O.load_reference()
+    rng = np.random.default_rng(31)
+    for n, lr, count, eps_root in [(1, 1e-3, 1, 0.0), (1003, 1e-3, 7, 0.0), (200_003, 0.05, 1000, 1e-8)]:
+        g, m, v = _rand(dtype, n, n)
+        p = rng.standard_normal(n).astype(dtype)
+        tg, tm, tv, tp = (torch.from_numpy(x.copy()) for x in (g, m, v, p))
+        if maximize:
+            tg.neg_()
+        if ref is not None:
+            ref.adam_op.forward_(tg, tm, tv, 0.9, 0.999, 1e-8, eps_root, count)
+        else:
+            O.forward_inplace(tg.numpy(), tm.numpy(), tv.numpy(), 0.9, 0.999, 1e-8, eps_root, count)
+        tg.mul_(-lr)
+        tp.add_(tg)
+        for write_updates in (True, False):
+            op, og, om, ov = p.copy(), g.copy(), m.copy(), v.copy()
+            O.fused_step(op, og, om, ov, 0.9, 0.999, 1e-8, eps_root, count, lr, maximize,
+                         write_updates)
+            assert_bit_equal(op, tp.numpy(), 'params')
+            assert_bit_equal(om, tm.numpy(), 'mu')
+            assert_bit_equal(ov, tv.numpy(), 'nu')
+            assert_bit_equal(og, tg.numpy() if write_updates else g, 'updates')
+
+
+def test_fused_step_scales_by_the_rounded_learning_rate():
+    """In float32 the step is u * float32(-lr), not float32(u * -lr in double): pick lr = 0.1."""
+    one = np.ones(8, np.float32)
+    p = np.zeros(8, np.float32)
+    g = one.copy()
+    O.fused_step(p, g, np.zeros(8, np.float32), np.zeros(8, np.float32), 0.9, 0.999, 0.0, 0.0, 1,
+                 0.1, False, True)
+    u = O.forward_inplace(one.copy(), np.zeros(8, np.float32), np.zeros(8, np.float32), 0.9, 0.999,
+                          0.0, 0.0, 1)[0]
+    assert_bit_equal(g, u * np.float32(-0.1))
+    assert_bit_equal(p, np.float32(0) + u * np.float32(-0.1))
+
+
 # ---------------------------------------------------------------------------------------------
 # What the mathematics fixes
 # ---------------------------------------------------------------------------------------------

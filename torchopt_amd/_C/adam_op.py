@@ -18,7 +18,9 @@ Differences from the reference, all deliberate:
     length is handled (the reference's device kernels drop the last n % 4
     elements for n >= 1024, adam_op_impl_cuda.cu:95-96);
   * additive multi-tensor entry points (`forward_multi_`, ...) run a whole list
-    of tensors in one launch.
+    of tensors in one launch;
+  * additive `fused_step_` / `fused_step_multi_` run the classic in-place step
+    (Adam, scale by -lr, add to the parameters) in one pass.
 """
 
 from __future__ import annotations
@@ -47,6 +49,8 @@ __all__ = [
     'backward_mu_multi',
     'backward_nu_multi',
     'backward_updates_multi',
+    'fused_step_',
+    'fused_step_multi_',
 ]
 
 _DTYPES = {torch.float32: _lib.TOA_F32, torch.float64: _lib.TOA_F64}
@@ -443,3 +447,50 @@ def backward_updates_multi(dupdates, updates, new_mu, new_nu, b1, b2, eps_root, 
                 _ptr_array(dmu_out), _ptr_array(dnu_out), stream)
         _lib.check(rc, name)
     return dmu_out, dnu_out
+
+
+# --------------------------------------------------------------------------- fused optimizer step
+
+
+def fused_step_(params, updates, mu, nu, b1, b2, eps, eps_root, count, lr, *, maximize=False,
+                write_updates=False):
+    """The classic in-place step in one pass: `forward_`, then ``updates *= -lr``
+    (/root/reference/torchopt/transform/scale.py:93-98) and ``params += updates``
+    (/root/reference/torchopt/update.py:71-74), bit-identical to the three passes.
+
+    Overwrites `params`, `mu`, `nu`; `updates` receives the scaled update only if
+    `write_updates` (the reference chain leaves it there), otherwise it is only read.
+    `maximize` negates the gradient first (/root/reference/torchopt/alias/utils.py:148).
+    Returns ``[params, updates, mu, nu]``.
+    """
+    name = 'adamFusedStep'
+    code, n = _gate(name, updates, (mu, nu, params))
+    c = _count(count)
+    if n:
+        for what, t in (('params', params), ('updates', updates), ('mu', mu), ('nu', nu)):
+            _require_dense(name, what, t)
+        if n > 1 and not (params.stride() == updates.stride() == mu.stride() == nu.stride()):
+            raise RuntimeError(f'{name}: params, updates, mu and nu must share one memory layout')
+        with _on_device_of(updates) as stream:
+            rc = _lib.load().toa_adam_fused_step(
+                code, params.data_ptr(), updates.data_ptr(), mu.data_ptr(), nu.data_ptr(), n,
+                b1, b2, eps, eps_root, c, lr, int(bool(maximize)), int(bool(write_updates)),
+                stream)
+        _lib.check(rc, name)
+    return [params, updates, mu, nu]
+
+
+def fused_step_multi_(params, updates, mu, nu, b1, b2, eps, eps_root, counts, lr, *,
+                      maximize=False, write_updates=False):
+    """`fused_step_` over lists of tensors; returns ``(params, updates, mu, nu)``."""
+    name = 'adamFusedStepMulti'
+    code, num = _gate_multi(name, (updates, mu, nu, params))
+    if num:
+        carr, call = _counts_array(counts, num)
+        with _on_device_of(updates[0]) as stream:
+            rc = _lib.load().toa_adam_fused_step_multi(
+                code, num, _ptr_array(params), _ptr_array(updates), _ptr_array(mu),
+                _ptr_array(nu), _size_array(updates), b1, b2, eps, eps_root, carr, call, lr,
+                int(bool(maximize)), int(bool(write_updates)), stream)
+        _lib.check(rc, name)
+    return params, updates, mu, nu

@@ -8,7 +8,8 @@
 from torchopt_amd import accelerated_op
 from torchopt_amd.accelerated_op import AdamOp, MultiAdamOp
 from torchopt_amd.accelerated_op import is_available as accelerated_op_available
+from torchopt_amd.optim import FusedAdam
 
 __version__ = '0.1.0'
 
-__all__ = ['AdamOp', 'MultiAdamOp', 'accelerated_op', 'accelerated_op_available']
+__all__ = ['AdamOp', 'FusedAdam', 'MultiAdamOp', 'accelerated_op', 'accelerated_op_available']

@@ -175,6 +175,38 @@ struct BackwardUpdates {
     }
 };
 
+// The classic optimizer step in one pass: the in-place Adam step followed by what
+// the reference chain does next with its result -- scale by -lr
+// (/root/reference/torchopt/transform/scale.py:93-98 via alias/utils.py:226) and
+// add to the parameters (/root/reference/torchopt/update.py:71-74) -- each still
+// rounded on its own, so the result equals the three separate passes bit for
+// bit while streaming 28 (or 32) bytes per float32 element instead of 44.
+// `maximize` negates the gradient first (alias/utils.py:148).
+// Slots: 0 updates (gradients), 1 mu, 2 nu, 3 params.
+template <typename T, bool WRITE_UPDATES>
+struct FusedStep {
+    static constexpr int NIN = 4, NOUT = WRITE_UPDATES ? 4 : 3, NPTR = 4;
+    static constexpr int kWavesPerCU = 13;
+    // outputs: mu', nu', params', then the scaled update
+    __device__ static constexpr int out_slot(int j) { return j == 3 ? 0 : j + 1; }
+    T b1, b2, c1, c2, eps, eps_root, neg_lr;
+    bool maximize;
+    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
+        const T g = maximize ? -in[0] : in[0];
+        const T m = in[1], v = in[2], p = in[3];
+        const T m1 = b1 * m + (1 - b1) * g;
+        const T v1 = b2 * v + (1 - b2) * g * g;
+        const T mh = m1 * c1;
+        const T vh = v1 * c2;
+        const T u1 = mh / (toa_sqrt(vh + eps_root) + eps);
+        const T step = u1 * neg_lr;
+        out[0] = m1;
+        out[1] = v1;
+        out[2] = p + step;
+        if constexpr (WRITE_UPDATES) out[3] = step;
+    }
+};
+
 // ---------------------------------------------------------------------------
 // Tile processing.  A tile is kBlock * UNROLL vectors (that * Vec<T>::N
 // elements) of one tensor; the library instantiates UNROLL = 1.
