@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused Adam operator on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config {0,1,2,3,4}]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config {0,1,2,3,4,5}]
 
 A "step" is one pass of the hot path over one batch of synthetic state that is already
 resident in HBM: for the default workload (config 2) one fused in-place `forward_` over three
@@ -87,6 +87,9 @@ CONFIGS = {
     4: dict(name='config4: multi-tensor forward_ in place over the GPT-2-medium parameter list '
                  '(float32), count=1',
             dtype='f32', shapes=gpt2_medium_shapes(), eps_root=0.0, count=1),
+    5: dict(name='config5: classic optimizer step (Adam + scale(-lr) + apply) in one pass over the '
+                 'GPT-2-medium parameter list (float32), count=1; beside it the three-pass chain',
+            dtype='f32', shapes=gpt2_medium_shapes(), eps_root=0.0, count=1, fused_step=True),
 }
 
 
@@ -216,6 +219,34 @@ def run_gpu(cfg_id, steps, warmup):
             if rc:
                 raise RuntimeError(lib.toa_adam_error_string(rc).decode())
         extra = {'tensors': num}
+        if cfg.get('fused_step'):
+            ps = [torch.randn(n, device='cuda', dtype=dtype, generator=g)
+                  for n, g in zip(sizes, gens)]
+            pp = (ctypes.c_void_p * num)(*[t.data_ptr() for t in ps])
+            lr = 1e-3
+
+            def chain_step():  # the reference's three passes, per-leaf PyTorch kernels for two
+                step()
+                torch._foreach_mul_(us, -lr)
+                torch._foreach_add_(ps, us)
+
+            for _ in range(3):
+                chain_step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                chain_step()
+            torch.cuda.synchronize()
+            chain_ms = (time.perf_counter() - t0) * 1e3 / steps
+
+            def step():  # noqa: F811
+                rc = lib.toa_adam_fused_step_multi(code, num, pp, pu, pm, pv, ns, B1, B2, EPS,
+                                                   eps_root, None, count, lr, 0, 0, sptr)
+                if rc:
+                    raise RuntimeError(lib.toa_adam_error_string(rc).decode())
+            bytes_per_elem = 7 * esize  # reads g, mu, nu, p; writes mu, nu, p
+            extra.update(three_pass_chain_ms_per_step=round(chain_ms, 5),
+                         three_pass_chain_bytes_per_element=11 * esize)
     else:
         total = cfg['n']
         u, mu, nu = make_state(torch, total, dtype, 1000 * cfg_id)
@@ -365,6 +396,7 @@ def main(argv=None):
         del src, dst
     line = {
         'metric': ('adam_forward_backward_elements_per_s' if cfg.get('differentiable')
+                   else 'adam_fused_step_elements_per_s' if cfg.get('fused_step')
                    else 'adam_forward_inplace_elements_per_s'),
         'value': gpu['value'],
         'unit': 'elements/s',
