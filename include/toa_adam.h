@@ -11,7 +11,7 @@
  * replaced by (pointer, n, dtype).
  *
  * Conventions
- *   dtype     TOA_F32 or TOA_F64; all arrays of one call share it.
+ *   dtype     one of the TOA_F* codes below; all arrays of one call share it.
  *   pointers  device memory on the CURRENT HIP device, contiguous, n elements
  *             each.  Any alignment is accepted; 16-byte aligned pointers take
  *             the 128-bit path.  In toa_adam_forward_inplace the three arrays
@@ -41,10 +41,14 @@ extern "C" {
 
 #define TOA_API __attribute__((visibility("default")))
 
-enum { TOA_F32 = 0, TOA_F64 = 1 };
+/* Element types.  TOA_F16 (IEEE half) and TOA_BF16 (bfloat16) follow the arithmetic the
+ * reference CPU op performs on at::Half / at::BFloat16 tensors: every operation between two
+ * 16-bit values is rounded back to 16 bits, the square root and division of the update run in
+ * float and are rounded once.  The fused optimizer step takes TOA_F32 / TOA_F64 only. */
+enum { TOA_F32 = 0, TOA_F64 = 1, TOA_F16 = 2, TOA_BF16 = 3 };
 
 enum {
-    TOA_EDTYPE = -1, /* dtype is not TOA_F32 / TOA_F64            */
+    TOA_EDTYPE = -1, /* dtype not served by this entry point      */
     TOA_ENULL = -2,  /* a required pointer is NULL while n > 0    */
     TOA_ESIZE = -3   /* a tensor is too large for the launch grid */
 };

@@ -24,6 +24,7 @@
 
 #include <math.h>
 #include <omp.h>
+#include <string.h>
 
 #define MIN_N_PARALLEL 1000u
 
@@ -187,3 +188,183 @@ ORACLE_DEFINE(float, f32, sqrtf)
 ORACLE_DEFINE(double, f64, sqrt)
 ORACLE_DEFINE_STEP(float, f32, sqrtf)
 ORACLE_DEFINE_STEP(double, f64, sqrt)
+
+
+/* ---------------------------------------------------------------------------------------------
+ * Half precision and bfloat16.
+ *
+ * The reference CPU op also dispatches at::Half and at::BFloat16 (include/common.h:26-31 with
+ * USE_FP16 undefined, the default build).  The kernels are then instantiated with scalar_t =
+ * c10::Half / c10::BFloat16, whose arithmetic is: convert both operands to float, operate in
+ * float, and -- when both operands are the 16-bit type (or an int, which converts to it first) --
+ * round the result back to 16 bits; an operation between the 16-bit type and a float (double)
+ * yields a float (double) that is not rounded.  Consequences for adam_op_impl_cpu.cpp:
+ *   - every product, sum and difference in the moment updates is rounded to 16 bits;
+ *   - sqrt(nu_hat + eps_root) is the float overload applied to the 16-bit sum, so the square
+ *     root, "+ eps" and the division run in float and only the quotient is rounded (":59");
+ *   - the tail of backward_updates runs in double after two 16-bit products, and the result
+ *     goes double -> float -> 16 bits (":314-315");
+ *   - every scalar goes double -> float -> 16 bits (":78-84").
+ * Values are kept as float holding an exactly representable 16-bit value; RND() rounds a float
+ * to the format and back.  Storage is uint16_t bit patterns.
+ * ------------------------------------------------------------------------------------------- */
+
+static inline uint32_t f32_bits(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float f32_from(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+/* IEEE binary16 <- binary32, round to nearest even; NaN -> sign | 0x7e00. */
+static inline uint16_t f16_from_f32(float f) {
+    const uint32_t x = f32_bits(f);
+    const uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+    const uint32_t a = x & 0x7fffffffu;
+    if (a > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);
+    if (a >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u); /* >= 65520 rounds to infinity */
+    if (a < 0x38800000u) {                                   /* below 2^-14: subnormal or zero */
+        /* units of 2^-24; exact product, then one round-to-nearest-even to an integer */
+        const float units = nearbyintf(f32_from(a) * 0x1p24f);
+        return (uint16_t)(sign | (uint16_t)units);
+    }
+    uint32_t h = (((a >> 23) - 112u) << 10) | ((a & 0x7fffffu) >> 13);
+    const uint32_t rest = a & 0x1fffu;
+    if (rest > 0x1000u || (rest == 0x1000u && (h & 1u))) ++h; /* carry may bump the exponent */
+    return (uint16_t)(sign | h);
+}
+
+static inline float f32_from_f16(uint16_t h) {
+    const uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+    const uint32_t e = (h >> 10) & 0x1fu, m = h & 0x3ffu;
+    if (e == 0) {
+        const float mag = (float)m * 0x1p-24f;
+        return sign ? -mag : mag;
+    }
+    if (e == 31) return f32_from(sign | 0x7f800000u | (m << 13));
+    return f32_from(sign | ((e + 112u) << 23) | (m << 13));
+}
+
+/* bfloat16 <- binary32: round to nearest even on the upper 16 bits; NaN -> 0x7fc0. */
+static inline uint16_t bf16_from_f32(float f) {
+    const uint32_t x = f32_bits(f);
+    if ((x & 0x7fffffffu) > 0x7f800000u) return 0x7fc0u;
+    return (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);
+}
+static inline float f32_from_bf16(uint16_t b) { return f32_from((uint32_t)b << 16); }
+
+#define ORACLE_DEFINE_LOWP(SFX, TO16, FROM16)                                                  \
+    static inline float rnd_##SFX(float x) { return FROM16(TO16(x)); }                         \
+                                                                                               \
+    void oracle_adam_forward_inplace_##SFX(uint16_t *updates, uint16_t *mu, uint16_t *nu,      \
+                                           size_t n, double b1_, double b2_, double eps_,      \
+                                           double eps_root_, uint64_t count) {                 \
+        double s[4];                                                                           \
+        oracle_adam_host_scalars(b1_, b2_, eps_root_, count, s);                               \
+        const float b1 = rnd_##SFX((float)b1_), b2 = rnd_##SFX((float)b2_);                    \
+        const float eps = rnd_##SFX((float)eps_), er = rnd_##SFX((float)eps_root_);            \
+        const float c1 = rnd_##SFX((float)s[0]), c2 = rnd_##SFX((float)s[1]);                  \
+        PAR_FOR(n)                                                                             \
+        for (size_t i = 0; i < n; ++i) {                                                       \
+            const float g = FROM16(updates[i]), m = FROM16(mu[i]), v = FROM16(nu[i]);          \
+            const float m1 =                                                                   \
+                rnd_##SFX(rnd_##SFX(b1 * m) + rnd_##SFX(rnd_##SFX(1.0f - b1) * g));            \
+            const float v1 = rnd_##SFX(                                                        \
+                rnd_##SFX(b2 * v) + rnd_##SFX(rnd_##SFX(rnd_##SFX(1.0f - b2) * g) * g));       \
+            const float mh = rnd_##SFX(m1 * c1), vh = rnd_##SFX(v1 * c2);                      \
+            const float u1 = mh / (sqrtf(rnd_##SFX(vh + er)) + eps);                           \
+            mu[i] = TO16(m1);                                                                  \
+            nu[i] = TO16(v1);                                                                  \
+            updates[i] = TO16(u1);                                                             \
+        }                                                                                      \
+    }                                                                                          \
+                                                                                               \
+    void oracle_adam_forward_mu_##SFX(const uint16_t *updates, const uint16_t *mu, size_t n,   \
+                                      double b1_, uint16_t *mu_out) {                          \
+        const float b1 = rnd_##SFX((float)b1_);                                                \
+        PAR_FOR(n)                                                                             \
+        for (size_t i = 0; i < n; ++i)                                                         \
+            mu_out[i] = TO16(rnd_##SFX(b1 * FROM16(mu[i])) +                                   \
+                             rnd_##SFX(rnd_##SFX(1.0f - b1) * FROM16(updates[i])));            \
+    }                                                                                          \
+                                                                                               \
+    void oracle_adam_forward_nu_##SFX(const uint16_t *updates, const uint16_t *nu, size_t n,   \
+                                      double b2_, uint16_t *nu_out) {                          \
+        const float b2 = rnd_##SFX((float)b2_);                                                \
+        PAR_FOR(n)                                                                             \
+        for (size_t i = 0; i < n; ++i) {                                                       \
+            const float g = FROM16(updates[i]);                                                \
+            nu_out[i] = TO16(rnd_##SFX(b2 * FROM16(nu[i])) +                                   \
+                             rnd_##SFX(rnd_##SFX(rnd_##SFX(1.0f - b2) * g) * g));              \
+        }                                                                                      \
+    }                                                                                          \
+                                                                                               \
+    void oracle_adam_forward_updates_##SFX(const uint16_t *new_mu, const uint16_t *new_nu,     \
+                                           size_t n, double b1_, double b2_, double eps_,      \
+                                           double eps_root_, uint64_t count,                   \
+                                           uint16_t *updates_out) {                            \
+        double s[4];                                                                           \
+        oracle_adam_host_scalars(b1_, b2_, eps_root_, count, s);                               \
+        const float eps = rnd_##SFX((float)eps_), er = rnd_##SFX((float)eps_root_);            \
+        const float c1 = rnd_##SFX((float)s[0]), c2 = rnd_##SFX((float)s[1]);                  \
+        PAR_FOR(n)                                                                             \
+        for (size_t i = 0; i < n; ++i) {                                                       \
+            const float mh = rnd_##SFX(FROM16(new_mu[i]) * c1);                                \
+            const float vh = rnd_##SFX(FROM16(new_nu[i]) * c2);                                \
+            updates_out[i] = TO16(mh / (sqrtf(rnd_##SFX(vh + er)) + eps));                     \
+        }                                                                                      \
+    }                                                                                          \
+                                                                                               \
+    void oracle_adam_backward_mu_##SFX(const uint16_t *dmu, size_t n, double b1_,              \
+                                       uint16_t *dupdates_out, uint16_t *dmu_out) {            \
+        const float b1 = rnd_##SFX((float)b1_);                                                \
+        PAR_FOR(n)                                                                             \
+        for (size_t i = 0; i < n; ++i) {                                                       \
+            const float d = FROM16(dmu[i]);                                                    \
+            dupdates_out[i] = TO16(rnd_##SFX(1.0f - b1) * d);                                  \
+            dmu_out[i] = TO16(b1 * d);                                                         \
+        }                                                                                      \
+    }                                                                                          \
+                                                                                               \
+    void oracle_adam_backward_nu_##SFX(const uint16_t *dnu, const uint16_t *updates, size_t n, \
+                                       double b2_, uint16_t *dupdates_out,                     \
+                                       uint16_t *dnu_out) {                                    \
+        const float b2 = rnd_##SFX((float)b2_);                                                \
+        PAR_FOR(n)                                                                             \
+        for (size_t i = 0; i < n; ++i) {                                                       \
+            const float d = FROM16(dnu[i]), g = FROM16(updates[i]);                            \
+            dupdates_out[i] =                                                                  \
+                TO16(rnd_##SFX(rnd_##SFX(2.0f * rnd_##SFX(1.0f - b2)) * g) * d);               \
+            dnu_out[i] = TO16(b2 * d);                                                         \
+        }                                                                                      \
+    }                                                                                          \
+                                                                                               \
+    void oracle_adam_backward_updates_##SFX(const uint16_t *dupdates, const uint16_t *updates, \
+                                            const uint16_t *new_mu, size_t n, double b1_,      \
+                                            double b2_, double eps_root_, uint64_t count,      \
+                                            uint16_t *dnew_mu_out, uint16_t *dnew_nu_out) {    \
+        double s[4];                                                                           \
+        oracle_adam_host_scalars(b1_, b2_, eps_root_, count, s);                               \
+        const float p1 = rnd_##SFX((float)s[2]), q2 = rnd_##SFX((float)s[3]);                  \
+        PAR_FOR(n)                                                                             \
+        for (size_t i = 0; i < n; ++i) {                                                       \
+            const float d = FROM16(dupdates[i]), u = FROM16(updates[i]);                       \
+            const float m1 = FROM16(new_mu[i]);                                                \
+            if (m1 == 0) {                                                                     \
+                dnew_mu_out[i] = 0;                                                            \
+                dnew_nu_out[i] = 0;                                                            \
+                continue;                                                                      \
+            }                                                                                  \
+            const float r = rnd_##SFX(u / m1);                                                 \
+            const float den = rnd_##SFX(r * p1);                                               \
+            dnew_mu_out[i] = TO16(d * r);                                                      \
+            const float head = rnd_##SFX(rnd_##SFX(-d * u) * den);                             \
+            const double tail = (double)head * 0.5 * (double)q2 * (double)den;                 \
+            dnew_nu_out[i] = TO16((float)tail);                                                \
+        }                                                                                      \
+    }
+
+ORACLE_DEFINE_LOWP(f16, f16_from_f32, f32_from_f16)
+ORACLE_DEFINE_LOWP(bf16, bf16_from_f32, f32_from_bf16)
+
+/* conversions, exported so tests can pin them against NumPy's float16 and torch's bfloat16 */
+uint16_t oracle_f16_from_f32(float f) { return f16_from_f32(f); }
+float oracle_f32_from_f16(uint16_t h) { return f32_from_f16(h); }
+uint16_t oracle_bf16_from_f32(float f) { return bf16_from_f32(f); }
+float oracle_f32_from_bf16(uint16_t b) { return f32_from_bf16(b); }

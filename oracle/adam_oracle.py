@@ -23,8 +23,10 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, 'liboracle_adam.so')
 
-_SFX = {np.dtype(np.float32): 'f32', np.dtype(np.float64): 'f64'}
-_CT = {np.dtype(np.float32): ctypes.c_float, np.dtype(np.float64): ctypes.c_double}
+# float16 arrays are NumPy's own; bfloat16 has no NumPy dtype, so bfloat16 data travels as uint16
+# bit patterns (a uint16 array always means bfloat16 here).
+_SFX = {np.dtype(np.float32): 'f32', np.dtype(np.float64): 'f64', np.dtype(np.float16): 'f16',
+        np.dtype(np.uint16): 'bf16'}
 
 _lib = None
 
@@ -46,6 +48,12 @@ def lib() -> ctypes.CDLL:
         _lib = ctypes.CDLL(_LIB_PATH)
         _lib.oracle_adam_threads_for.restype = ctypes.c_int
         _lib.oracle_adam_threads_for.argtypes = [ctypes.c_size_t]
+        for name in ('oracle_f16_from_f32', 'oracle_bf16_from_f32'):
+            getattr(_lib, name).restype = ctypes.c_uint16
+            getattr(_lib, name).argtypes = [ctypes.c_float]
+        for name in ('oracle_f32_from_f16', 'oracle_f32_from_bf16'):
+            getattr(_lib, name).restype = ctypes.c_float
+            getattr(_lib, name).argtypes = [ctypes.c_uint16]
     return _lib
 
 
@@ -61,6 +69,21 @@ def _fn(name: str, dtype):
 _D = ctypes.c_double
 _U64 = ctypes.c_uint64
 _SZ = ctypes.c_size_t
+
+
+def bf16_bits(a) -> np.ndarray:
+    """float32 array -> bfloat16 bit patterns (uint16), round to nearest even, NaN -> 0x7fc0:
+    the conversion c10::BFloat16 performs."""
+    x = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+    out = ((x + np.uint32(0x7fff) + ((x >> np.uint32(16)) & np.uint32(1))) >> np.uint32(16))
+    out = out.astype(np.uint16)
+    out[np.isnan(np.asarray(a, dtype=np.float32))] = 0x7fc0
+    return out
+
+
+def bf16_to_f32(bits) -> np.ndarray:
+    return (np.ascontiguousarray(bits, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(
+        np.float32)
 
 
 def host_scalars(b1, b2, eps_root, count):

@@ -11,6 +11,14 @@ disagreement means one of the two mis-states an evaluation order, a promotion
 or a rounding point.
 
 All functions are out-of-place and return new arrays.
+
+float16 arrays are covered too: NumPy's float16 arithmetic converts to float32, operates and
+rounds back, which is what c10::Half does for an operation between two halves.  Where the
+reference's expression mixes a half with a float (the square root is the float overload, so
+"sqrt(.) + eps" and the division stay in float) or a double (the tail of backward_updates),
+the spec widens explicitly, and every scalar goes double -> float -> half as `Half(float(x))`
+does.  bfloat16 has no NumPy type and is pinned by the compiled reference and the golden
+vectors only.
 """
 
 from __future__ import annotations
@@ -28,7 +36,15 @@ def host_scalars(b1: float, b2: float, eps_root: float, count: int):
 
 
 def _t(dtype, x):
+    """Python scalar -> element type; a half is reached through float, as c10::Half(float)."""
+    if np.dtype(dtype) == np.float16:
+        return np.float16(np.float32(x))
     return np.dtype(dtype).type(x)
+
+
+def _wide(dtype):
+    """The type in which an expression mixing the element type with a float runs."""
+    return np.float32 if np.dtype(dtype) == np.float16 else np.dtype(dtype).type
 
 
 def forward_mu(updates: np.ndarray, mu: np.ndarray, b1: float) -> np.ndarray:
@@ -56,11 +72,12 @@ def forward_updates(new_mu, new_nu, b1, b2, eps, eps_root, count) -> np.ndarray:
     T = new_mu.dtype
     c1d, c2d, _, _ = host_scalars(b1, b2, eps_root, count)
     c1, c2 = _t(T, c1d), _t(T, c2d)
+    W = _wide(T)
     mu_hat = new_mu * c1
     nu_hat = new_nu * c2
     with np.errstate(all='ignore'):
-        root = np.sqrt(nu_hat + _t(T, eps_root))
-        return mu_hat / (root + _t(T, eps))
+        root = np.sqrt((nu_hat + _t(T, eps_root)).astype(W))  # the sum is rounded to T first
+        return (mu_hat.astype(W) / (root + W(_t(T, eps)))).astype(T)
 
 
 def forward_inplace(updates, mu, nu, b1, b2, eps, eps_root, count):
@@ -98,7 +115,7 @@ def backward_updates(dupdates, updates, new_mu, b1, b2, eps_root, count):
         head = ((-dupdates) * updates) * den  # two roundings in T
         # the literal 0.5 is a double: the remaining products run in float64
         tail = ((head.astype(np.float64) * 0.5) * np.float64(q2)) * den.astype(np.float64)
-        dnew_nu = tail.astype(T)
+        dnew_nu = tail.astype(_wide(T)).astype(T)  # a half is reached through float
     zero = new_mu == 0  # true for +0 and -0, false for NaN
     dnew_mu = np.where(zero, _t(T, 0), dnew_mu)
     dnew_nu = np.where(zero, _t(T, 0), dnew_nu)

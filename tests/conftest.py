@@ -43,9 +43,14 @@ def hyper_of(case):
 
 def bits(a: np.ndarray) -> np.ndarray:
     """Bit patterns, with every NaN collapsed to one pattern (NaN payloads and signs are not
-    part of the contract: x86 and the GPU propagate different ones)."""
+    part of the contract: x86 and the GPU propagate different ones).  uint16 arrays are
+    bfloat16 bit patterns."""
     a = np.ascontiguousarray(a)
-    u = a.view(np.uint32 if a.dtype == np.float32 else np.uint64).copy()
+    if a.dtype == np.uint16:  # bfloat16: NaN = exponent all ones, mantissa non-zero
+        u = a.copy()
+        u[(a & 0x7fff) > 0x7f80] = 0xffff
+        return u
+    u = a.view({2: np.uint16, 4: np.uint32, 8: np.uint64}[a.dtype.itemsize]).copy()
     u[np.isnan(a)] = np.iinfo(u.dtype).max
     return u
 

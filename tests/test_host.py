@@ -61,6 +61,9 @@ def test_abi_version_and_error_strings():
         assert b'toa_adam' in lib.toa_adam_error_string(code)
     with pytest.raises(RuntimeError, match='unsupported dtype'):
         _lib.check(-1, 'x')
+    # the fused optimizer step serves float32 / float64 only
+    assert lib.toa_adam_fused_step(_lib.TOA_F16, None, None, None, None, 0, 0.9, 0.999, 1e-8, 0.0, 1,
+                                   1e-3, 0, 0, None) == -1
 
 
 def test_argument_errors_need_no_device():
@@ -73,7 +76,7 @@ def test_argument_errors_need_no_device():
                                          None) == 0
     assert lib.toa_adam_forward_inplace_multi(0, 0, None, None, None, None, 0.9, 0.999, 1e-8, 0.0,
                                               None, 1, None) == 0
-    assert lib.toa_adam_forward_inplace_multi(3, 2, None, None, None, None, 0.9, 0.999, 1e-8, 0.0,
+    assert lib.toa_adam_forward_inplace_multi(9, 2, None, None, None, None, 0.9, 0.999, 1e-8, 0.0,
                                               None, 1, None) == -1
     assert lib.toa_adam_forward_inplace_multi(0, 2, None, None, None, None, 0.9, 0.999, 1e-8, 0.0,
                                               None, 1, None) == -2

@@ -1,0 +1,162 @@
+"""float16 and bfloat16 tensors through the GPU op against the CPU oracle and the golden vectors
+of the reference CPU op (which serves at::Half / at::BFloat16 with per-operation rounding,
+/root/reference/include/common.h:26-31).  Bit for bit."""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import assert_bit_equal, hyper_of, load_golden
+from oracle import adam_oracle as O
+from torchopt_amd import AdamOp
+from torchopt_amd._C import adam_op
+
+pytestmark = pytest.mark.gpu
+
+TORCH = {'f16': torch.float16, 'bf16': torch.bfloat16}
+
+
+@pytest.fixture(scope='module', autouse=True)
+def _gpu():
+    assert torch.cuda.is_available(), 'these tests need a GPU; there is no fallback path'
+    yield
+    torch.cuda.synchronize()
+
+
+def dev(a, tag):
+    """NumPy float16 array, or uint16 bfloat16 bit patterns, to a GPU tensor of that type."""
+    a = np.ascontiguousarray(a)
+    if tag == 'bf16':
+        return torch.from_numpy(a.view(np.int16)).cuda().view(torch.bfloat16)
+    return torch.from_numpy(a).cuda()
+
+
+def host(t, tag):
+    if tag == 'bf16':
+        return t.detach().contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+    return t.detach().cpu().numpy()
+
+
+def draw(tag, n, seed):
+    rng = np.random.default_rng(seed)
+
+    def fmt(x):
+        return O.bf16_bits(x.astype(np.float32)) if tag == 'bf16' else x.astype(np.float16)
+
+    return {'updates': fmt(rng.standard_normal(n)), 'mu': fmt(0.1 * rng.standard_normal(n)),
+            'nu': fmt(np.abs(0.01 * rng.standard_normal(n))), 'dmu': fmt(rng.standard_normal(n)),
+            'dnu': fmt(rng.standard_normal(n)), 'dupdates': fmt(rng.standard_normal(n))}
+
+
+def check_all_seven(tag, inp, hyper, label, exp=None):
+    b1, b2, eps, er, c = hyper
+    u, m, v = inp['updates'], inp['mu'], inp['nu']
+    if exp is None:
+        ou, om, ov = O.forward_inplace(u.copy(), m.copy(), v.copy(), b1, b2, eps, er, c)
+        exp = {'new_mu': O.forward_mu(u, m, b1), 'new_nu': O.forward_nu(u, v, b2),
+               'inplace_updates': ou, 'inplace_mu': om, 'inplace_nu': ov}
+        exp['new_updates'] = O.forward_updates(exp['new_mu'], exp['new_nu'], b1, b2, eps, er, c)
+        exp['bmu_dupdates'], exp['bmu_dmu'] = O.backward_mu(inp['dmu'], b1)
+        exp['bnu_dupdates'], exp['bnu_dnu'] = O.backward_nu(inp['dnu'], u, b2)
+        exp['bup_dnew_mu'], exp['bup_dnew_nu'] = O.backward_updates(
+            inp['dupdates'], exp['new_updates'], exp['new_mu'], b1, b2, er, c)
+    g = {k: dev(a, tag) for k, a in inp.items()}
+
+    def same(t, key):
+        assert_bit_equal(host(t, tag), exp[key], f'{label} {key}')
+
+    same(adam_op.forward_mu(g['updates'], g['mu'], b1), 'new_mu')
+    same(adam_op.forward_nu(g['updates'], g['nu'], b2), 'new_nu')
+    emu, env = dev(exp['new_mu'], tag), dev(exp['new_nu'], tag)
+    same(adam_op.forward_updates(emu, env, b1, b2, eps, er, c), 'new_updates')
+    iu, im, iv = g['updates'].clone(), g['mu'].clone(), g['nu'].clone()
+    adam_op.forward_(iu, im, iv, b1, b2, eps, er, c)
+    same(iu, 'inplace_updates'), same(im, 'inplace_mu'), same(iv, 'inplace_nu')
+    du, dm = adam_op.backward_mu(g['dmu'], g['updates'], g['mu'], b1)
+    same(du, 'bmu_dupdates'), same(dm, 'bmu_dmu')
+    du, dn = adam_op.backward_nu(g['dnu'], g['updates'], g['nu'], b2)
+    same(du, 'bnu_dupdates'), same(dn, 'bnu_dnu')
+    dm, dn = adam_op.backward_updates(g['dupdates'], dev(exp['new_updates'], tag), emu, env, b1,
+                                      b2, er, c)
+    same(dm, 'bup_dnew_mu'), same(dn, 'bup_dnew_nu')
+
+
+@pytest.mark.parametrize('tag', ['f16', 'bf16'])
+def test_golden_vectors(tag):
+    for name, case in sorted(load_golden(tag).items()):
+        inp = {k: case[k] for k in ('updates', 'mu', 'nu', 'dmu', 'dnu', 'dupdates')}
+        check_all_seven(tag, inp, hyper_of(case), f'{tag}/{name}', exp=case)
+
+
+@pytest.mark.parametrize('tag', ['f16', 'bf16'])
+def test_sizes_against_oracle(tag):
+    """Eight elements per 128-bit access, 512 per tile: sizes around those boundaries."""
+    hypers = [(0.9, 0.999, 1e-3, 0.0, 10), (0.9, 0.999, 1e-3, 1e-4, 5), (0.8, 0.95, 1e-2, 1e-3, 77)]
+    for k, n in enumerate([1, 7, 8, 9, 511, 512, 513, 4095, 4097, 65537, (1 << 20) + 5]):
+        check_all_seven(tag, draw(tag, n, 700 + n), hypers[k % 3], f'{tag}/n={n}')
+
+
+@pytest.mark.parametrize('tag', ['f16', 'bf16'])
+def test_misaligned_views(tag):
+    n = 30_001
+    inp = draw(tag, n + 8, 5)
+    for off in (1, 3, 4, 7):
+        cut = {k: a[off:off + n].copy() for k, a in inp.items()}
+        e = O.forward_inplace(cut['updates'], cut['mu'], cut['nu'], 0.9, 0.999, 1e-3, 0.0, 4)
+        full = {k: dev(inp[k], tag) for k in ('updates', 'mu', 'nu')}
+        views = [full[k][off:off + n] for k in ('updates', 'mu', 'nu')]
+        adam_op.forward_(*views, 0.9, 0.999, 1e-3, 0.0, 4)
+        for t, want, k in zip(views, e, ('updates', 'mu', 'nu')):
+            assert_bit_equal(host(t, tag), want, f'offset {off} {k}')
+            h = host(full[k], tag)
+            assert_bit_equal(h[:off], inp[k][:off], 'head guard')
+            assert_bit_equal(h[off + n:], inp[k][off + n:], 'tail guard')
+
+
+@pytest.mark.parametrize('tag', ['f16', 'bf16'])
+def test_multi_tensor_and_autograd(tag):
+    sizes = [864, 9216, 32, 4000, 5, 0, 70_001]
+    hs = [draw(tag, n, 40 + k) for k, n in enumerate(sizes)]
+    us, ms, vs = ([dev(h[key], tag) for h in hs] for key in ('updates', 'mu', 'nu'))
+    adam_op.forward_multi_(us, ms, vs, 0.9, 0.999, 1e-3, 1e-4, 3)
+    for k, h in enumerate(hs):
+        eu, em, ev = O.forward_inplace(h['updates'].copy(), h['mu'].copy(), h['nu'].copy(), 0.9,
+                                       0.999, 1e-3, 1e-4, 3)
+        assert_bit_equal(host(us[k], tag), eu, f'multi updates[{k}]')
+        assert_bit_equal(host(vs[k], tag), ev, f'multi nu[{k}]')
+    # differentiable chain on one leaf
+    h = hs[1]
+    g, m, v = (dev(h[key], tag).requires_grad_(True) for key in ('updates', 'mu', 'nu'))
+    new_mu, new_nu, new_u = AdamOp(0.9, 0.999, 1e-3, eps_root=1e-4, inplace=False)(m, v, g, 2)
+    new_u.backward(dev(h['dupdates'], tag))
+    e_mu, e_nu = O.forward_mu(h['updates'], h['mu'], 0.9), O.forward_nu(h['updates'], h['nu'], 0.999)
+    e_u = O.forward_updates(e_mu, e_nu, 0.9, 0.999, 1e-3, 1e-4, 2)
+    assert_bit_equal(host(new_u, tag), e_u, 'forward chain')
+    bm, bv = O.backward_updates(h['dupdates'], e_u, e_mu, 0.9, 0.999, 1e-4, 2)
+    _, gm = O.backward_mu(bm, 0.9)
+    _, gv = O.backward_nu(bv, h['updates'], 0.999)
+    assert_bit_equal(host(m.grad, tag), gm, 'd mu')
+    assert_bit_equal(host(v.grad, tag), gv, 'd nu')
+
+
+def test_throughput_is_reported_not_assumed(capsys):
+    """Not an assertion on speed: prints the in-place step's rate for 2^27 16-bit elements so the
+    log of a GPU run shows where the 16-bit types stand (12 bytes per element)."""
+    n = 1 << 27
+    for tag, dt in TORCH.items():
+        u = torch.randn(n, device='cuda').to(dt)
+        m = (0.1 * torch.randn(n, device='cuda')).to(dt)
+        v = (0.01 * torch.randn(n, device='cuda')).abs().to(dt)
+        for _ in range(3):
+            adam_op.forward_(u, m, v, 0.9, 0.999, 1e-3, 0.0, 10)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            adam_op.forward_(u, m, v, 0.9, 0.999, 1e-3, 0.0, 10)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / 10
+        with capsys.disabled():
+            print(f'\n[{tag}] forward_ 2^27 elements: {ms:.4f} ms, {12 * n / ms / 1e6:.0f} GB/s')

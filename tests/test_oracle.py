@@ -22,7 +22,7 @@ from oracle import adam_oracle as O
 from oracle import adam_spec as S
 
 DTYPES = [np.float32, np.float64]
-TAG = {np.float32: 'f32', np.float64: 'f64'}
+TAG = {np.float32: 'f32', np.float64: 'f64', np.float16: 'f16', 'bf16': 'bf16'}
 
 
 def _cases(dtype):
@@ -33,13 +33,16 @@ def _ids(dtype):
     return [f'{TAG[dtype]}-{name}' for name, _ in _cases(dtype)]
 
 
-ALL_CASES = [(dt, name, case) for dt in DTYPES for name, case in _cases(dt)]
+GOLDEN_DTYPES = [np.float32, np.float64, np.float16, 'bf16']
+ALL_CASES = [(dt, name, case) for dt in GOLDEN_DTYPES for name, case in _cases(dt)]
 ALL_IDS = [f'{TAG[dt]}-{name}' for dt, name, _ in ALL_CASES]
 
 
 @pytest.mark.parametrize('dtype,name,case', ALL_CASES, ids=ALL_IDS)
 @pytest.mark.parametrize('impl', [O, S], ids=['c_oracle', 'numpy_spec'])
 def test_against_reference_golden(impl, dtype, name, case):
+    if impl is S and dtype == 'bf16':
+        pytest.skip('NumPy has no bfloat16; the spec covers float16, float32, float64')
     b1, b2, eps, eps_root, count = hyper_of(case)
     u, mu, nu = case['updates'], case['mu'], case['nu']
     with np.errstate(all='ignore'):
@@ -65,7 +68,7 @@ def test_against_reference_golden(impl, dtype, name, case):
         assert_bit_equal(dn, case['bup_dnew_nu'], 'backward_updates dnew_nu')
 
 
-@pytest.mark.parametrize('dtype', DTYPES, ids=['f32', 'f64'])
+@pytest.mark.parametrize('dtype', GOLDEN_DTYPES, ids=['f32', 'f64', 'f16', 'bf16'])
 def test_golden_internal_consistency(dtype):
     """In the reference's own outputs the fused step equals the three split ops chained."""
     for name, case in _cases(dtype):
@@ -189,6 +192,97 @@ def test_fused_step_scales_by_the_rounded_learning_rate():
                           0.0, 0.0, 1)[0]
     assert_bit_equal(g, u * np.float32(-0.1))
     assert_bit_equal(p, np.float32(0) + u * np.float32(-0.1))
+
+
+def test_half_conversions_against_numpy_and_torch():
+    """The oracle's own float<->half and float->bfloat16 conversions: every half value, every
+    midpoint between neighbouring halves (ties to even), the overflow threshold, subnormals."""
+    import torch
+
+    L = O.lib()
+    halves = np.arange(65536, dtype=np.uint16)
+    as_f32 = halves.view(np.float16).astype(np.float32)
+    back = np.array([L.oracle_f32_from_f16(int(h)) for h in halves], dtype=np.float32)
+    assert_bit_equal(back, as_f32, 'half -> float, all 65536 values')
+    fin = np.isfinite(as_f32[:-1]) & np.isfinite(as_f32[1:])
+    mids = ((as_f32[:-1].astype(np.float64) + as_f32[1:].astype(np.float64)) / 2)[fin]
+    rng = np.random.default_rng(0)
+    xs = np.concatenate([
+        mids.astype(np.float32),
+        np.array([65504, 65519.996, 65520, 65536, 1e30, -65520, 2.0 ** -24, 2.0 ** -25,
+                  2.0 ** -25 * 1.0001, 0.0, -0.0, np.inf, -np.inf], dtype=np.float32),
+        (rng.standard_normal(20000) * 1e-6).astype(np.float32),
+        rng.standard_normal(20000).astype(np.float32),
+        rng.integers(0, 2 ** 32, 20000, dtype=np.uint64).astype(np.uint32).view(np.float32)])
+    xs = xs[~np.isnan(xs)]
+    with np.errstate(all='ignore'):
+        want = xs.astype(np.float16).view(np.uint16)
+    got = np.array([L.oracle_f16_from_f32(float(x)) for x in xs], dtype=np.uint16)
+    assert np.array_equal(got, want)
+    want = torch.from_numpy(xs).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    got = np.array([L.oracle_bf16_from_f32(float(x)) for x in xs], dtype=np.uint16)
+    assert np.array_equal(got, want) and np.array_equal(O.bf16_bits(xs), want)
+    assert L.oracle_bf16_from_f32(float('nan')) == 0x7fc0
+    assert L.oracle_f16_from_f32(float('nan')) & 0x7fff == 0x7e00
+
+
+def test_half_division_stays_in_float_until_the_end():
+    """mu_hat / (sqrt(.) + eps) with half data: the square root, the sum and the quotient run in
+    float and are rounded once.  Rounding the root or the denominator to half first changes
+    thousands of results on random data, so the distinction is observable."""
+    rng = np.random.default_rng(4)
+    n = 20000
+    m = (0.1 * rng.standard_normal(n)).astype(np.float16)
+    v = np.abs(0.01 * rng.standard_normal(n)).astype(np.float16)
+    got = O.forward_updates(m, v, 0.9, 0.999, 1e-3, 1e-4, 5)
+    f, h = np.float32, np.float16
+    c1, c2 = h(f(1 / (1 - 0.9 ** 5))), h(f(1 / (1 - 0.999 ** 5)))
+    mh, vh = m * c1, v * c2
+    t = vh + h(f(1e-4))
+    kept = (mh.astype(f) / (np.sqrt(t.astype(f)) + f(h(f(1e-3))))).astype(h)
+    rounded = mh / (np.sqrt(t) + h(f(1e-3)))
+    assert_bit_equal(got, kept)
+    assert (kept != rounded).sum() > 100
+
+
+@pytest.mark.parametrize('fmt', ['f16', 'bf16'])
+def test_low_precision_oracle_equals_compiled_reference(fmt):
+    ref = O.load_reference()
+    if ref is None:
+        pytest.skip('oracle/_ref not built (needs the reference sources; `make -C oracle ref`)')
+    import torch
+
+    tdt = torch.float16 if fmt == 'f16' else torch.bfloat16
+    rng = np.random.default_rng(8)
+    n = 200_003
+
+    def tens(a):
+        return torch.from_numpy(np.asarray(a, dtype=np.float32)).to(tdt)
+
+    def arr(t):
+        if fmt == 'bf16':
+            return t.contiguous().view(torch.int16).numpy().view(np.uint16).copy()
+        return t.numpy().copy()
+
+    g, m = tens(rng.standard_normal(n)), tens(0.1 * rng.standard_normal(n))
+    v = tens(np.abs(0.01 * rng.standard_normal(n)))
+    d1, d2, d3 = (tens(rng.standard_normal(n)) for _ in range(3))
+    op = ref.adam_op
+    for b1, b2, eps, er, count in [(0.9, 0.999, 1e-3, 0.0, 10), (0.9, 0.999, 1e-3, 1e-4, 3)]:
+        tg, tm, tv = g.clone(), m.clone(), v.clone()
+        op.forward_(tg, tm, tv, b1, b2, eps, er, count)
+        og, om, ov = arr(g), arr(m), arr(v)
+        O.forward_inplace(og, om, ov, b1, b2, eps, er, count)
+        assert_bit_equal(og, arr(tg)), assert_bit_equal(om, arr(tm)), assert_bit_equal(ov, arr(tv))
+        for a, b in zip(O.backward_mu(arr(d1), b1), op.backward_mu(d1, g, m, b1)):
+            assert_bit_equal(a, arr(b))
+        for a, b in zip(O.backward_nu(arr(d2), arr(g), b2), op.backward_nu(d2, g, v, b2)):
+            assert_bit_equal(a, arr(b))
+        tm0 = tm.clone()
+        tm0[::9] = 0
+        for a, b in zip(O.backward_updates(arr(d3), arr(tg), arr(tm0), b1, b2, er, count),
+                        op.backward_updates(d3, tg, tm0, tv, b1, b2, er, count)):
+            assert_bit_equal(a, arr(b))
 
 
 # ---------------------------------------------------------------------------------------------

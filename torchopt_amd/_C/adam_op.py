@@ -53,7 +53,8 @@ __all__ = [
     'fused_step_multi_',
 ]
 
-_DTYPES = {torch.float32: _lib.TOA_F32, torch.float64: _lib.TOA_F64}
+_DTYPES = {torch.float32: _lib.TOA_F32, torch.float64: _lib.TOA_F64,
+           torch.float16: _lib.TOA_F16, torch.bfloat16: _lib.TOA_BF16}
 
 
 # --------------------------------------------------------------------------- helpers

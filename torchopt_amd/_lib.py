@@ -16,6 +16,8 @@ LIB_PATH = os.path.join(PKG_DIR, 'libtoa_adam.so')
 
 TOA_F32 = 0
 TOA_F64 = 1
+TOA_F16 = 2
+TOA_BF16 = 3
 ABI_VERSION = 1
 
 _vp = ctypes.c_void_p

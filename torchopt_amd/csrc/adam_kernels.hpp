@@ -34,17 +34,136 @@ namespace toa {
 
 constexpr int kBlock = 64;  // one wavefront per workgroup
 
+// ---------------------------------------------------------------------------
+// 16-bit element types with the arithmetic of c10::Half / c10::BFloat16, which
+// is what the reference CPU op computes in when it is handed such tensors
+// (/root/reference/include/common.h:26-31): an operation between two 16-bit
+// values (or an int, which converts first) runs in float and is rounded back to
+// 16 bits; an operation with a float (double) operand yields an unrounded float
+// (double); a double reaches 16 bits through float.
+// ---------------------------------------------------------------------------
+struct HalfFormat {  // IEEE binary16
+    static __host__ __device__ inline uint16_t encode(float f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+        return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));  // v_cvt_f16_f32, RNE
+#else
+        uint32_t x = __builtin_bit_cast(uint32_t, f);
+        const uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+        x &= 0x7fffffffu;
+        if (x > 0x7f800000u) return sign | 0x7e00u;
+        if (x >= 0x477ff000u) return sign | 0x7c00u;
+        if (x < 0x38800000u) {  // subnormal: count units of 2^-24, ties to even
+            const float units = __builtin_bit_cast(float, x) * 16777216.0f;
+            uint32_t q = (uint32_t)units;
+            const float frac = units - (float)q;
+            if (frac > 0.5f || (frac == 0.5f && (q & 1u))) ++q;
+            return sign | (uint16_t)q;
+        }
+        uint32_t h = (((x >> 23) - 112u) << 10) | ((x & 0x7fffffu) >> 13);
+        const uint32_t rest = x & 0x1fffu;
+        if (rest > 0x1000u || (rest == 0x1000u && (h & 1u))) ++h;
+        return sign | (uint16_t)h;
+#endif
+    }
+    static __host__ __device__ inline float decode(uint16_t h) {
+#if defined(__HIP_DEVICE_COMPILE__)
+        return static_cast<float>(__builtin_bit_cast(_Float16, h));
+#else
+        const uint32_t sign = ((uint32_t)h & 0x8000u) << 16, e = (h >> 10) & 0x1fu, m = h & 0x3ffu;
+        if (e == 0) return __builtin_bit_cast(float, sign) + (sign ? -1.0f : 1.0f) * (float)m * 5.9604644775390625e-8f;
+        if (e == 31) return __builtin_bit_cast(float, sign | 0x7f800000u | (m << 13));
+        return __builtin_bit_cast(float, sign | ((e + 112u) << 23) | (m << 13));
+#endif
+    }
+};
+
+struct BFloatFormat {  // upper half of a binary32, round to nearest even
+    static __host__ __device__ inline uint16_t encode(float f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+        // v_cvt_pk_bf16_f32: same rounding; a NaN stays a (quiet) NaN with its own payload
+        return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
+#else
+        const uint32_t x = __builtin_bit_cast(uint32_t, f);
+        if ((x & 0x7fffffffu) > 0x7f800000u) return 0x7fc0u;
+        return (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);
+#endif
+    }
+    static __host__ __device__ inline float decode(uint16_t b) {
+        return __builtin_bit_cast(float, (uint32_t)b << 16);
+    }
+};
+
+template <class F>
+struct R16 {
+    uint16_t bits;
+    R16() = default;
+    __host__ __device__ R16(float f) : bits(F::encode(f)) {}
+    __host__ __device__ explicit R16(double d) : bits(F::encode((float)d)) {}
+    __host__ __device__ R16(int i) : bits(F::encode((float)i)) {}
+    __host__ __device__ static R16 from_bits(uint16_t b) {
+        R16 r;
+        r.bits = b;
+        return r;
+    }
+    __host__ __device__ operator float() const { return F::decode(bits); }
+};
+#define TOA_R16_BINOP(OP)                                                                        \
+    template <class F>                                                                           \
+    __host__ __device__ inline R16<F> operator OP(R16<F> a, R16<F> b) {                          \
+        return R16<F>((float)a OP(float) b);                                                     \
+    }                                                                                            \
+    template <class F>                                                                           \
+    __host__ __device__ inline R16<F> operator OP(int a, R16<F> b) {                             \
+        return R16<F>(a) OP b;                                                                   \
+    }                                                                                            \
+    template <class F>                                                                           \
+    __host__ __device__ inline float operator OP(R16<F> a, float b) { return (float)a OP b; }    \
+    template <class F>                                                                           \
+    __host__ __device__ inline float operator OP(float a, R16<F> b) { return a OP(float) b; }    \
+    template <class F>                                                                           \
+    __host__ __device__ inline double operator OP(R16<F> a, double b) {                          \
+        return (double)(float)a OP b;                                                            \
+    }                                                                                            \
+    template <class F>                                                                           \
+    __host__ __device__ inline double operator OP(double a, R16<F> b) {                          \
+        return a OP(double)(float) b;                                                            \
+    }
+TOA_R16_BINOP(+)
+TOA_R16_BINOP(-)
+TOA_R16_BINOP(*)
+TOA_R16_BINOP(/)
+#undef TOA_R16_BINOP
+template <class F>
+__host__ __device__ inline R16<F> operator-(R16<F> a) { return R16<F>(-(float)a); }
+template <class F>
+__host__ __device__ inline bool operator==(R16<F> a, int b) { return (float)a == (float)b; }
+
+using half_t = R16<HalfFormat>;
+using bfloat_t = R16<BFloatFormat>;
+
+// 128-bit access types and element accessors.
 template <typename T>
 struct Vec;
 template <>
 struct Vec<float> {
     typedef float type __attribute__((ext_vector_type(4)));
     static constexpr int N = 4;
+    __device__ static float get(const type &v, int e) { return v[e]; }
+    __device__ static void set(type &v, int e, float x) { v[e] = x; }
 };
 template <>
 struct Vec<double> {
     typedef double type __attribute__((ext_vector_type(2)));
     static constexpr int N = 2;
+    __device__ static double get(const type &v, int e) { return v[e]; }
+    __device__ static void set(type &v, int e, double x) { v[e] = x; }
+};
+template <class F>
+struct Vec<R16<F>> {
+    typedef uint16_t type __attribute__((ext_vector_type(8)));
+    static constexpr int N = 8;
+    __device__ static R16<F> get(const type &v, int e) { return R16<F>::from_bits(v[e]); }
+    __device__ static void set(type &v, int e, R16<F> x) { v[e] = x.bits; }
 };
 
 template <bool NT, typename V>
@@ -62,6 +181,9 @@ __device__ __forceinline__ void st(V *p, V v) {
 
 __device__ __forceinline__ float toa_sqrt(float x) { return sqrtf(x); }
 __device__ __forceinline__ double toa_sqrt(double x) { return sqrt(x); }
+// a 16-bit value picks the float overload; the root is NOT rounded back
+template <class F>
+__device__ __forceinline__ float toa_sqrt(R16<F> x) { return sqrtf((float)x); }
 
 // ---------------------------------------------------------------------------
 // Element-wise ops.  Pointer slots: inputs first, then outputs; an in-place op
@@ -73,7 +195,9 @@ __device__ __forceinline__ double toa_sqrt(double x) { return sqrt(x); }
 template <typename T>
 struct ForwardInplace {
     static constexpr int NIN = 3, NOUT = 3, NPTR = 3;
-    static constexpr int kWavesPerCU = 13;  // read-modify-write: a tight window wins
+    // read-modify-write: a tight window wins; the 16-bit types spend twice the ALU time per
+    // byte on conversions and want more waves to hide it
+    static constexpr int kWavesPerCU = sizeof(T) == 2 ? 22 : 13;
     // outputs are produced as (mu', nu', updates') and stored in that order
     __device__ static constexpr int out_slot(int j) { return j == 0 ? 1 : (j == 1 ? 2 : 0); }
     T b1, b2, c1, c2, eps, eps_root;
@@ -245,10 +369,10 @@ __device__ __forceinline__ void tile_full(const Op &op, const TensorPtrs<T, Op> 
         for (int e = 0; e < VN; ++e) {
             T a[Op::NIN], r[Op::NOUT];
 #pragma unroll
-            for (int i = 0; i < Op::NIN; ++i) a[i] = in[i][k][e];
+            for (int i = 0; i < Op::NIN; ++i) a[i] = Vec<T>::get(in[i][k], e);
             op(a, r);
 #pragma unroll
-            for (int j = 0; j < Op::NOUT; ++j) out[j][k][e] = r[j];
+            for (int j = 0; j < Op::NOUT; ++j) Vec<T>::set(out[j][k], e, r[j]);
         }
 
 #pragma unroll
@@ -276,10 +400,10 @@ __device__ __forceinline__ void tile_partial(const Op &op, const TensorPtrs<T, O
         for (int e = 0; e < VN; ++e) {
             T a[Op::NIN], r[Op::NOUT];
 #pragma unroll
-            for (int i = 0; i < Op::NIN; ++i) a[i] = in[i][e];
+            for (int i = 0; i < Op::NIN; ++i) a[i] = Vec<T>::get(in[i], e);
             op(a, r);
 #pragma unroll
-            for (int j = 0; j < Op::NOUT; ++j) out[j][e] = r[j];
+            for (int j = 0; j < Op::NOUT; ++j) Vec<T>::set(out[j], e, r[j]);
         }
 #pragma unroll
         for (int j = 0; j < Op::NOUT; ++j)

@@ -171,6 +171,7 @@ T *mut(const void *p) {
     return static_cast<T *>(const_cast<void *>(p));
 }
 
+// float32 and float64 only (the fused optimizer step)
 #define TOA_DISPATCH(dtype, ...)                  \
     switch (dtype) {                              \
         case TOA_F32: {                           \
@@ -179,6 +180,29 @@ T *mut(const void *p) {
         }                                         \
         case TOA_F64: {                           \
             using T = double;                     \
+            return __VA_ARGS__();                 \
+        }                                         \
+        default:                                  \
+            return TOA_EDTYPE;                    \
+    }
+
+// every element type the reference CPU op serves
+#define TOA_DISPATCH_ALL(dtype, ...)              \
+    switch (dtype) {                              \
+        case TOA_F32: {                           \
+            using T = float;                      \
+            return __VA_ARGS__();                 \
+        }                                         \
+        case TOA_F64: {                           \
+            using T = double;                     \
+            return __VA_ARGS__();                 \
+        }                                         \
+        case TOA_F16: {                           \
+            using T = half_t;                     \
+            return __VA_ARGS__();                 \
+        }                                         \
+        case TOA_BF16: {                          \
+            using T = bfloat_t;                   \
             return __VA_ARGS__();                 \
         }                                         \
         default:                                  \
@@ -200,7 +224,7 @@ int toa_adam_set_waves_per_cu(int waves) {
 const char *toa_adam_error_string(int code) {
     switch (code) {
         case 0: return "success";
-        case TOA_EDTYPE: return "toa_adam: unsupported dtype (expected TOA_F32 or TOA_F64)";
+        case TOA_EDTYPE: return "toa_adam: unsupported dtype for this entry point";
         case TOA_ENULL: return "toa_adam: null pointer for a non-empty tensor";
         case TOA_ESIZE: return "toa_adam: tensor too large for one launch";
         default: return code > 0 ? hipGetErrorString((hipError_t)code) : "toa_adam: unknown error";
@@ -211,7 +235,7 @@ int toa_adam_forward_inplace(int dtype, void *updates, void *mu, void *nu, size_
                              double b2, double eps, double eps_root, uint64_t count,
                              void *stream) {
     const HostScalars s = host_scalars(b1, b2, eps_root, count);
-    TOA_DISPATCH(dtype, [&] {
+    TOA_DISPATCH_ALL(dtype, [&] {
         const ForwardInplace<T> op{(T)b1, (T)b2, (T)s.c1, (T)s.c2, (T)eps, (T)eps_root};
         T *const p[3] = {(T *)updates, (T *)mu, (T *)nu};
         return launch_single<T>(op, p, n, stream);
@@ -220,7 +244,7 @@ int toa_adam_forward_inplace(int dtype, void *updates, void *mu, void *nu, size_
 
 int toa_adam_forward_mu(int dtype, const void *updates, const void *mu, size_t n, double b1,
                         void *mu_out, void *stream) {
-    TOA_DISPATCH(dtype, [&] {
+    TOA_DISPATCH_ALL(dtype, [&] {
         const ForwardMu<T> op{(T)b1};
         T *const p[3] = {mut<T>(updates), mut<T>(mu), (T *)mu_out};
         return launch_single<T>(op, p, n, stream);
@@ -229,7 +253,7 @@ int toa_adam_forward_mu(int dtype, const void *updates, const void *mu, size_t n
 
 int toa_adam_forward_nu(int dtype, const void *updates, const void *nu, size_t n, double b2,
                         void *nu_out, void *stream) {
-    TOA_DISPATCH(dtype, [&] {
+    TOA_DISPATCH_ALL(dtype, [&] {
         const ForwardNu<T> op{(T)b2};
         T *const p[3] = {mut<T>(updates), mut<T>(nu), (T *)nu_out};
         return launch_single<T>(op, p, n, stream);
@@ -240,7 +264,7 @@ int toa_adam_forward_updates(int dtype, const void *new_mu, const void *new_nu, 
                              double b1, double b2, double eps, double eps_root, uint64_t count,
                              void *updates_out, void *stream) {
     const HostScalars s = host_scalars(b1, b2, eps_root, count);
-    TOA_DISPATCH(dtype, [&] {
+    TOA_DISPATCH_ALL(dtype, [&] {
         const ForwardUpdates<T> op{(T)s.c1, (T)s.c2, (T)eps, (T)eps_root};
         T *const p[3] = {mut<T>(new_mu), mut<T>(new_nu), (T *)updates_out};
         return launch_single<T>(op, p, n, stream);
@@ -249,7 +273,7 @@ int toa_adam_forward_updates(int dtype, const void *new_mu, const void *new_nu, 
 
 int toa_adam_backward_mu(int dtype, const void *dmu, size_t n, double b1, void *dupdates_out,
                          void *dmu_out, void *stream) {
-    TOA_DISPATCH(dtype, [&] {
+    TOA_DISPATCH_ALL(dtype, [&] {
         const BackwardMu<T> op{(T)b1};
         T *const p[3] = {mut<T>(dmu), (T *)dupdates_out, (T *)dmu_out};
         return launch_single<T>(op, p, n, stream);
@@ -258,7 +282,7 @@ int toa_adam_backward_mu(int dtype, const void *dmu, size_t n, double b1, void *
 
 int toa_adam_backward_nu(int dtype, const void *dnu, const void *updates, size_t n, double b2,
                          void *dupdates_out, void *dnu_out, void *stream) {
-    TOA_DISPATCH(dtype, [&] {
+    TOA_DISPATCH_ALL(dtype, [&] {
         const BackwardNu<T> op{(T)b2};
         T *const p[4] = {mut<T>(dnu), mut<T>(updates), (T *)dupdates_out, (T *)dnu_out};
         return launch_single<T>(op, p, n, stream);
@@ -270,7 +294,7 @@ int toa_adam_backward_updates(int dtype, const void *dupdates, const void *updat
                               double eps_root, uint64_t count, void *dnew_mu_out,
                               void *dnew_nu_out, void *stream) {
     const HostScalars s = host_scalars(b1, b2, eps_root, count);
-    TOA_DISPATCH(dtype, [&] {
+    TOA_DISPATCH_ALL(dtype, [&] {
         const BackwardUpdates<T> op{(T)s.p1, (T)s.q2};
         T *const p[5] = {mut<T>(dupdates), mut<T>(updates), mut<T>(new_mu), (T *)dnew_mu_out,
                          (T *)dnew_nu_out};
@@ -286,7 +310,7 @@ int toa_adam_forward_inplace_multi(int dtype, size_t num_tensors, void *const *u
                                    void *const *mu, void *const *nu, const size_t *n, double b1,
                                    double b2, double eps, double eps_root,
                                    const uint64_t *counts, uint64_t count_all, void *stream) {
-    TOA_DISPATCH(dtype, [&] {
+    TOA_DISPATCH_ALL(dtype, [&] {
         const void *const *const lists[3] = {CPP(updates), CPP(mu), CPP(nu)};
         auto make = [&](uint64_t c) {
             const HostScalars s = host_scalars(b1, b2, eps_root, c);
@@ -300,7 +324,7 @@ int toa_adam_forward_inplace_multi(int dtype, size_t num_tensors, void *const *u
 int toa_adam_forward_mu_multi(int dtype, size_t num_tensors, const void *const *updates,
                               const void *const *mu, const size_t *n, double b1,
                               void *const *mu_out, void *stream) {
-    TOA_DISPATCH(dtype, [&] {
+    TOA_DISPATCH_ALL(dtype, [&] {
         const void *const *const lists[3] = {updates, mu, CPP(mu_out)};
         auto make = [&](uint64_t) { return ForwardMu<T>{(T)b1}; };
         return launch_multi<T, ForwardMu<T>>(make, num_tensors, lists, n, nullptr, 0, stream);
@@ -310,7 +334,7 @@ int toa_adam_forward_mu_multi(int dtype, size_t num_tensors, const void *const *
 int toa_adam_forward_nu_multi(int dtype, size_t num_tensors, const void *const *updates,
                               const void *const *nu, const size_t *n, double b2,
                               void *const *nu_out, void *stream) {
-    TOA_DISPATCH(dtype, [&] {
+    TOA_DISPATCH_ALL(dtype, [&] {
         const void *const *const lists[3] = {updates, nu, CPP(nu_out)};
         auto make = [&](uint64_t) { return ForwardNu<T>{(T)b2}; };
         return launch_multi<T, ForwardNu<T>>(make, num_tensors, lists, n, nullptr, 0, stream);
@@ -322,7 +346,7 @@ int toa_adam_forward_updates_multi(int dtype, size_t num_tensors, const void *co
                                    double b2, double eps, double eps_root,
                                    const uint64_t *counts, uint64_t count_all,
                                    void *const *updates_out, void *stream) {
-    TOA_DISPATCH(dtype, [&] {
+    TOA_DISPATCH_ALL(dtype, [&] {
         const void *const *const lists[3] = {new_mu, new_nu, CPP(updates_out)};
         auto make = [&](uint64_t c) {
             const HostScalars s = host_scalars(b1, b2, eps_root, c);
@@ -336,7 +360,7 @@ int toa_adam_forward_updates_multi(int dtype, size_t num_tensors, const void *co
 int toa_adam_backward_mu_multi(int dtype, size_t num_tensors, const void *const *dmu,
                                const size_t *n, double b1, void *const *dupdates_out,
                                void *const *dmu_out, void *stream) {
-    TOA_DISPATCH(dtype, [&] {
+    TOA_DISPATCH_ALL(dtype, [&] {
         const void *const *const lists[3] = {dmu, CPP(dupdates_out), CPP(dmu_out)};
         auto make = [&](uint64_t) { return BackwardMu<T>{(T)b1}; };
         return launch_multi<T, BackwardMu<T>>(make, num_tensors, lists, n, nullptr, 0, stream);
@@ -346,7 +370,7 @@ int toa_adam_backward_mu_multi(int dtype, size_t num_tensors, const void *const 
 int toa_adam_backward_nu_multi(int dtype, size_t num_tensors, const void *const *dnu,
                                const void *const *updates, const size_t *n, double b2,
                                void *const *dupdates_out, void *const *dnu_out, void *stream) {
-    TOA_DISPATCH(dtype, [&] {
+    TOA_DISPATCH_ALL(dtype, [&] {
         const void *const *const lists[4] = {dnu, updates, CPP(dupdates_out), CPP(dnu_out)};
         auto make = [&](uint64_t) { return BackwardNu<T>{(T)b2}; };
         return launch_multi<T, BackwardNu<T>>(make, num_tensors, lists, n, nullptr, 0, stream);
@@ -359,7 +383,7 @@ int toa_adam_backward_updates_multi(int dtype, size_t num_tensors, const void *c
                                     const uint64_t *counts, uint64_t count_all,
                                     void *const *dnew_mu_out, void *const *dnew_nu_out,
                                     void *stream) {
-    TOA_DISPATCH(dtype, [&] {
+    TOA_DISPATCH_ALL(dtype, [&] {
         const void *const *const lists[5] = {dupdates, updates, new_mu, CPP(dnew_mu_out),
                                              CPP(dnew_nu_out)};
         auto make = [&](uint64_t c) {
