@@ -5,10 +5,17 @@
     from torchopt_amd import accelerated_op_available
 """
 
+import sys as _sys
+
 from torchopt_amd import accelerated_op
 from torchopt_amd.accelerated_op import AdamOp, MultiAdamOp
 from torchopt_amd.accelerated_op import is_available as accelerated_op_available
 from torchopt_amd.optim import FusedAdam
+
+# `import torchopt_amd._C.adam_op` should work like `from torchopt_amd._C import adam_op`
+from torchopt_amd import _C  # noqa: E402
+
+_sys.modules.setdefault('torchopt_amd._C.adam_op', _C.adam_op)
 
 __version__ = '0.1.0'
 

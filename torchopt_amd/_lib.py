@@ -59,7 +59,7 @@ _lock = threading.Lock()
 
 
 class LibraryNotBuiltError(ImportError):
-    """libtoa_adam.so is missing; run `python -m torchopt_amd.build`."""
+    """libtoa_adam.so is missing; run `python torchopt_amd/build.py`."""
 
 
 def load() -> ctypes.CDLL:
@@ -73,7 +73,7 @@ def load() -> ctypes.CDLL:
         if not os.path.exists(LIB_PATH):
             raise LibraryNotBuiltError(
                 f'{LIB_PATH} not found: the HIP library has not been built '
-                '(run `python -m torchopt_amd.build`); there is no fallback path',
+                '(run `python torchopt_amd/build.py`); there is no fallback path',
             )
         lib = ctypes.CDLL(LIB_PATH)
         lib.toa_adam_abi_version.restype = _i

@@ -21,7 +21,13 @@ from typing import Any
 
 import torch
 
-from torchopt_amd._C import adam_op
+try:
+    from torchopt_amd._C import adam_op
+except ImportError as exc:  # no fallback module: the op is the compiled extension or nothing
+    raise ImportError(
+        'torchopt_amd._C, the compiled extension in front of libtoa_adam.so, cannot be '
+        f'imported ({exc}); build it with `python torchopt_amd/build.py`. There is no '
+        'pure-Python or CPU fallback.') from exc
 
 
 class AdamOp:

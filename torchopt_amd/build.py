@@ -1,8 +1,12 @@
-"""Compile libtoa_adam.so (HIP, gfx950 only) in-tree with hipcc.
+"""Compile the two in-tree binaries:
 
-    python -m torchopt_amd.build
+  libtoa_adam.so              the HIP kernels behind the C ABI (hipcc, gfx950 only)
+  _C.<python-abi>.so          the PyTorch extension module in front of it (g++, host only)
 
-hipcc cross-compiles without a GPU, so this runs anywhere ROCm is installed.
+    python torchopt_amd/build.py
+
+(run as a script, or load this file by path: importing the package itself needs the binaries
+this file produces).  hipcc cross-compiles without a GPU, so this runs anywhere ROCm and PyTorch-ROCm are installed.
 """
 
 from __future__ import annotations
@@ -11,6 +15,7 @@ import os
 import shutil
 import subprocess
 import sys
+import sysconfig
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 REPO_DIR = os.path.dirname(PKG_DIR)
@@ -72,5 +77,46 @@ def build_library(force: bool = True, verbose: bool = False) -> str:
     return LIB_PATH
 
 
+BINDING_SRC = os.path.join(PKG_DIR, 'csrc', 'binding.cpp')
+BINDING_PATH = os.path.join(PKG_DIR, '_C' + sysconfig.get_config_var('EXT_SUFFIX'))
+
+
+def build_binding(verbose: bool = False) -> str:
+    """Compile torchopt_amd/_C*.so: pybind11 + ATen on the host side, linked against
+    libtoa_adam.so (found next to it at run time through an $ORIGIN rpath)."""
+    import torch
+    from torch.utils import cpp_extension
+
+    if not os.path.exists(LIB_PATH):
+        build_library()
+    rocm = os.environ.get('ROCM_PATH', '/opt/rocm')
+    torch_lib = cpp_extension.library_paths()[0]
+    includes = [os.path.join(REPO_DIR, 'include'), *cpp_extension.include_paths(),
+                sysconfig.get_paths()['include'], os.path.join(rocm, 'include')]
+    cmd = [os.environ.get('CXX', 'g++'), '-O2', '-std=c++17', '-fPIC', '-shared',
+           '-fvisibility=hidden', '-Wall', '-Wno-unused-function',
+           '-D__HIP_PLATFORM_AMD__=1', '-DUSE_ROCM=1', '-DTORCH_EXTENSION_NAME=_C',
+           f'-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}',
+           *[f'-I{p}' for p in includes], BINDING_SRC, '-o', BINDING_PATH + '.tmp',
+           f'-L{torch_lib}', f'-L{PKG_DIR}', f'-L{os.path.join(rocm, "lib")}',
+           '-ltorch_python', '-ltorch', '-ltorch_cpu', '-lc10', '-lc10_hip', '-ltorch_hip',
+           '-l:libtoa_adam.so', '-lamdhip64',
+           '-Wl,-rpath,$ORIGIN', f'-Wl,-rpath,{torch_lib}', f'-Wl,-rpath,{os.path.join(rocm, "lib")}']
+    if verbose:
+        print(' '.join(cmd), flush=True)
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f'{cmd[0]} failed ({proc.returncode}):\n{proc.stderr[-4000:]}')
+    if verbose and proc.stderr.strip():
+        print(proc.stderr, file=sys.stderr)
+    os.replace(BINDING_PATH + '.tmp', BINDING_PATH)
+    return BINDING_PATH
+
+
+def build_all(verbose: bool = False) -> list[str]:
+    return [build_library(force=True, verbose=verbose), build_binding(verbose=verbose)]
+
+
 if __name__ == '__main__':
-    print(build_library(force=True, verbose=True))
+    for path in build_all(verbose=True):
+        print(path)

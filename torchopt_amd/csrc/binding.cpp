@@ -1,0 +1,567 @@
+// torchopt_amd._C -- the PyTorch-ROCm extension module in front of libtoa_adam.so.
+//
+// Counterpart of the reference's pybind11 module: PYBIND11_MODULE(_C) with one
+// submodule, `adam_op` (/root/reference/src/extension.cpp:20,
+// /root/reference/src/adam_op/adam_op.cpp:155-215).  Same seven functions, same
+// keyword names (including backward_nu's fourth keyword being registered as
+// "b1", adam_op.cpp:203), same conversions (double for floats, size_t for
+// `count`, so a 0-dim integer tensor is accepted through __index__), same
+// return conventions (std::array -> list; forward_ hands back its inputs), same
+// exception classes.  It is thin on purpose: checks, empty_like, device and
+// stream, then one call into the C ABI (include/toa_adam.h).  No arithmetic
+// happens here and no torch type crosses the ABI.
+//
+// Deliberate differences from the reference dispatcher (adam_op.cpp:32-153):
+//   * only GPU tensors are served; every other device raises
+//     std::runtime_error("Not implemented"), the reference's own error for a
+//     device it has no kernel for (adam_op.cpp:47-49);
+//   * kernels go to PyTorch's current stream of the tensors' device instead of
+//     the null stream (adam_op_impl_cuda.cu:83);
+//   * element counts, dtypes, devices and memory layouts are checked instead of
+//     assumed;
+//   * additive list entry points (forward_multi_, ...) and the fused optimizer
+//     step (fused_step_, fused_step_multi_).
+#include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime_api.h>
+#include <pybind11/stl.h>
+#include <torch/extension.h>
+
+#include <array>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "toa_adam.h"
+
+namespace py = pybind11;
+
+namespace {
+
+using at::Tensor;
+using TensorList = std::vector<Tensor>;
+
+int dtypeCode(const Tensor &t, const char *name) {
+    switch (t.scalar_type()) {
+        case at::kFloat: return TOA_F32;
+        case at::kDouble: return TOA_F64;
+        case at::kHalf: return TOA_F16;
+        case at::kBFloat16: return TOA_BF16;
+        default:
+            // wording of ATen's dispatch failure, which is what the reference raises
+            TORCH_CHECK(false, "\"", name, "\" not implemented for '", t.scalar_type(), "'");
+    }
+}
+
+void check(int rc, const char *name) {
+    TORCH_CHECK(rc == 0, name, ": ", toa_adam_error_string(rc), " (code ", rc, ")");
+}
+
+// Device, dtype and size agreement; returns the dtype code and sets n.
+int gate(const char *name, const Tensor &lead, std::initializer_list<const Tensor *> others,
+         size_t *n) {
+    if (!lead.is_cuda()) throw std::runtime_error("Not implemented");
+    const int code = dtypeCode(lead, name);
+    *n = (size_t)lead.numel();
+    for (const Tensor *t : others) {
+        TORCH_CHECK(t->device() == lead.device(), name, ": expected all tensors on ",
+                    lead.device(), ", got one on ", t->device());
+        TORCH_CHECK(t->scalar_type() == lead.scalar_type(), name, ": expected scalar type ",
+                    lead.scalar_type(), " but found ", t->scalar_type());
+        TORCH_CHECK((size_t)t->numel() == *n, name, ": size mismatch, ", *n, " vs ", t->numel(),
+                    " elements");
+    }
+    return code;
+}
+
+void requireDense(const char *name, const char *what, const Tensor &t) {
+    TORCH_CHECK(t.is_non_overlapping_and_dense(), name, ": `", what,
+                "` must be contiguous (non-overlapping and dense), got sizes ", t.sizes(),
+                " strides ", t.strides());
+}
+
+bool sameLayout(const Tensor &a, const Tensor &b) {
+    return a.numel() <= 1 || a.strides() == b.strides();
+}
+
+// A read-only operand in the memory order of `donor`, copying only if it is not already.
+// (The reference makes incoming gradients .contiguous(), adam_op.cpp:107,123,143.)
+Tensor asLayoutOf(const Tensor &x, const Tensor &donor) {
+    if (x.numel() <= 1 || (x.is_contiguous() && donor.is_contiguous())) return x;
+    if (x.sizes() == donor.sizes())
+        return x.strides() == donor.strides() ? x : at::empty_like(donor).copy_(x);
+    TORCH_CHECK(donor.is_contiguous(), "operands of different shapes must be contiguous");
+    return x.contiguous();
+}
+
+// Makes the tensors' device current for the launch (the C ABI uses the current device) and
+// hands out PyTorch's current stream on it.
+class OnDeviceOf {
+  public:
+    explicit OnDeviceOf(const Tensor &t) : index_((int)t.get_device()) {
+        if (hipGetDevice(&prev_) != hipSuccess) prev_ = index_;
+        if (prev_ != index_) TORCH_CHECK(hipSetDevice(index_) == hipSuccess, "hipSetDevice failed");
+    }
+    ~OnDeviceOf() {
+        if (prev_ != index_) (void)hipSetDevice(prev_);
+    }
+    void *stream() const {
+        return (void *)c10::hip::getCurrentHIPStream((c10::DeviceIndex)index_).stream();
+    }
+
+  private:
+    int index_;
+    int prev_ = 0;
+};
+
+// ---- single tensor -------------------------------------------------------------------------
+
+std::array<Tensor, 3> forwardInplace(const Tensor &updates, const Tensor &mu, const Tensor &nu,
+                                     double b1, double b2, double eps, double eps_root,
+                                     size_t count) {
+    const char *name = "adamForwardInplace";
+    size_t n;
+    const int code = gate(name, updates, {&mu, &nu}, &n);
+    if (n) {
+        requireDense(name, "updates", updates);
+        requireDense(name, "mu", mu);
+        requireDense(name, "nu", nu);
+        TORCH_CHECK(sameLayout(updates, mu) && sameLayout(updates, nu), name,
+                    ": updates, mu and nu must share one memory layout");
+        const OnDeviceOf dev(updates);
+        check(toa_adam_forward_inplace(code, updates.data_ptr(), mu.data_ptr(), nu.data_ptr(), n,
+                                       b1, b2, eps, eps_root, count, dev.stream()),
+              name);
+    }
+    return {updates, mu, nu};
+}
+
+Tensor forwardMu(const Tensor &updates_in, const Tensor &mu, double b1) {
+    const char *name = "adamForwardMu";
+    size_t n;
+    const int code = gate(name, updates_in, {&mu}, &n);
+    requireDense(name, "mu", mu);
+    Tensor mu_out = at::empty_like(mu);
+    if (n) {
+        const Tensor updates = asLayoutOf(updates_in, mu);
+        const OnDeviceOf dev(mu);
+        check(toa_adam_forward_mu(code, updates.data_ptr(), mu.data_ptr(), n, b1,
+                                  mu_out.data_ptr(), dev.stream()),
+              name);
+    }
+    return mu_out;
+}
+
+Tensor forwardNu(const Tensor &updates_in, const Tensor &nu, double b2) {
+    const char *name = "adamForwardNu";
+    size_t n;
+    const int code = gate(name, updates_in, {&nu}, &n);
+    requireDense(name, "nu", nu);
+    Tensor nu_out = at::empty_like(nu);
+    if (n) {
+        const Tensor updates = asLayoutOf(updates_in, nu);
+        const OnDeviceOf dev(nu);
+        check(toa_adam_forward_nu(code, updates.data_ptr(), nu.data_ptr(), n, b2,
+                                  nu_out.data_ptr(), dev.stream()),
+              name);
+    }
+    return nu_out;
+}
+
+Tensor forwardUpdates(const Tensor &new_mu, const Tensor &new_nu_in, double b1, double b2,
+                      double eps, double eps_root, size_t count) {
+    const char *name = "adamForwardUpdates";
+    size_t n;
+    const int code = gate(name, new_mu, {&new_nu_in}, &n);
+    requireDense(name, "new_mu", new_mu);
+    Tensor updates_out = at::empty_like(new_mu);
+    if (n) {
+        const Tensor new_nu = asLayoutOf(new_nu_in, new_mu);
+        const OnDeviceOf dev(new_mu);
+        check(toa_adam_forward_updates(code, new_mu.data_ptr(), new_nu.data_ptr(), n, b1, b2, eps,
+                                       eps_root, count, updates_out.data_ptr(), dev.stream()),
+              name);
+    }
+    return updates_out;
+}
+
+std::array<Tensor, 2> backwardMu(const Tensor &dmu_in, const Tensor &updates, const Tensor &mu,
+                                 double b1) {
+    const char *name = "adamBackwardMu";
+    size_t n;
+    const int code = gate(name, dmu_in, {&updates, &mu}, &n);
+    requireDense(name, "updates", updates);
+    requireDense(name, "mu", mu);
+    Tensor dupdates_out = at::empty_like(updates);
+    Tensor dmu_out = at::empty_like(mu);
+    if (n) {
+        TORCH_CHECK(sameLayout(dupdates_out, dmu_out), name,
+                    ": updates and mu must share one memory layout");
+        const Tensor dmu = asLayoutOf(dmu_in, dmu_out);
+        const OnDeviceOf dev(dmu);
+        check(toa_adam_backward_mu(code, dmu.data_ptr(), n, b1, dupdates_out.data_ptr(),
+                                   dmu_out.data_ptr(), dev.stream()),
+              name);
+    }
+    return {dupdates_out, dmu_out};
+}
+
+std::array<Tensor, 2> backwardNu(const Tensor &dnu_in, const Tensor &updates, const Tensor &nu,
+                                 double b2) {
+    const char *name = "adamBackwardNu";
+    size_t n;
+    const int code = gate(name, dnu_in, {&updates, &nu}, &n);
+    requireDense(name, "updates", updates);
+    requireDense(name, "nu", nu);
+    Tensor dupdates_out = at::empty_like(updates);
+    Tensor dnu_out = at::empty_like(nu);
+    if (n) {
+        TORCH_CHECK(sameLayout(dupdates_out, dnu_out), name,
+                    ": updates and nu must share one memory layout");
+        const Tensor dnu = asLayoutOf(dnu_in, dnu_out);
+        const OnDeviceOf dev(dnu);
+        check(toa_adam_backward_nu(code, dnu.data_ptr(), updates.data_ptr(), n, b2,
+                                   dupdates_out.data_ptr(), dnu_out.data_ptr(), dev.stream()),
+              name);
+    }
+    return {dupdates_out, dnu_out};
+}
+
+std::array<Tensor, 2> backwardUpdates(const Tensor &dupdates_in, const Tensor &updates_in,
+                                      const Tensor &new_mu, const Tensor &new_nu, double b1,
+                                      double b2, double eps_root, size_t count) {
+    const char *name = "adamBackwardUpdates";
+    size_t n;
+    const int code = gate(name, dupdates_in, {&updates_in, &new_mu, &new_nu}, &n);
+    requireDense(name, "new_mu", new_mu);
+    requireDense(name, "new_nu", new_nu);
+    Tensor dmu_out = at::empty_like(new_mu);
+    Tensor dnu_out = at::empty_like(new_nu);
+    if (n) {
+        TORCH_CHECK(sameLayout(dmu_out, dnu_out), name,
+                    ": new_mu and new_nu must share one memory layout");
+        const Tensor dupdates = asLayoutOf(dupdates_in, dmu_out);
+        const Tensor updates = asLayoutOf(updates_in, dmu_out);
+        const OnDeviceOf dev(dupdates);
+        check(toa_adam_backward_updates(code, dupdates.data_ptr(), updates.data_ptr(),
+                                        new_mu.data_ptr(), n, b1, b2, eps_root, count,
+                                        dmu_out.data_ptr(), dnu_out.data_ptr(), dev.stream()),
+              name);
+    }
+    return {dmu_out, dnu_out};
+}
+
+std::array<Tensor, 4> fusedStep(const Tensor &params, const Tensor &updates, const Tensor &mu,
+                                const Tensor &nu, double b1, double b2, double eps,
+                                double eps_root, size_t count, double lr, bool maximize,
+                                bool write_updates) {
+    const char *name = "adamFusedStep";
+    size_t n;
+    const int code = gate(name, updates, {&mu, &nu, &params}, &n);
+    if (n) {
+        requireDense(name, "params", params);
+        requireDense(name, "updates", updates);
+        requireDense(name, "mu", mu);
+        requireDense(name, "nu", nu);
+        TORCH_CHECK(sameLayout(params, updates) && sameLayout(params, mu) && sameLayout(params, nu),
+                    name, ": params, updates, mu and nu must share one memory layout");
+        const OnDeviceOf dev(updates);
+        check(toa_adam_fused_step(code, params.data_ptr(), updates.data_ptr(), mu.data_ptr(),
+                                  nu.data_ptr(), n, b1, b2, eps, eps_root, count, lr,
+                                  (int)maximize, (int)write_updates, dev.stream()),
+              name);
+    }
+    return {params, updates, mu, nu};
+}
+
+// ---- lists of tensors ----------------------------------------------------------------------
+
+struct Lists {
+    int code = TOA_F32;
+    size_t num = 0;
+    std::vector<size_t> n;
+    std::vector<std::vector<void *>> ptr;  // one vector per operand list
+};
+
+// Checks for a list call: equal lengths, one device and dtype, per-tensor size agreement and a
+// shared dense layout.  Collects sizes and data pointers on the way.
+Lists gateLists(const char *name, std::initializer_list<const TensorList *> lists) {
+    Lists out;
+    const TensorList &first = **lists.begin();
+    out.num = first.size();
+    for (const TensorList *l : lists)
+        TORCH_CHECK(l->size() == out.num, name, ": tensor lists differ in length");
+    if (out.num == 0) return out;
+    const Tensor &lead = first[0];
+    if (!lead.is_cuda()) throw std::runtime_error("Not implemented");
+    out.code = dtypeCode(lead, name);
+    out.n.resize(out.num);
+    for (size_t k = 0; k < out.num; ++k) out.n[k] = (size_t)first[k].numel();
+    for (const TensorList *l : lists) {
+        std::vector<void *> p(out.num);
+        for (size_t k = 0; k < out.num; ++k) {
+            const Tensor &t = (*l)[k];
+            TORCH_CHECK(t.device() == lead.device(), name,
+                        ": all tensors of one call must be on ", lead.device());
+            TORCH_CHECK(t.scalar_type() == lead.scalar_type(), name, ": expected scalar type ",
+                        lead.scalar_type(), " but found ", t.scalar_type());
+            TORCH_CHECK((size_t)t.numel() == out.n[k], name, ": size mismatch in tensor ", k);
+            if (out.n[k] > 1)
+                TORCH_CHECK(t.is_non_overlapping_and_dense() && t.strides() == first[k].strides(),
+                            name, ": tensor ", k, " operands must share one dense layout");
+            p[k] = out.n[k] ? t.data_ptr() : nullptr;
+        }
+        out.ptr.push_back(std::move(p));
+    }
+    return out;
+}
+
+struct Counts {
+    std::vector<uint64_t> each;  // empty when one value serves all
+    uint64_t all = 0;
+    const uint64_t *data() const { return each.empty() ? nullptr : each.data(); }
+};
+
+uint64_t toCount(const py::handle &h) {
+    // what pybind11 does for a size_t parameter: __index__, non-negative
+    py::object idx = py::reinterpret_steal<py::object>(PyNumber_Index(h.ptr()));
+    if (!idx) throw py::error_already_set();
+    if (PyObject_RichCompareBool(idx.ptr(), py::int_(0).ptr(), Py_LT) == 1)
+        throw py::type_error("count must be a non-negative integer");
+    return idx.cast<uint64_t>();
+}
+
+// `counts`: one step number for all tensors, or a list/tuple with one per tensor (ints or
+// 0-dim integer tensors; a list of device tensors is read back with one transfer).
+Counts parseCounts(const py::object &counts, size_t num) {
+    Counts out;
+    if (!py::isinstance<py::list>(counts) && !py::isinstance<py::tuple>(counts)) {
+        out.all = toCount(counts);
+        return out;
+    }
+    const py::sequence seq = py::reinterpret_borrow<py::sequence>(counts);
+    TORCH_CHECK((size_t)py::len(seq) == num, "expected ", num, " counts, got ", py::len(seq));
+    std::vector<uint64_t> values(num);
+    bool all_tensors = num > 0;
+    for (const py::handle &h : seq) all_tensors = all_tensors && THPVariable_Check(h.ptr());
+    if (all_tensors) {
+        TensorList ts;
+        ts.reserve(num);
+        for (const py::handle &h : seq) ts.push_back(THPVariable_Unpack(h.ptr()).reshape({}));
+        const Tensor host = at::stack(ts).to(at::kLong).cpu();
+        const int64_t *v = host.data_ptr<int64_t>();
+        for (size_t k = 0; k < num; ++k) {
+            if (v[k] < 0) throw py::type_error("counts must be non-negative integers");
+            values[k] = (uint64_t)v[k];
+        }
+    } else {
+        size_t k = 0;
+        for (const py::handle &h : seq) values[k++] = toCount(h);
+    }
+    bool uniform = true;
+    for (size_t k = 1; k < num; ++k) uniform = uniform && values[k] == values[0];
+    if (uniform)
+        out.all = num ? values[0] : 0;
+    else
+        out.each = std::move(values);
+    return out;
+}
+
+TensorList emptyLike(const TensorList &donors) {
+    TensorList out;
+    out.reserve(donors.size());
+    for (const Tensor &t : donors) out.push_back(at::empty_like(t));
+    return out;
+}
+
+TensorList asLayoutOfEach(const TensorList &xs, const TensorList &donors, const char *name) {
+    TORCH_CHECK(xs.size() == donors.size(), name, ": tensor lists differ in length");
+    TensorList out;
+    out.reserve(xs.size());
+    for (size_t k = 0; k < xs.size(); ++k) out.push_back(asLayoutOf(xs[k], donors[k]));
+    return out;
+}
+
+const Tensor &firstNonEmpty(const TensorList &l) { return l[0]; }
+
+py::tuple forwardMultiInplace(const py::object &updates_o, const py::object &mu_o,
+                              const py::object &nu_o, double b1, double b2, double eps,
+                              double eps_root, const py::object &counts) {
+    const char *name = "adamForwardInplaceMulti";
+    const auto updates = updates_o.cast<TensorList>();
+    const auto mu = mu_o.cast<TensorList>();
+    const auto nu = nu_o.cast<TensorList>();
+    Lists l = gateLists(name, {&updates, &mu, &nu});
+    if (l.num) {
+        const Counts c = parseCounts(counts, l.num);
+        const OnDeviceOf dev(firstNonEmpty(updates));
+        check(toa_adam_forward_inplace_multi(l.code, l.num, l.ptr[0].data(), l.ptr[1].data(),
+                                             l.ptr[2].data(), l.n.data(), b1, b2, eps, eps_root,
+                                             c.data(), c.all, dev.stream()),
+              name);
+    }
+    return py::make_tuple(updates_o, mu_o, nu_o);  // the caller's own lists, mutated in place
+}
+
+TensorList forwardMuMulti(const TensorList &updates, const TensorList &mu, double b1) {
+    const char *name = "adamForwardMuMulti";
+    TensorList out = emptyLike(mu);
+    Lists l = gateLists(name, {&updates, &mu, &out});
+    if (l.num) {
+        const OnDeviceOf dev(firstNonEmpty(mu));
+        check(toa_adam_forward_mu_multi(l.code, l.num, l.ptr[0].data(), l.ptr[1].data(),
+                                        l.n.data(), b1, l.ptr[2].data(), dev.stream()),
+              name);
+    }
+    return out;
+}
+
+TensorList forwardNuMulti(const TensorList &updates, const TensorList &nu, double b2) {
+    const char *name = "adamForwardNuMulti";
+    TensorList out = emptyLike(nu);
+    Lists l = gateLists(name, {&updates, &nu, &out});
+    if (l.num) {
+        const OnDeviceOf dev(firstNonEmpty(nu));
+        check(toa_adam_forward_nu_multi(l.code, l.num, l.ptr[0].data(), l.ptr[1].data(),
+                                        l.n.data(), b2, l.ptr[2].data(), dev.stream()),
+              name);
+    }
+    return out;
+}
+
+TensorList forwardUpdatesMulti(const TensorList &new_mu, const TensorList &new_nu, double b1,
+                               double b2, double eps, double eps_root, const py::object &counts) {
+    const char *name = "adamForwardUpdatesMulti";
+    TensorList out = emptyLike(new_mu);
+    Lists l = gateLists(name, {&new_mu, &new_nu, &out});
+    if (l.num) {
+        const Counts c = parseCounts(counts, l.num);
+        const OnDeviceOf dev(firstNonEmpty(new_mu));
+        check(toa_adam_forward_updates_multi(l.code, l.num, l.ptr[0].data(), l.ptr[1].data(),
+                                             l.n.data(), b1, b2, eps, eps_root, c.data(), c.all,
+                                             l.ptr[2].data(), dev.stream()),
+              name);
+    }
+    return out;
+}
+
+std::tuple<TensorList, TensorList> backwardMuMulti(const TensorList &dmu_in,
+                                                   const TensorList &updates,
+                                                   const TensorList &mu, double b1) {
+    const char *name = "adamBackwardMuMulti";
+    TensorList dupdates_out = emptyLike(updates), dmu_out = emptyLike(mu);
+    const TensorList dmu = asLayoutOfEach(dmu_in, dmu_out, name);
+    Lists l = gateLists(name, {&dmu, &dupdates_out, &dmu_out});
+    if (l.num) {
+        const OnDeviceOf dev(firstNonEmpty(dmu));
+        check(toa_adam_backward_mu_multi(l.code, l.num, l.ptr[0].data(), l.n.data(), b1,
+                                         l.ptr[1].data(), l.ptr[2].data(), dev.stream()),
+              name);
+    }
+    return {dupdates_out, dmu_out};
+}
+
+std::tuple<TensorList, TensorList> backwardNuMulti(const TensorList &dnu_in,
+                                                   const TensorList &updates,
+                                                   const TensorList &nu, double b2) {
+    const char *name = "adamBackwardNuMulti";
+    TensorList dupdates_out = emptyLike(updates), dnu_out = emptyLike(nu);
+    const TensorList dnu = asLayoutOfEach(dnu_in, dnu_out, name);
+    Lists l = gateLists(name, {&dnu, &updates, &dupdates_out, &dnu_out});
+    if (l.num) {
+        const OnDeviceOf dev(firstNonEmpty(dnu));
+        check(toa_adam_backward_nu_multi(l.code, l.num, l.ptr[0].data(), l.ptr[1].data(),
+                                         l.n.data(), b2, l.ptr[2].data(), l.ptr[3].data(),
+                                         dev.stream()),
+              name);
+    }
+    return {dupdates_out, dnu_out};
+}
+
+std::tuple<TensorList, TensorList> backwardUpdatesMulti(
+    const TensorList &dupdates_in, const TensorList &updates, const TensorList &new_mu,
+    const TensorList &new_nu, double b1, double b2, double eps_root, const py::object &counts) {
+    const char *name = "adamBackwardUpdatesMulti";
+    TensorList dmu_out = emptyLike(new_mu), dnu_out = emptyLike(new_nu);
+    const TensorList dupdates = asLayoutOfEach(dupdates_in, dmu_out, name);
+    Lists l = gateLists(name, {&dupdates, &updates, &new_mu, &dmu_out, &dnu_out});
+    if (l.num) {
+        const Counts c = parseCounts(counts, l.num);
+        const OnDeviceOf dev(firstNonEmpty(dupdates));
+        check(toa_adam_backward_updates_multi(l.code, l.num, l.ptr[0].data(), l.ptr[1].data(),
+                                              l.ptr[2].data(), l.n.data(), b1, b2, eps_root,
+                                              c.data(), c.all, l.ptr[3].data(), l.ptr[4].data(),
+                                              dev.stream()),
+              name);
+    }
+    return {dmu_out, dnu_out};
+}
+
+py::tuple fusedStepMulti(const py::object &params_o, const py::object &updates_o,
+                         const py::object &mu_o, const py::object &nu_o, double b1, double b2,
+                         double eps, double eps_root, const py::object &counts, double lr,
+                         bool maximize, bool write_updates) {
+    const char *name = "adamFusedStepMulti";
+    const auto params = params_o.cast<TensorList>();
+    const auto updates = updates_o.cast<TensorList>();
+    const auto mu = mu_o.cast<TensorList>();
+    const auto nu = nu_o.cast<TensorList>();
+    Lists l = gateLists(name, {&updates, &mu, &nu, &params});
+    if (l.num) {
+        const Counts c = parseCounts(counts, l.num);
+        const OnDeviceOf dev(firstNonEmpty(updates));
+        check(toa_adam_fused_step_multi(l.code, l.num, l.ptr[3].data(), l.ptr[0].data(),
+                                        l.ptr[1].data(), l.ptr[2].data(), l.n.data(), b1, b2, eps,
+                                        eps_root, c.data(), c.all, lr, (int)maximize,
+                                        (int)write_updates, dev.stream()),
+              name);
+    }
+    return py::make_tuple(params_o, updates_o, mu_o, nu_o);
+}
+
+}  // namespace
+
+PYBIND11_MODULE(_C, mod) {
+    mod.doc() = "MI355X-native counterpart of torchopt._C";
+    py::module m = mod.def_submodule("adam_op", "Adam Ops");
+    using namespace py::literals;
+
+    // the reference's seven (names and keywords as in adam_op.cpp:157-214)
+    m.def("forward_", &forwardInplace, "Adam forward inplace", "updates"_a, "mu"_a, "nu"_a, "b1"_a,
+          "b2"_a, "eps"_a, "eps_root"_a, "count"_a);
+    m.def("forward_mu", &forwardMu, "Adam forward mu", "updates"_a, "mu"_a, "b1"_a);
+    m.def("forward_nu", &forwardNu, "Adam forward nu", "updates"_a, "nu"_a, "b2"_a);
+    m.def("forward_updates", &forwardUpdates, "Adam forward updates", "new_mu"_a, "new_nu"_a,
+          "b1"_a, "b2"_a, "eps"_a, "eps_root"_a, "count"_a);
+    m.def("backward_mu", &backwardMu, "Adam backward mu", "dmu"_a, "updates"_a, "mu"_a, "b1"_a);
+    m.def("backward_nu", &backwardNu, "Adam backward nu", "dnu"_a, "updates"_a, "nu"_a,
+          "b1"_a);  // the decay is b2; the reference registers the keyword as b1
+    m.def("backward_updates", &backwardUpdates, "Adam backward updates", "dupdates"_a, "updates"_a,
+          "new_mu"_a, "new_nu"_a, "b1"_a, "b2"_a, "eps_root"_a, "count"_a);
+
+    // lists of tensors: one launch per hundred-odd tensors
+    m.def("forward_multi_", &forwardMultiInplace,
+          "forward_ over lists; mutates and returns (updates, mu, nu)", "updates"_a, "mu"_a,
+          "nu"_a, "b1"_a, "b2"_a, "eps"_a, "eps_root"_a, "counts"_a);
+    m.def("forward_mu_multi", &forwardMuMulti, "forward_mu over lists", "updates"_a, "mu"_a,
+          "b1"_a);
+    m.def("forward_nu_multi", &forwardNuMulti, "forward_nu over lists", "updates"_a, "nu"_a,
+          "b2"_a);
+    m.def("forward_updates_multi", &forwardUpdatesMulti, "forward_updates over lists", "new_mu"_a,
+          "new_nu"_a, "b1"_a, "b2"_a, "eps"_a, "eps_root"_a, "counts"_a);
+    m.def("backward_mu_multi", &backwardMuMulti, "backward_mu over lists -> (dupdates, dmu)",
+          "dmu"_a, "updates"_a, "mu"_a, "b1"_a);
+    m.def("backward_nu_multi", &backwardNuMulti, "backward_nu over lists -> (dupdates, dnu)",
+          "dnu"_a, "updates"_a, "nu"_a, "b2"_a);
+    m.def("backward_updates_multi", &backwardUpdatesMulti,
+          "backward_updates over lists -> (dnew_mu, dnew_nu)", "dupdates"_a, "updates"_a,
+          "new_mu"_a, "new_nu"_a, "b1"_a, "b2"_a, "eps_root"_a, "counts"_a);
+
+    // the classic in-place optimizer step in one pass
+    m.def("fused_step_", &fusedStep,
+          "Adam + scale(-lr) + apply in one pass; returns [params, updates, mu, nu]", "params"_a,
+          "updates"_a, "mu"_a, "nu"_a, "b1"_a, "b2"_a, "eps"_a, "eps_root"_a, "count"_a, "lr"_a,
+          py::kw_only(), "maximize"_a = false, "write_updates"_a = false);
+    m.def("fused_step_multi_", &fusedStepMulti, "fused_step_ over lists", "params"_a, "updates"_a,
+          "mu"_a, "nu"_a, "b1"_a, "b2"_a, "eps"_a, "eps_root"_a, "counts"_a, "lr"_a,
+          py::kw_only(), "maximize"_a = false, "write_updates"_a = false);
+}

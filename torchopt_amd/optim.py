@@ -23,7 +23,7 @@ from typing import Callable, Iterable, Sequence
 
 import torch
 
-from torchopt_amd._C import adam_op
+from torchopt_amd.accelerated_op.adam_op import adam_op
 from torchopt_amd.transform.scale_by_adam import ScaleByAdamState, _inc_counts, _remember
 
 

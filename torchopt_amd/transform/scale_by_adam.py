@@ -141,12 +141,15 @@ def _scale_by_accelerated_adam(
         raise ValueError(f'Invalid beta parameter at index 1: {b2}')
 
     def flatten(tree):
-        if already_flattened:
+        # a plain list / tuple of tensors and Nones is its own flattening; the general walk
+        # (pure Python in torch.utils._pytree) costs ~3 us per leaf per tree
+        if already_flattened or (type(tree) in (list, tuple) and all(
+                t is None or isinstance(t, torch.Tensor) for t in tree)):
             return list(tree), None
         return pytree.tree_flatten(tree)
 
     def rebuild(leaves, like, spec):
-        if already_flattened:
+        if spec is None:
             return leaves if type(like) is list else type(like)(leaves)
         return pytree.tree_unflatten(leaves, spec)
 
