@@ -27,7 +27,7 @@
  *   return    0 on success; a positive value is a hipError_t from the launch;
  *             a negative value is one of the TOA_E* argument errors below.
  *             toa_adam_error_string() names either kind.
- *   threads   re-entrant; the only global state is the residency knob below.
+ *   threads   re-entrant; the only global state is the two tuning knobs below.
  */
 #ifndef TOA_ADAM_H
 #define TOA_ADAM_H
@@ -64,6 +64,13 @@ TOA_API int toa_adam_abi_version(void);
  * variable TOA_ADAM_WAVES_PER_CU sets the initial override.  Returns the
  * previous override (0 = none).  No counterpart in the reference. */
 TOA_API int toa_adam_set_waves_per_cu(int waves);
+
+/* Cap on workgroups per launch (default and maximum 2^25).  Every kernel normally runs one
+ * workgroup per 1 KiB tile; beyond the cap workgroups stride over the remaining tiles.  Lowering
+ * the cap exercises that path on small inputs (tests) and trades dispatch work for loop
+ * iterations.  0 or an out-of-range value restores the default.  Returns the previous cap.
+ * No counterpart in the reference. */
+TOA_API unsigned toa_adam_set_max_grid(unsigned workgroups);
 
 /* Human-readable name of a return code from any function below. */
 TOA_API const char *toa_adam_error_string(int code);

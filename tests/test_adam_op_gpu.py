@@ -286,6 +286,28 @@ def test_tail_guard_aligned():
                 assert_bit_equal(host(full[k])[n:], inp[k][n:], f'{tag} n={n} {k} tail')
 
 
+def test_stride_loop_when_tiles_exceed_the_grid_cap():
+    """Tensors with more tiles than the launch cap are covered by the kernels' stride loop; with
+    the cap lowered to a handful of workgroups the same code runs on a small input."""
+    lib = _lib.load()
+    prev = lib.toa_adam_set_max_grid(7)
+    try:
+        for tag in ('f32', 'f64'):
+            route = ROUTES['module'](tag)
+            check_all_seven(route, rand(NP[tag], 100_003, 17), HYPERS[1], f'{tag}/cap=7')
+        sizes = [5000, 3, 70_001, 256]
+        hs = [rand(np.float32, n, 60 + k) for k, n in enumerate(sizes)]
+        ds = [{k: dev(a) for k, a in h.items()} for h in hs]
+        adam_op.forward_multi_([d['updates'] for d in ds], [d['mu'] for d in ds],
+                               [d['nu'] for d in ds], *HYPERS[0])
+        for k, (h, d) in enumerate(zip(hs, ds)):
+            eu, em, ev = O.forward_inplace(h['updates'], h['mu'], h['nu'], *HYPERS[0])
+            assert_parity(host(d['updates']), eu, f'multi cap=7 updates[{k}]')
+            assert_parity(host(d['nu']), ev, f'multi cap=7 nu[{k}]')
+    finally:
+        lib.toa_adam_set_max_grid(prev)
+
+
 def test_empty_tensors():
     for dt in (torch.float32, torch.float64):
         e = torch.empty(0, device='cuda', dtype=dt)

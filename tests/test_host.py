@@ -22,7 +22,7 @@ HEADER = os.path.join(REPO, 'include', 'toa_adam.h')
 def declared_functions():
     text = open(HEADER).read()
     text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
-    decls = re.findall(r'TOA_API\s+(?:const\s+char\s*\*|int)\s*(\w+)\s*\(([^;]*?)\)\s*;', text,
+    decls = re.findall(r'TOA_API\s+(?:const\s+char\s*\*|int|unsigned)\s*(\w+)\s*\(([^;]*?)\)\s*;', text,
                        flags=re.S)
     return {name: [a.strip() for a in args.split(',')] if args.strip() != 'void' else []
             for name, args in decls}
@@ -34,7 +34,7 @@ def test_header_declares_the_expected_surface():
                'backward_nu', 'backward_updates'}
     want = {f'toa_adam_{s}' for s in singles} | {f'toa_adam_{s}_multi' for s in singles}
     want |= {'toa_adam_abi_version', 'toa_adam_error_string', 'toa_adam_set_waves_per_cu',
-             'toa_adam_fused_step', 'toa_adam_fused_step_multi'}
+             'toa_adam_fused_step', 'toa_adam_fused_step_multi', 'toa_adam_set_max_grid'}
     assert names == want
 
 
@@ -86,6 +86,14 @@ def test_waves_knob_round_trip():
     first = lib.toa_adam_set_waves_per_cu(16)
     assert lib.toa_adam_set_waves_per_cu(99) == 16  # out of range restores the per-op defaults
     assert lib.toa_adam_set_waves_per_cu(first) == 0
+
+
+def test_max_grid_knob_round_trip():
+    lib = _lib.load()
+    default = lib.toa_adam_set_max_grid(64)
+    assert default == 1 << 25
+    assert lib.toa_adam_set_max_grid(0) == 64  # 0 restores the default
+    assert lib.toa_adam_set_max_grid(default) == default
 
 
 def test_python_surface_names_and_keywords():

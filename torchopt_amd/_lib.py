@@ -32,6 +32,7 @@ _i = ctypes.c_int
 # name -> argtypes; every function returns int except the two noted below.
 SIGNATURES = {
     'toa_adam_set_waves_per_cu': [_i],
+    'toa_adam_set_max_grid': [ctypes.c_uint],
     'toa_adam_forward_inplace': [_i, _vp, _vp, _vp, _sz, _d, _d, _d, _d, _u64, _vp],
     'toa_adam_forward_mu': [_i, _vp, _vp, _sz, _d, _vp, _vp],
     'toa_adam_forward_nu': [_i, _vp, _vp, _sz, _d, _vp, _vp],
@@ -85,7 +86,7 @@ def load() -> ctypes.CDLL:
             raise ImportError(f'{LIB_PATH}: ABI version {got}, expected {ABI_VERSION}; rebuild it')
         for name, argtypes in SIGNATURES.items():
             fn = getattr(lib, name)
-            fn.restype = _i
+            fn.restype = ctypes.c_uint if name == 'toa_adam_set_max_grid' else _i
             fn.argtypes = argtypes
         _lib = lib
     return _lib

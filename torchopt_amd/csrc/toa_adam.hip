@@ -23,7 +23,7 @@ using namespace toa;
 // Launch shape of the streaming kernels (see adam_kernels.hpp).
 constexpr int kUnroll = 1;           // one 16-byte access per lane per stream
 constexpr bool kNonTemporal = true;  // every array is touched once
-constexpr unsigned kMaxGrid = 1u << 25;  // workgroups per launch; larger tensors stride
+constexpr unsigned kMaxGrid = 1u << 25;  // default cap on workgroups per launch
 constexpr int kLdsPerCU = 160 * 1024;    // gfx950
 // The multi-tensor kernel spends three dependent scalar loads finding its tensor
 // before any memory traffic starts; a few more resident waves cover that.
@@ -58,8 +58,13 @@ unsigned lds_reservation(int extra_waves = 0) {
     return (unsigned)((kLdsPerCU / w) & ~1023);
 }
 
+// Workgroups per launch are capped; a tensor with more tiles than the cap is covered by the
+// kernels' stride loop.  The cap is adjustable so that path can be exercised on small inputs.
+std::atomic<unsigned> g_max_grid{kMaxGrid};
+
 unsigned grid_for(size_t num_tiles) {
-    return (unsigned)(num_tiles < kMaxGrid ? num_tiles : kMaxGrid);
+    const unsigned cap = g_max_grid.load(std::memory_order_relaxed);
+    return (unsigned)(num_tiles < cap ? num_tiles : cap);
 }
 
 struct HostScalars {
@@ -218,6 +223,13 @@ int toa_adam_abi_version(void) { return 1; }
 int toa_adam_set_waves_per_cu(int waves) {
     const int prev = waves_override();
     g_waves_override.store(waves >= 1 && waves <= 32 ? waves : 0, std::memory_order_relaxed);
+    return prev;
+}
+
+unsigned toa_adam_set_max_grid(unsigned workgroups) {
+    const unsigned prev = g_max_grid.load(std::memory_order_relaxed);
+    g_max_grid.store(workgroups >= 1 && workgroups <= kMaxGrid ? workgroups : kMaxGrid,
+                     std::memory_order_relaxed);
     return prev;
 }
 
