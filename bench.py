@@ -82,7 +82,7 @@ CONFIGS = {
     0: dict(name='config0: fused forward_ in place, 1 048 576 float32 elements, count=10',
             dtype='f32', n=1 << 20, eps_root=0.0, count=10),
     1: dict(name='config1: forward mu/nu/updates + backward updates/nu/mu over the MAML pytree '
-                 '(10 float32 tensors, 32 645 elements), six multi-tensor launches per step',
+                 '(10 float32 tensors, 32 645 elements), one multi-tensor pass per direction',
             dtype='f32', shapes=maml_shapes(), eps_root=1e-8, count=5, differentiable=True),
     2: dict(name='config2: fused forward_ in place, 268 435 456 float32 elements '
                  '(1 GiB per state array), count=1000',
@@ -154,7 +154,7 @@ def run_gpu(cfg_id, steps, warmup):
             if rc:
                 raise RuntimeError(lib.toa_adam_error_string(rc).decode())
 
-        def step():
+        def six_launch_step():
             check(lib.toa_adam_forward_mu_multi(code, num, a_up, a_mu, ns, B1, o[0], sptr))
             check(lib.toa_adam_forward_nu_multi(code, num, a_up, a_nu, ns, B2, o[1], sptr))
             check(lib.toa_adam_forward_updates_multi(code, num, o[0], o[1], ns, B1, B2, EPS,
@@ -163,6 +163,13 @@ def run_gpu(cfg_id, steps, warmup):
                                                       eps_root, None, count, o[3], o[4], sptr))
             check(lib.toa_adam_backward_nu_multi(code, num, a_dv, a_up, ns, B2, o[5], o[6], sptr))
             check(lib.toa_adam_backward_mu_multi(code, num, a_dm, ns, B1, o[7], o[8], sptr))
+
+        def step():  # the whole differentiable step: one pass forward, one pass backward
+            check(lib.toa_adam_forward_all_multi(code, num, a_up, a_mu, a_nu, ns, B1, B2, EPS,
+                                                 eps_root, None, count, o[0], o[1], o[2], sptr))
+            check(lib.toa_adam_backward_all_multi(code, num, a_du, o[2], o[0], a_up, a_dm, a_dv,
+                                                  ns, B1, B2, eps_root, None, count, o[3], o[4],
+                                                  o[5], sptr))
 
         ptrs = [[t.data_ptr() for t in x] for x in (ups, mus, nus, d_u, d_m, d_v, *outs)]
 
@@ -178,18 +185,23 @@ def run_gpu(cfg_id, steps, warmup):
                 lib.toa_adam_backward_nu(code, p[5], p[0], n, B2, p[11], p[12], sptr)
                 lib.toa_adam_backward_mu(code, p[4], n, B1, p[13], p[14], sptr)
 
-        for _ in range(warmup):
-            per_tensor_step()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            per_tensor_step()
-        torch.cuda.synchronize()
-        per_leaf_ms = (time.perf_counter() - t0) * 1e3 / steps
-        bytes_per_elem = sum(BYTES_PER_ELEM[k] for k in (
-            'forward_mu', 'forward_nu', 'forward_updates', 'backward_updates', 'backward_nu',
-            'backward_mu')) * esize
-        extra = {'tensors': num, 'launches_per_step': 6,
+        def wall_ms(fn):
+            for _ in range(warmup):
+                fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                fn()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) * 1e3 / steps
+
+        per_leaf_ms = wall_ms(per_tensor_step)
+        six_ms = wall_ms(six_launch_step)
+        # the one-pass pair streams 24 + 36 bytes per float32 element (3R+3W, 6R+3W); the
+        # separate ops stream 84
+        bytes_per_elem = (6 + 9) * esize
+        extra = {'tensors': num, 'launches_per_step': 2,
+                 'six_list_launches_ms_per_step': round(six_ms, 5),
                  'per_leaf_loop_ms_per_step': round(per_leaf_ms, 5),
                  'per_leaf_loop_launches_per_step': 6 * num}
     elif 'shapes' in cfg:

@@ -163,6 +163,50 @@ TOA_API int toa_adam_backward_updates_multi(int dtype, size_t num_tensors, const
                                     void *const *dnew_mu_out, void *const *dnew_nu_out,
                                     void *stream);
 
+/* ---- whole differentiable step in two passes ----------------------------------
+ * The differentiable branch of the reference runs three forward ops and three
+ * backward ops per leaf (/root/reference/torchopt/accelerated_op/adam_op.py:167-180
+ * and :52-60, :78-86, :104-121).  These entry points do each direction in one pass
+ * with results bit-identical to the separate ops:
+ *   forward_all   new_mu, new_nu, new_updates from one read of updates, mu, nu
+ *                 (= forward_mu, forward_nu, forward_updates; 24 instead of 36 bytes
+ *                 per float32 element);
+ *   backward_all  d(updates), d(mu), d(nu) from d(new_updates) and the saved
+ *                 new_updates, new_mu, updates (= backward_updates, then
+ *                 backward_mu and backward_nu, with the additions autograd performs
+ *                 between them).  dnew_mu / dnew_nu are the gradients reaching
+ *                 new_mu / new_nu from outside the step; either may be NULL (for
+ *                 the list form: the whole list pointer NULL), meaning none.
+ * No single counterpart in the reference. */
+TOA_API int toa_adam_forward_all(int dtype, const void *updates, const void *mu, const void *nu,
+                                 size_t n, double b1, double b2, double eps, double eps_root,
+                                 uint64_t count, void *new_mu, void *new_nu, void *new_updates,
+                                 void *stream);
+
+TOA_API int toa_adam_forward_all_multi(int dtype, size_t num_tensors,
+                                       const void *const *updates, const void *const *mu,
+                                       const void *const *nu, const size_t *n, double b1,
+                                       double b2, double eps, double eps_root,
+                                       const uint64_t *counts, uint64_t count_all,
+                                       void *const *new_mu, void *const *new_nu,
+                                       void *const *new_updates, void *stream);
+
+TOA_API int toa_adam_backward_all(int dtype, const void *dnew_updates, const void *new_updates,
+                                  const void *new_mu, const void *updates, const void *dnew_mu,
+                                  const void *dnew_nu, size_t n, double b1, double b2,
+                                  double eps_root, uint64_t count, void *dupdates, void *dmu,
+                                  void *dnu, void *stream);
+
+TOA_API int toa_adam_backward_all_multi(int dtype, size_t num_tensors,
+                                        const void *const *dnew_updates,
+                                        const void *const *new_updates,
+                                        const void *const *new_mu, const void *const *updates,
+                                        const void *const *dnew_mu, const void *const *dnew_nu,
+                                        const size_t *n, double b1, double b2, double eps_root,
+                                        const uint64_t *counts, uint64_t count_all,
+                                        void *const *dupdates, void *const *dmu,
+                                        void *const *dnu, void *stream);
+
 /* ---- fused optimizer step ------------------------------------------------
  * The classic in-place step of `Adam(..., use_accelerated_op=True).step()` in
  * one pass over memory: the Adam update (as toa_adam_forward_inplace), then

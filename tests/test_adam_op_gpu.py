@@ -308,6 +308,49 @@ def test_stride_loop_when_tiles_exceed_the_grid_cap():
         lib.toa_adam_set_max_grid(prev)
 
 
+@pytest.mark.parametrize('tag', ['f32', 'f64'])
+def test_one_pass_forward_and_backward_against_oracle_chain(tag):
+    """forward_all / backward_all through the module and through the raw C ABI, against the
+    oracle's separate functions composed with the additions autograd performs between them."""
+    dtype = NP[tag]
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    for k, n in enumerate([1, 5, 257, 4099, 300_001]):
+        b1, b2, eps, er, c = HYPERS[k % 3]
+        inp = rand(dtype, n, 900 + n)
+        g = {key: dev(a) for key, a in inp.items()}
+        e_mu, e_nu = O.forward_mu(inp['updates'], inp['mu'], b1), O.forward_nu(inp['updates'],
+                                                                              inp['nu'], b2)
+        e_u = O.forward_updates(e_mu, e_nu, b1, b2, eps, er, c)
+        new_mu, new_nu, new_u = adam_op.forward_all(g['updates'], g['mu'], g['nu'], b1, b2, eps,
+                                                    er, c)
+        assert_parity(host(new_mu), e_mu, f'n={n} forward_all new_mu')
+        assert_parity(host(new_nu), e_nu, f'n={n} forward_all new_nu')
+        assert_parity(host(new_u), e_u, f'n={n} forward_all new_updates')
+        bm, bv = O.backward_updates(inp['dupdates'], e_u, e_mu, b1, b2, er, c)
+        for has_m, has_v in [(False, False), (True, False), (False, True), (True, True)]:
+            tot_m = inp['dmu'] + bm if has_m else bm
+            tot_v = inp['dnu'] + bv if has_v else bv
+            du1, dmu = O.backward_mu(tot_m, b1)
+            du2, dnu = O.backward_nu(tot_v, inp['updates'], b2)
+            got = adam_op.backward_all(g['dupdates'], g['dmu'] if has_m else None,
+                                       g['dnu'] if has_v else None, new_u, new_mu, g['updates'],
+                                       b1, b2, er, c)
+            label = f'n={n} backward_all dm={has_m} dv={has_v}'
+            assert_parity(host(got[0]), du1 + du2, f'{label} dupdates')
+            assert_parity(host(got[1]), dmu, f'{label} dmu')
+            assert_parity(host(got[2]), dnu, f'{label} dnu')
+            outs = [torch.empty_like(new_mu) for _ in range(3)]
+            rc = lib.toa_adam_backward_all(
+                CODE[tag], g['dupdates'].data_ptr(), new_u.data_ptr(), new_mu.data_ptr(),
+                g['updates'].data_ptr(), g['dmu'].data_ptr() if has_m else None,
+                g['dnu'].data_ptr() if has_v else None, n, b1, b2, er, c, outs[0].data_ptr(),
+                outs[1].data_ptr(), outs[2].data_ptr(), stream)
+            assert rc == 0
+            for a, b in zip(outs, got):
+                assert torch.equal(a, b), f'{label}: C ABI and module disagree'
+
+
 def test_empty_tensors():
     for dt in (torch.float32, torch.float64):
         e = torch.empty(0, device='cuda', dtype=dt)

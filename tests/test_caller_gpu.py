@@ -166,6 +166,44 @@ def test_differentiable_branch_matches_per_leaf_adam_op():
             assert torch.equal(a.grad, b.grad), f'leaf {k} grad wrt {what}'
 
 
+@pytest.mark.parametrize('which', ['updates_only', 'updates_and_mu', 'ragged'])
+def test_differentiable_branch_with_missing_outside_gradients(which):
+    """Only some outputs feed the loss: the one-pass backward must give what the per-leaf chain
+    gives when autograd has nothing to add at new_mu / new_nu (for all leaves, or for some)."""
+    shapes = [(7, 5), (300,), (3, 4, 5), ()]
+    rng = np.random.default_rng(21)
+    data = [[np.asarray(rng.standard_normal(s), dtype=np.float64) for _ in range(3)]
+            for s in shapes]
+    cots = [[np.asarray(rng.standard_normal(s), dtype=np.float64) for _ in range(3)]
+            for s in shapes]
+
+    def leaves():
+        return [[dev(a).requires_grad_(True) for a in (g, 0.1 * m, np.abs(0.01 * v) + 1e-3)]
+                for g, m, v in data]
+
+    def loss_terms(outs):
+        terms = []
+        for k, (new_mu, new_nu, new_u) in enumerate(outs):
+            terms.append((new_u * dev(cots[k][2])).sum())
+            if which == 'updates_and_mu' or (which == 'ragged' and k % 2 == 0):
+                terms.append((new_mu * dev(cots[k][0])).sum())
+            if which == 'ragged' and k == 1:
+                terms.append((new_nu * dev(cots[k][1])).sum())
+        return sum(terms)
+
+    single = leaves()
+    op = AdamOp(B1, B2, EPS, eps_root=1e-8, inplace=False)
+    loss_terms([op(m, v, g, 3) for g, m, v in single]).backward()
+    multi = leaves()
+    mop = MultiAdamOp(B1, B2, EPS, eps_root=1e-8, inplace=False)
+    new_mu, new_nu, new_u = mop([x[1] for x in multi], [x[2] for x in multi],
+                                [x[0] for x in multi], 3)
+    loss_terms(list(zip(new_mu, new_nu, new_u))).backward()
+    for k in range(len(shapes)):
+        for a, b, what in zip(single[k], multi[k], ('updates', 'mu', 'nu')):
+            assert_bit_equal(host(b.grad), host(a.grad), f'{which} leaf {k} grad wrt {what}')
+
+
 def test_meta_step_through_the_transformation():
     """A MAML-style inner step: params' = params - lr * adam(grad); the outer loss
     differentiates through the update, the moments and the step."""

@@ -50,6 +50,13 @@ SIGNATURES = {
     'toa_adam_backward_nu_multi': [_i, _sz, _vpp, _vpp, _szp, _d, _vpp, _vpp, _vp],
     'toa_adam_backward_updates_multi': [_i, _sz, _vpp, _vpp, _vpp, _szp, _d, _d, _d, _u64p, _u64,
                                         _vpp, _vpp, _vp],
+    'toa_adam_forward_all': [_i, _vp, _vp, _vp, _sz, _d, _d, _d, _d, _u64, _vp, _vp, _vp, _vp],
+    'toa_adam_forward_all_multi': [_i, _sz, _vpp, _vpp, _vpp, _szp, _d, _d, _d, _d, _u64p, _u64,
+                                   _vpp, _vpp, _vpp, _vp],
+    'toa_adam_backward_all': [_i, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _d, _d, _d, _u64, _vp, _vp,
+                              _vp, _vp],
+    'toa_adam_backward_all_multi': [_i, _sz, _vpp, _vpp, _vpp, _vpp, _vpp, _vpp, _szp, _d, _d, _d,
+                                    _u64p, _u64, _vpp, _vpp, _vpp, _vp],
     'toa_adam_fused_step': [_i, _vp, _vp, _vp, _vp, _sz, _d, _d, _d, _d, _u64, _d, _i, _i, _vp],
     'toa_adam_fused_step_multi': [_i, _sz, _vpp, _vpp, _vpp, _vpp, _szp, _d, _d, _d, _d, _u64p,
                                   _u64, _d, _i, _i, _vp],

@@ -118,69 +118,53 @@ class MultiAdamOp:
 
     The reference applies `AdamOp` leaf by leaf from Python
     (/root/reference/torchopt/transform/scale_by_adam.py:325-332): one launch, and on the
-    differentiable path three autograd nodes, per leaf.  This callable takes the flattened tree
-    at once: the in-place branch is one `forward_multi_` call, and the differentiable branch is
-    three autograd Functions whose forward and backward each make one multi-tensor call, so a
-    tree of any size costs six launches per step instead of six per leaf.  Results are
-    bit-identical to the per-leaf `AdamOp`.
+    differentiable path three autograd nodes with three forward and three backward launches,
+    per leaf.  This callable takes the flattened tree at once: the in-place branch is one
+    `forward_multi_` call, and the differentiable branch is ONE autograd Function whose forward
+    (`forward_all_multi`) and backward (`backward_all_multi`) are one multi-tensor pass each, so
+    a tree of any size costs two launches per step instead of six per leaf, and each direction
+    reads its operands once.  Values and gradients are bit-identical to the per-leaf `AdamOp`.
 
     All lists must be free of ``None`` and live on one device with one dtype; the caller groups
     leaves accordingly.  `counts` is one step number for all leaves or one per leaf (ints or
     0-dim integer tensors).
     """
 
-    class MuOp(torch.autograd.Function):
-        """``new_mu[k] = b1*mu[k] + (1-b1)*updates[k]`` for every k."""
-
-        @staticmethod
-        def forward(ctx: Any, b1: float, k: int, *tensors: torch.Tensor):
-            ctx.save_for_backward(*tensors)
-            ctx.b1, ctx.k = b1, k
-            return tuple(adam_op.forward_mu_multi(list(tensors[:k]), list(tensors[k:]), b1))
-
-        @staticmethod
-        def backward(ctx: Any, *dmu: torch.Tensor):
-            saved, k = ctx.saved_tensors, ctx.k
-            dupdates, dmu_in = adam_op.backward_mu_multi(
-                list(dmu), list(saved[:k]), list(saved[k:]), ctx.b1)
-            return (None, None, *dupdates, *dmu_in)
-
-    class NuOp(torch.autograd.Function):
-        """``new_nu[k] = b2*nu[k] + (1-b2)*updates[k]**2`` for every k."""
-
-        @staticmethod
-        def forward(ctx: Any, b2: float, k: int, *tensors: torch.Tensor):
-            ctx.save_for_backward(*tensors)
-            ctx.b2, ctx.k = b2, k
-            return tuple(adam_op.forward_nu_multi(list(tensors[:k]), list(tensors[k:]), b2))
-
-        @staticmethod
-        def backward(ctx: Any, *dnu: torch.Tensor):
-            saved, k = ctx.saved_tensors, ctx.k
-            dupdates, dnu_in = adam_op.backward_nu_multi(
-                list(dnu), list(saved[:k]), list(saved[k:]), ctx.b2)
-            return (None, None, *dupdates, *dnu_in)
-
-    class UpdatesOp(torch.autograd.Function):
-        """Step directions for every leaf; backward is the reference's hand-derived formula."""
+    class StepOp(torch.autograd.Function):
+        """(updates, mu, nu) -> (new_mu, new_nu, new_updates) for every leaf."""
 
         @staticmethod
         def forward(ctx: Any, hyper: tuple, k: int, *tensors: torch.Tensor):
             b1, b2, eps, eps_root, counts = hyper
-            new_updates = adam_op.forward_updates_multi(
-                list(tensors[:k]), list(tensors[k:]), b1, b2, eps, eps_root, counts)
-            ctx.save_for_backward(*new_updates, *tensors)
+            updates = list(tensors[:k])
+            new_mu, new_nu, new_updates = adam_op.forward_all_multi(
+                updates, list(tensors[k:2 * k]), list(tensors[2 * k:]), b1, b2, eps, eps_root,
+                counts)
+            ctx.save_for_backward(*new_updates, *new_mu, *updates)
             ctx.hyper, ctx.k = hyper, k
-            return tuple(new_updates)
+            ctx.set_materialize_grads(False)  # a missing gradient must stay missing, see below
+            return (*new_mu, *new_nu, *new_updates)
 
         @staticmethod
-        def backward(ctx: Any, *dupdates: torch.Tensor):
+        def backward(ctx: Any, *grads: torch.Tensor | None):
             saved, k = ctx.saved_tensors, ctx.k
             b1, b2, _eps, eps_root, counts = ctx.hyper
-            dnew_mu, dnew_nu = adam_op.backward_updates_multi(
-                list(dupdates), list(saved[:k]), list(saved[k:2 * k]), list(saved[2 * k:]),
-                b1, b2, eps_root, counts)
-            return (None, None, *dnew_mu, *dnew_nu)
+            new_updates, new_mu, updates = saved[:k], saved[k:2 * k], saved[2 * k:]
+
+            def outside(gs):
+                # Gradients reaching new_mu / new_nu from outside the step.  None at all: the
+                # kernel skips the addition, as autograd would.  Some: members without one get
+                # -0.0, the exact identity of IEEE addition (x + -0.0 is x for every x, signed
+                # zeros included), so they too come out as if nothing had been added.
+                if all(g is None for g in gs):
+                    return None
+                return [torch.full_like(m, -0.0) if g is None else g for g, m in zip(gs, new_mu)]
+
+            d_u = [torch.zeros_like(m) if g is None else g for g, m in zip(grads[2 * k:], new_mu)]
+            dupdates, dmu, dnu = adam_op.backward_all_multi(
+                d_u, outside(grads[:k]), outside(grads[k:2 * k]), list(new_updates),
+                list(new_mu), list(updates), b1, b2, eps_root, counts)
+            return (None, None, *dupdates, *dmu, *dnu)
 
     def __init__(
         self,
@@ -207,8 +191,6 @@ class MultiAdamOp:
             adam_op.forward_multi_(updates, mus, nus, self.b1, self.b2, self.eps, self.eps_root,
                                    counts)
             return mus, nus, updates
-        new_mus = self.MuOp.apply(self.b1, k, *updates, *mus)
-        new_nus = self.NuOp.apply(self.b2, k, *updates, *nus)
         hyper = (self.b1, self.b2, self.eps, self.eps_root, counts)
-        new_updates = self.UpdatesOp.apply(hyper, k, *new_mus, *new_nus)
-        return list(new_mus), list(new_nus), list(new_updates)
+        out = self.StepOp.apply(hyper, k, *updates, *mus, *nus)
+        return list(out[:k]), list(out[k:2 * k]), list(out[2 * k:])

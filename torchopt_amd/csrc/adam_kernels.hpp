@@ -299,6 +299,60 @@ struct BackwardUpdates {
     }
 };
 
+// The whole differentiable forward of one step in one pass: what forward_mu, forward_nu and
+// forward_updates produce, from one read of updates, mu and nu (24 instead of 36 bytes per
+// float32 element, one launch instead of three).  Same expressions as ForwardInplace, written
+// to fresh outputs.  Slots: 0 updates, 1 mu, 2 nu, 3 new_mu, 4 new_nu, 5 new_updates.
+template <typename T>
+struct ForwardAll {
+    static constexpr int NIN = 3, NOUT = 3, NPTR = 6;
+    static constexpr int kWavesPerCU = 24;
+    __device__ static constexpr int out_slot(int j) { return NIN + j; }
+    T b1, b2, c1, c2, eps, eps_root;
+    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
+        const T g = in[0], m = in[1], v = in[2];
+        const T m1 = b1 * m + (1 - b1) * g;
+        const T v1 = b2 * v + (1 - b2) * g * g;
+        const T mh = m1 * c1;
+        const T vh = v1 * c2;
+        out[0] = m1;
+        out[1] = v1;
+        out[2] = mh / (toa_sqrt(vh + eps_root) + eps);
+    }
+};
+
+// The whole backward of that step in one pass: backward_updates, the two sums autograd would
+// form (gradient arriving at new_mu / new_nu from elsewhere plus the one from the update), then
+// backward_mu and backward_nu and the sum of their two contributions to d(updates) -- each
+// still rounded on its own, so the result equals the three separate passes plus autograd's
+// additions bit for bit.  HAS_DM / HAS_DV say whether an outside gradient for new_mu / new_nu
+// exists; without one the sum is skipped, exactly as autograd skips it.
+// Slots: 0 d(new_updates), 1 new_updates, 2 new_mu, 3 updates, [d(new_mu)], [d(new_nu)],
+// then outputs d(updates), d(mu), d(nu).
+template <typename T, bool HAS_DM, bool HAS_DV>
+struct BackwardAll {
+    static constexpr int NIN = 4 + (HAS_DM ? 1 : 0) + (HAS_DV ? 1 : 0), NOUT = 3,
+                         NPTR = NIN + NOUT;
+    static constexpr int kWavesPerCU = 24;
+    __device__ static constexpr int out_slot(int j) { return NIN + j; }
+    T b1, b2, p1, q2;
+    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
+        const T d = in[0], u = in[1], m1 = in[2], g = in[3];
+        const T r = u / m1;
+        const T den = r * p1;
+        const bool zero = (m1 == 0);
+        T tot_m = zero ? T(0) : T(d * r);
+        T tot_v = zero ? T(0) : static_cast<T>(-d * u * den * 0.5 * q2 * den);
+        if constexpr (HAS_DM) tot_m = in[4] + tot_m;
+        if constexpr (HAS_DV) tot_v = in[HAS_DM ? 5 : 4] + tot_v;
+        const T du_from_mu = (1 - b1) * tot_m;
+        const T du_from_nu = 2 * (1 - b2) * g * tot_v;
+        out[0] = du_from_mu + du_from_nu;
+        out[1] = b1 * tot_m;
+        out[2] = b2 * tot_v;
+    }
+};
+
 // The classic optimizer step in one pass: the in-place Adam step followed by what
 // the reference chain does next with its result -- scale by -lr
 // (/root/reference/torchopt/transform/scale.py:93-98 via alias/utils.py:226) and

@@ -250,6 +250,65 @@ std::array<Tensor, 2> backwardUpdates(const Tensor &dupdates_in, const Tensor &u
     return {dmu_out, dnu_out};
 }
 
+// The differentiable step in one pass per direction (no single counterpart in the reference;
+// results equal forward_mu / forward_nu / forward_updates and the backward chain bit for bit).
+std::array<Tensor, 3> forwardAll(const Tensor &updates_in, const Tensor &mu, const Tensor &nu_in,
+                                 double b1, double b2, double eps, double eps_root,
+                                 size_t count) {
+    const char *name = "adamForwardAll";
+    size_t n;
+    const int code = gate(name, updates_in, {&mu, &nu_in}, &n);
+    requireDense(name, "mu", mu);
+    Tensor new_mu = at::empty_like(mu), new_nu = at::empty_like(mu), new_updates = at::empty_like(mu);
+    if (n) {
+        const Tensor updates = asLayoutOf(updates_in, mu);
+        const Tensor nu = asLayoutOf(nu_in, mu);
+        const OnDeviceOf dev(mu);
+        check(toa_adam_forward_all(code, updates.data_ptr(), mu.data_ptr(), nu.data_ptr(), n, b1,
+                                   b2, eps, eps_root, count, new_mu.data_ptr(), new_nu.data_ptr(),
+                                   new_updates.data_ptr(), dev.stream()),
+              name);
+    }
+    return {new_mu, new_nu, new_updates};
+}
+
+// dnew_mu / dnew_nu: gradients reaching new_mu / new_nu from outside the step, or None.
+std::array<Tensor, 3> backwardAll(const Tensor &dnew_updates_in,
+                                  const c10::optional<Tensor> &dnew_mu_in,
+                                  const c10::optional<Tensor> &dnew_nu_in,
+                                  const Tensor &new_updates_in, const Tensor &new_mu,
+                                  const Tensor &updates_in, double b1, double b2, double eps_root,
+                                  size_t count) {
+    const char *name = "adamBackwardAll";
+    size_t n;
+    const int code = gate(name, dnew_updates_in, {&new_updates_in, &new_mu, &updates_in}, &n);
+    requireDense(name, "new_mu", new_mu);
+    Tensor dupdates = at::empty_like(new_mu), dmu = at::empty_like(new_mu),
+           dnu = at::empty_like(new_mu);
+    if (n) {
+        const Tensor du = asLayoutOf(dnew_updates_in, new_mu);
+        const Tensor nu_ = asLayoutOf(new_updates_in, new_mu);
+        const Tensor up = asLayoutOf(updates_in, new_mu);
+        Tensor dm, dv;
+        for (auto pair : {std::make_pair(&dnew_mu_in, &dm), std::make_pair(&dnew_nu_in, &dv)}) {
+            if (!pair.first->has_value()) continue;
+            const Tensor &t = pair.first->value();
+            TORCH_CHECK(t.device() == new_mu.device() && t.scalar_type() == new_mu.scalar_type() &&
+                            (size_t)t.numel() == n,
+                        name, ": outside gradient does not match new_mu");
+            *pair.second = asLayoutOf(t, new_mu);
+        }
+        const OnDeviceOf dev(new_mu);
+        check(toa_adam_backward_all(code, du.data_ptr(), nu_.data_ptr(), new_mu.data_ptr(),
+                                    up.data_ptr(), dm.defined() ? dm.data_ptr() : nullptr,
+                                    dv.defined() ? dv.data_ptr() : nullptr, n, b1, b2, eps_root,
+                                    count, dupdates.data_ptr(), dmu.data_ptr(), dnu.data_ptr(),
+                                    dev.stream()),
+              name);
+    }
+    return {dupdates, dmu, dnu};
+}
+
 std::array<Tensor, 4> fusedStep(const Tensor &params, const Tensor &updates, const Tensor &mu,
                                 const Tensor &nu, double b1, double b2, double eps,
                                 double eps_root, size_t count, double lr, bool maximize,
@@ -496,6 +555,62 @@ std::tuple<TensorList, TensorList> backwardUpdatesMulti(
     return {dmu_out, dnu_out};
 }
 
+std::tuple<TensorList, TensorList, TensorList> forwardAllMulti(
+    const TensorList &updates, const TensorList &mu, const TensorList &nu, double b1, double b2,
+    double eps, double eps_root, const py::object &counts) {
+    const char *name = "adamForwardAllMulti";
+    TensorList new_mu = emptyLike(mu), new_nu = emptyLike(mu), new_updates = emptyLike(mu);
+    Lists l = gateLists(name, {&updates, &mu, &nu, &new_mu, &new_nu, &new_updates});
+    if (l.num) {
+        const Counts c = parseCounts(counts, l.num);
+        const OnDeviceOf dev(firstNonEmpty(mu));
+        check(toa_adam_forward_all_multi(l.code, l.num, l.ptr[0].data(), l.ptr[1].data(),
+                                         l.ptr[2].data(), l.n.data(), b1, b2, eps, eps_root,
+                                         c.data(), c.all, l.ptr[3].data(), l.ptr[4].data(),
+                                         l.ptr[5].data(), dev.stream()),
+              name);
+    }
+    return {new_mu, new_nu, new_updates};
+}
+
+// dnew_mu / dnew_nu: a list of outside gradients, or None when there are none at all (a list
+// may not mix tensors and None: the caller substitutes zeros for the missing members).
+std::tuple<TensorList, TensorList, TensorList> backwardAllMulti(
+    const TensorList &dnew_updates_in, const c10::optional<TensorList> &dnew_mu_in,
+    const c10::optional<TensorList> &dnew_nu_in, const TensorList &new_updates,
+    const TensorList &new_mu, const TensorList &updates, double b1, double b2, double eps_root,
+    const py::object &counts) {
+    const char *name = "adamBackwardAllMulti";
+    TensorList dupdates = emptyLike(new_mu), dmu = emptyLike(new_mu), dnu = emptyLike(new_mu);
+    const TensorList du = asLayoutOfEach(dnew_updates_in, new_mu, name);
+    Lists l = gateLists(name, {&du, &new_updates, &new_mu, &updates, &dupdates, &dmu, &dnu});
+    // outside gradients, brought to new_mu's layout; the (possibly copied) tensors live until
+    // the launch below has been enqueued
+    TensorList ext_m, ext_v;
+    std::vector<void *> pm, pv;
+    auto collect = [&](const c10::optional<TensorList> &in, TensorList *ext,
+                       std::vector<void *> *ptrs) {
+        if (!in.has_value()) return;
+        *ext = asLayoutOfEach(in.value(), new_mu, name);
+        Lists e = gateLists(name, {&new_mu, ext});
+        *ptrs = e.num ? e.ptr[1] : std::vector<void *>();
+    };
+    collect(dnew_mu_in, &ext_m, &pm);
+    collect(dnew_nu_in, &ext_v, &pv);
+    if (l.num) {
+        const Counts c = parseCounts(counts, l.num);
+        const OnDeviceOf dev(firstNonEmpty(new_mu));
+        check(toa_adam_backward_all_multi(
+                  l.code, l.num, l.ptr[0].data(), l.ptr[1].data(), l.ptr[2].data(),
+                  l.ptr[3].data(), dnew_mu_in.has_value() ? pm.data() : nullptr,
+                  dnew_nu_in.has_value() ? pv.data() : nullptr, l.n.data(), b1, b2, eps_root,
+                  c.data(), c.all, l.ptr[4].data(), l.ptr[5].data(), l.ptr[6].data(),
+                  dev.stream()),
+              name);
+    }
+    return {dupdates, dmu, dnu};
+}
+
 py::tuple fusedStepMulti(const py::object &params_o, const py::object &updates_o,
                          const py::object &mu_o, const py::object &nu_o, double b1, double b2,
                          double eps, double eps_root, const py::object &counts, double lr,
@@ -555,6 +670,20 @@ PYBIND11_MODULE(_C, mod) {
     m.def("backward_updates_multi", &backwardUpdatesMulti,
           "backward_updates over lists -> (dnew_mu, dnew_nu)", "dupdates"_a, "updates"_a,
           "new_mu"_a, "new_nu"_a, "b1"_a, "b2"_a, "eps_root"_a, "counts"_a);
+
+    // the differentiable step, one pass per direction
+    m.def("forward_all", &forwardAll,
+          "forward_mu, forward_nu and forward_updates in one pass -> [new_mu, new_nu, new_updates]",
+          "updates"_a, "mu"_a, "nu"_a, "b1"_a, "b2"_a, "eps"_a, "eps_root"_a, "count"_a);
+    m.def("backward_all", &backwardAll,
+          "backward of forward_all in one pass -> [dupdates, dmu, dnu]", "dnew_updates"_a,
+          "dnew_mu"_a, "dnew_nu"_a, "new_updates"_a, "new_mu"_a, "updates"_a, "b1"_a, "b2"_a,
+          "eps_root"_a, "count"_a);
+    m.def("forward_all_multi", &forwardAllMulti, "forward_all over lists", "updates"_a, "mu"_a,
+          "nu"_a, "b1"_a, "b2"_a, "eps"_a, "eps_root"_a, "counts"_a);
+    m.def("backward_all_multi", &backwardAllMulti, "backward_all over lists", "dnew_updates"_a,
+          "dnew_mu"_a, "dnew_nu"_a, "new_updates"_a, "new_mu"_a, "updates"_a, "b1"_a, "b2"_a,
+          "eps_root"_a, "counts"_a);
 
     // the classic in-place optimizer step in one pass
     m.def("fused_step_", &fusedStep,

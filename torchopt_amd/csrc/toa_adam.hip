@@ -12,6 +12,7 @@
 #include <atomic>
 #include <cmath>
 #include <cstdlib>
+#include <type_traits>
 #include <vector>
 
 #include "adam_kernels.hpp"
@@ -191,6 +192,64 @@ T *mut(const void *p) {
             return TOA_EDTYPE;                    \
     }
 
+#define CPP(x) reinterpret_cast<const void *const *>(x)
+
+// Calls f with two std::bool_constant tags for the run-time flags.
+template <class F>
+int with_flags(bool dm, bool dv, F f) {
+    if (dm) return dv ? f(std::true_type{}, std::true_type{}) : f(std::true_type{}, std::false_type{});
+    return dv ? f(std::false_type{}, std::true_type{}) : f(std::false_type{}, std::false_type{});
+}
+
+template <typename T, bool HAS_DM, bool HAS_DV>
+int backward_all_single(const void *dnew_updates, const void *new_updates, const void *new_mu,
+                        const void *updates, const void *dnew_mu, const void *dnew_nu, size_t n,
+                        double b1, double b2, const HostScalars &s, void *dupdates, void *dmu,
+                        void *dnu, void *stream) {
+    using Op = BackwardAll<T, HAS_DM, HAS_DV>;
+    const Op op{(T)b1, (T)b2, (T)s.p1, (T)s.q2};
+    T *p[Op::NPTR];
+    int k = 0;
+    p[k++] = mut<T>(dnew_updates);
+    p[k++] = mut<T>(new_updates);
+    p[k++] = mut<T>(new_mu);
+    p[k++] = mut<T>(updates);
+    if (HAS_DM) p[k++] = mut<T>(dnew_mu);
+    if (HAS_DV) p[k++] = mut<T>(dnew_nu);
+    p[k++] = (T *)dupdates;
+    p[k++] = (T *)dmu;
+    p[k++] = (T *)dnu;
+    T *const(&cp)[Op::NPTR] = p;
+    return launch_single<T>(op, cp, n, stream);
+}
+
+template <typename T, bool HAS_DM, bool HAS_DV>
+int backward_all_multi(size_t num, const void *const *dnew_updates,
+                       const void *const *new_updates, const void *const *new_mu,
+                       const void *const *updates, const void *const *dnew_mu,
+                       const void *const *dnew_nu, const size_t *n, double b1, double b2,
+                       double eps_root, const uint64_t *counts, uint64_t count_all,
+                       void *const *dupdates, void *const *dmu, void *const *dnu, void *stream) {
+    using Op = BackwardAll<T, HAS_DM, HAS_DV>;
+    const void *const *lists[Op::NPTR];
+    int k = 0;
+    lists[k++] = dnew_updates;
+    lists[k++] = new_updates;
+    lists[k++] = new_mu;
+    lists[k++] = updates;
+    if (HAS_DM) lists[k++] = dnew_mu;
+    if (HAS_DV) lists[k++] = dnew_nu;
+    lists[k++] = CPP(dupdates);
+    lists[k++] = CPP(dmu);
+    lists[k++] = CPP(dnu);
+    const void *const *const(&cl)[Op::NPTR] = lists;
+    auto make = [&](uint64_t c) {
+        const HostScalars s = host_scalars(b1, b2, eps_root, c);
+        return Op{(T)b1, (T)b2, (T)s.p1, (T)s.q2};
+    };
+    return launch_multi<T, Op>(make, num, cl, n, counts, count_all, stream);
+}
+
 // every element type the reference CPU op serves
 #define TOA_DISPATCH_ALL(dtype, ...)              \
     switch (dtype) {                              \
@@ -316,7 +375,6 @@ int toa_adam_backward_updates(int dtype, const void *dupdates, const void *updat
 
 // ---- multi-tensor -----------------------------------------------------------
 
-#define CPP(x) reinterpret_cast<const void *const *>(x)
 
 int toa_adam_forward_inplace_multi(int dtype, size_t num_tensors, void *const *updates,
                                    void *const *mu, void *const *nu, const size_t *n, double b1,
@@ -404,6 +462,69 @@ int toa_adam_backward_updates_multi(int dtype, size_t num_tensors, const void *c
         };
         return launch_multi<T, BackwardUpdates<T>>(make, num_tensors, lists, n, counts,
                                                    count_all, stream);
+    });
+}
+
+// ---- whole differentiable step: forward in one pass, backward in one pass -------------------
+
+int toa_adam_forward_all(int dtype, const void *updates, const void *mu, const void *nu, size_t n,
+                         double b1, double b2, double eps, double eps_root, uint64_t count,
+                         void *new_mu, void *new_nu, void *new_updates, void *stream) {
+    const HostScalars s = host_scalars(b1, b2, eps_root, count);
+    TOA_DISPATCH_ALL(dtype, [&] {
+        const ForwardAll<T> op{(T)b1, (T)b2, (T)s.c1, (T)s.c2, (T)eps, (T)eps_root};
+        T *const p[6] = {mut<T>(updates), mut<T>(mu), mut<T>(nu),
+                         (T *)new_mu,     (T *)new_nu, (T *)new_updates};
+        return launch_single<T>(op, p, n, stream);
+    });
+}
+
+int toa_adam_forward_all_multi(int dtype, size_t num_tensors, const void *const *updates,
+                               const void *const *mu, const void *const *nu, const size_t *n,
+                               double b1, double b2, double eps, double eps_root,
+                               const uint64_t *counts, uint64_t count_all, void *const *new_mu,
+                               void *const *new_nu, void *const *new_updates, void *stream) {
+    TOA_DISPATCH_ALL(dtype, [&] {
+        const void *const *const lists[6] = {updates,     mu,          nu,
+                                             CPP(new_mu), CPP(new_nu), CPP(new_updates)};
+        auto make = [&](uint64_t c) {
+            const HostScalars s = host_scalars(b1, b2, eps_root, c);
+            return ForwardAll<T>{(T)b1, (T)b2, (T)s.c1, (T)s.c2, (T)eps, (T)eps_root};
+        };
+        return launch_multi<T, ForwardAll<T>>(make, num_tensors, lists, n, counts, count_all,
+                                              stream);
+    });
+}
+
+int toa_adam_backward_all(int dtype, const void *dnew_updates, const void *new_updates,
+                          const void *new_mu, const void *updates, const void *dnew_mu,
+                          const void *dnew_nu, size_t n, double b1, double b2, double eps_root,
+                          uint64_t count, void *dupdates, void *dmu, void *dnu, void *stream) {
+    const HostScalars s = host_scalars(b1, b2, eps_root, count);
+    const bool dm = dnew_mu != nullptr, dv = dnew_nu != nullptr;
+    TOA_DISPATCH_ALL(dtype, [&] {
+        return with_flags(dm, dv, [&](auto DM, auto DV) {
+            return backward_all_single<T, decltype(DM)::value, decltype(DV)::value>(
+                dnew_updates, new_updates, new_mu, updates, dnew_mu, dnew_nu, n, b1, b2, s,
+                dupdates, dmu, dnu, stream);
+        });
+    });
+}
+
+int toa_adam_backward_all_multi(int dtype, size_t num_tensors, const void *const *dnew_updates,
+                                const void *const *new_updates, const void *const *new_mu,
+                                const void *const *updates, const void *const *dnew_mu,
+                                const void *const *dnew_nu, const size_t *n, double b1,
+                                double b2, double eps_root, const uint64_t *counts,
+                                uint64_t count_all, void *const *dupdates, void *const *dmu,
+                                void *const *dnu, void *stream) {
+    const bool dm = dnew_mu != nullptr, dv = dnew_nu != nullptr;
+    TOA_DISPATCH_ALL(dtype, [&] {
+        return with_flags(dm, dv, [&](auto DM, auto DV) {
+            return backward_all_multi<T, decltype(DM)::value, decltype(DV)::value>(
+                num_tensors, dnew_updates, new_updates, new_mu, updates, dnew_mu, dnew_nu, n, b1,
+                b2, eps_root, counts, count_all, dupdates, dmu, dnu, stream);
+        });
     });
 }
 
