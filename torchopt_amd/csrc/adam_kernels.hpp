@@ -306,7 +306,7 @@ struct BackwardUpdates {
 template <typename T>
 struct ForwardAll {
     static constexpr int NIN = 3, NOUT = 3, NPTR = 6;
-    static constexpr int kWavesPerCU = 24;
+    static constexpr int kWavesPerCU = 16;  // six streams per wave: few waves fill the queues
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T b1, b2, c1, c2, eps, eps_root;
     __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
@@ -333,7 +333,7 @@ template <typename T, bool HAS_DM, bool HAS_DV>
 struct BackwardAll {
     static constexpr int NIN = 4 + (HAS_DM ? 1 : 0) + (HAS_DV ? 1 : 0), NOUT = 3,
                          NPTR = NIN + NOUT;
-    static constexpr int kWavesPerCU = 24;
+    static constexpr int kWavesPerCU = 14;  // seven to nine streams per wave
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T b1, b2, p1, q2;
     __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
