@@ -1,0 +1,194 @@
+"""Functional `adam` / `adamw`, `chain`, `apply_updates` and `MetaAdam` on the GPU, pinned the way
+the reference pins its accelerated path: against `torch.optim.Adam` / `AdamW` in float64 at 25x
+the default tolerance (/root/reference/tests/test_alias.py:207-270, 487-550,
+tests/helpers.py:202-229), and the differentiable optimizer against the same inner loop written
+with plain differentiable tensor operations."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+
+import torchopt_amd as topt
+
+pytestmark = pytest.mark.gpu
+
+TOL = dict(rtol=25 * 1e-7, atol=25 * 1e-7)
+
+
+@pytest.fixture(scope='module', autouse=True)
+def _gpu():
+    assert torch.cuda.is_available(), 'these tests need a GPU; there is no fallback path'
+    yield
+    torch.cuda.synchronize()
+
+
+def make_models():
+    torch.manual_seed(7)
+
+    def net():
+        return torch.nn.Sequential(torch.nn.Linear(12, 24), torch.nn.Tanh(),
+                                   torch.nn.Linear(24, 3)).to('cuda', torch.float64)
+
+    a, b = net(), net()
+    b.load_state_dict(a.state_dict())
+    return a, b
+
+
+def batches(n):
+    g = torch.Generator(device='cuda').manual_seed(11)
+    for _ in range(n):
+        yield (torch.randn(32, 12, device='cuda', dtype=torch.float64, generator=g),
+               torch.randn(32, 3, device='cuda', dtype=torch.float64, generator=g))
+
+
+@pytest.mark.parametrize('inplace', [True, False])
+@pytest.mark.parametrize('weight_decay', [0.0, 1e-2])
+@pytest.mark.parametrize('maximize', [False, True])
+def test_adam_tracks_torch_optim(inplace, weight_decay, maximize):
+    model, ref = make_models()
+    lr = 1e-2
+    base = [p.detach().clone() for p in model.parameters()]
+    optim = topt.adam(lr, weight_decay=weight_decay, maximize=maximize)
+    params = tuple(model.parameters())
+    state = optim.init(params)
+    optim_ref = torch.optim.Adam(ref.parameters(), lr, weight_decay=weight_decay,
+                                 maximize=maximize)
+    for x, y in batches(5):
+        loss = ((model(x) - y) ** 2).mean()
+        grads = torch.autograd.grad(loss, params)
+        updates, state = optim.update(grads, state, params=params, inplace=inplace)
+        new = topt.apply_updates(params, updates, inplace=inplace)
+        if not inplace:
+            with torch.no_grad():
+                for p, q in zip(params, new):
+                    p.copy_(q)
+        optim_ref.zero_grad()
+        ((ref(x) - y) ** 2).mean().backward()
+        optim_ref.step()
+    for p, q, p0 in zip(model.parameters(), ref.parameters(), base):
+        torch.testing.assert_close(p - p0, q - p0, **TOL)
+
+
+@pytest.mark.parametrize('inplace', [True, False])
+def test_adamw_tracks_torch_optim(inplace):
+    model, ref = make_models()
+    lr, wd = 1e-2, 5e-2
+    optim = topt.adamw(lr, weight_decay=wd)
+    params = tuple(model.parameters())
+    state = optim.init(params)
+    optim_ref = torch.optim.AdamW(ref.parameters(), lr, weight_decay=wd)
+    for x, y in batches(5):
+        grads = torch.autograd.grad(((model(x) - y) ** 2).mean(), params)
+        updates, state = optim.update(grads, state, params=params, inplace=inplace)
+        with torch.no_grad():
+            for p, u in zip(params, updates):
+                p.add_(u)
+        optim_ref.zero_grad()
+        ((ref(x) - y) ** 2).mean().backward()
+        optim_ref.step()
+    for p, q in zip(model.parameters(), ref.parameters()):
+        torch.testing.assert_close(p, q, **TOL)
+
+
+def test_learning_rate_schedule_sees_the_count():
+    seen = []
+
+    def schedule(count):
+        seen.append(int(count))
+        return 0.1 / (1 + int(count))
+
+    optim = topt.adam(schedule)
+    p = (torch.ones(4, device='cuda'),)
+    state = optim.init(p)
+    for _ in range(3):
+        u, state = optim.update((torch.ones(4, device='cuda'),), state, params=p, inplace=True)
+    assert seen == [0, 1, 2]
+    # first step of Adam from zero state is sign(g) = 1: the update is -lr(count)
+    torch.testing.assert_close(u[0], torch.full((4,), -0.1 / 3, device='cuda'), rtol=1e-4, atol=0)
+
+
+def test_chain_state_and_missing_params():
+    optim = topt.adam(1e-3, weight_decay=0.1)
+    p = (torch.ones(3, device='cuda'),)
+    state = optim.init(p)
+    assert isinstance(state, tuple) and len(state) == 3
+    with pytest.raises(AssertionError, match='Parameters are required'):
+        optim.update((torch.ones(3, device='cuda'),), state, inplace=True)
+    with pytest.raises(ValueError, match='number of updates and states'):
+        optim.update((torch.ones(3, device='cuda'),), state[:2], params=p)
+
+
+def inner_loop_plain(w, b, x, y, steps, lr, b1, b2, eps, eps_root):
+    """The same MetaAdam inner loop with ordinary differentiable tensor operations."""
+    mw, vw, mb, vb = (torch.zeros_like(t) for t in (w, w, b, b))
+    for t in range(1, steps + 1):
+        loss = ((x @ w.t() + b - y) ** 2).mean()
+        gw, gb = torch.autograd.grad(loss, (w, b), create_graph=True)
+        mw, mb = b1 * mw + (1 - b1) * gw, b1 * mb + (1 - b1) * gb
+        vw, vb = b2 * vw + (1 - b2) * gw * gw, b2 * vb + (1 - b2) * gb * gb
+        c1, c2 = 1 / (1 - b1 ** t), 1 / (1 - b2 ** t)
+        w = w - lr * (mw * c1) / (torch.sqrt(vw * c2 + eps_root) + eps)
+        b = b - lr * (mb * c1) / (torch.sqrt(vb * c2 + eps_root) + eps)
+    return w, b
+
+
+@pytest.mark.parametrize('eps,er,rtol,atol', [(0.0, 0.0, 1e-8, 1e-11), (1e-8, 1e-8, 5e-3, 1e-5)],
+                         ids=['exact-when-eps-is-zero', 'reference-approximation'])
+def test_meta_adam_outer_gradient(eps, er, rtol, atol):
+    """Two inner steps of MetaAdam on a linear model, then an outer loss on the adapted
+    parameters, differentiated back to the initial parameters and to a learnable input scale.
+    The reference's backward of the update uses 1/(sqrt(v)+eps) where the exact derivative has
+    1/sqrt(v), and 1/(1-b2^t+eps_root) for the bias correction (adam_op_impl_cpu.cpp:309-329):
+    with eps = eps_root = 0 it is the exact derivative and must agree to rounding; otherwise it
+    is off by up to eps/sqrt(v) per element, by design."""
+    torch.manual_seed(5)
+    dt = torch.float64
+    lin = torch.nn.Linear(6, 4).to('cuda', dt)
+    w0, b0 = lin.weight, lin.bias
+    scale = torch.tensor(1.3, device='cuda', dtype=dt, requires_grad=True)
+    x = torch.randn(20, 6, device='cuda', dtype=dt)
+    y = torch.randn(20, 4, device='cuda', dtype=dt)
+    xo = torch.randn(20, 6, device='cuda', dtype=dt)
+    yo = torch.randn(20, 4, device='cuda', dtype=dt)
+    lr, b1, b2 = 0.05, 0.9, 0.999
+
+    opt = topt.MetaAdam(lin, lr, (b1, b2), eps, eps_root=er)
+    for _ in range(2):
+        opt.step(((lin(x * scale) - y) ** 2).mean())
+    assert lin.weight.grad_fn is not None  # parameters were replaced by differentiable results
+    outer = ((lin(xo) - yo) ** 2).mean()
+    got = torch.autograd.grad(outer, (w0, b0, scale))
+
+    w, b = inner_loop_plain(w0, b0, x * scale, y, 2, lr, b1, b2, eps, er)
+    outer_ref = ((xo @ w.t() + b - yo) ** 2).mean()
+    want = torch.autograd.grad(outer_ref, (w0, b0, scale))
+    torch.testing.assert_close(lin.weight, w, rtol=1e-9, atol=1e-12)
+    for g, r in zip(got, want):
+        torch.testing.assert_close(g, r, rtol=rtol, atol=atol)
+    counts = opt.state_dict()[0][1].count
+    assert [int(c) for c in counts] == [2, 2]
+
+
+def test_meta_adamw_and_unused_parameters():
+    """A parameter the loss does not touch gets no gradient (allow_unused) and stays put."""
+    torch.manual_seed(2)
+
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.used = torch.nn.Linear(5, 2)
+            self.unused = torch.nn.Linear(5, 2)
+
+        def forward(self, x):
+            return self.used(x)
+
+    net = Net().to('cuda')
+    before = net.unused.weight
+    opt = topt.MetaAdamW(net, 1e-2, weight_decay=0.1)
+    x = torch.randn(8, 5, device='cuda')
+    opt.step(net(x).pow(2).mean())
+    assert net.unused.weight is before and net.used.weight.grad_fn is not None
+    opt.step(net(x).pow(2).mean())
+    st = opt.state_dict()[0][1]
+    assert [int(c) for c in st.count] == [2, 2, 0, 0]

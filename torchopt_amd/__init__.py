@@ -10,6 +10,8 @@ import sys as _sys
 from torchopt_amd import accelerated_op
 from torchopt_amd.accelerated_op import AdamOp, MultiAdamOp
 from torchopt_amd.accelerated_op import is_available as accelerated_op_available
+from torchopt_amd.alias import adam, adamw, apply_updates, chain
+from torchopt_amd.meta import MetaAdam, MetaAdamW
 from torchopt_amd.optim import FusedAdam
 
 # `import torchopt_amd._C.adam_op` should work like `from torchopt_amd._C import adam_op`
@@ -19,4 +21,5 @@ _sys.modules.setdefault('torchopt_amd._C.adam_op', _C.adam_op)
 
 __version__ = '0.1.0'
 
-__all__ = ['AdamOp', 'FusedAdam', 'MultiAdamOp', 'accelerated_op', 'accelerated_op_available']
+__all__ = ['AdamOp', 'FusedAdam', 'MetaAdam', 'MetaAdamW', 'MultiAdamOp', 'accelerated_op',
+           'accelerated_op_available', 'adam', 'adamw', 'apply_updates', 'chain']
