@@ -208,28 +208,34 @@ TOA_API int toa_adam_backward_all_multi(int dtype, size_t num_tensors,
                                         void *const *dnu, void *stream);
 
 /* ---- fused optimizer step ------------------------------------------------
- * The classic in-place step of `Adam(..., use_accelerated_op=True).step()` in
- * one pass over memory: the Adam update (as toa_adam_forward_inplace), then
- * updates *= -lr (/root/reference/torchopt/transform/scale.py:93-98, reached
- * through alias/utils.py:226) and params += updates
- * (/root/reference/torchopt/update.py:71-74), each rounded separately so the
- * result is bit-identical to the three passes.  maximize != 0 negates the
- * gradients first (alias/utils.py:148).  mu, nu and params are overwritten;
- * `updates` is overwritten with the scaled update only if write_updates != 0
- * (otherwise it is read only: 28 instead of 32 bytes per float32 element,
- * against 44 for the separate passes).  Weight decay is not fused.  These two
- * entry points have no single counterpart in the reference. */
+ * The classic in-place step of `Adam(..., use_accelerated_op=True).step()` (or AdamW) in one
+ * pass over memory: the Adam update (as toa_adam_forward_inplace) together with its neighbours
+ * in the reference chain (paths under /root/reference/torchopt):
+ *   maximize != 0               gradients are negated first (alias/utils.py:148);
+ *   weight_decay, decoupled = 0 g += wd * p before the moments, as `adam` does
+ *                               (alias/utils.py:113-122);
+ *   weight_decay, decoupled = 1 u += wd * p after the Adam scaling, as `adamw` does
+ *                               (transform/add_decayed_weights.py:232-239);
+ *   updates *= -lr              (transform/scale.py:93-98 via alias/utils.py:226);
+ *   params += updates           (update.py:71-74).
+ * Every operation is rounded as the separate passes round it -- the two "+= wd * p" are
+ * single-rounding fused multiply-adds, which is what Tensor.add_(p, alpha=wd) computes -- so
+ * the result is bit-identical to them.  mu, nu and params are overwritten; `updates` is
+ * overwritten with the scaled update only if write_updates != 0 (otherwise it is read only:
+ * 28 instead of 32 bytes per float32 element, against 44 and more for the separate passes).
+ * TOA_F32 / TOA_F64 only.  No single counterpart in the reference. */
 TOA_API int toa_adam_fused_step(int dtype, void *params, void *updates, void *mu, void *nu,
                                 size_t n, double b1, double b2, double eps, double eps_root,
-                                uint64_t count, double lr, int maximize, int write_updates,
-                                void *stream);
+                                uint64_t count, double lr, double weight_decay, int decoupled,
+                                int maximize, int write_updates, void *stream);
 
 TOA_API int toa_adam_fused_step_multi(int dtype, size_t num_tensors, void *const *params,
                                       void *const *updates, void *const *mu, void *const *nu,
                                       const size_t *n, double b1, double b2, double eps,
                                       double eps_root, const uint64_t *counts,
-                                      uint64_t count_all, double lr, int maximize,
-                                      int write_updates, void *stream);
+                                      uint64_t count_all, double lr, double weight_decay,
+                                      int decoupled, int maximize, int write_updates,
+                                      void *stream);
 
 #ifdef __cplusplus
 }

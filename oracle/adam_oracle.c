@@ -150,32 +150,37 @@ void oracle_adam_host_scalars(double b1, double b2, double eps_root, uint64_t co
         }                                                                                      \
     }
 
-/* The classic in-place optimizer step as the reference chain performs it, three
- * passes restated as three statements per element (element-wise, so the order of
- * passes and elements is immaterial):
- *   1. [maximize] g = -g                 /root/reference/torchopt/alias/utils.py:148
- *   2. Adam forward_ in place            adam_op_impl_cpu.cpp:32-91
- *   3. updates *= -lr (scalar rounded to T)  /root/reference/torchopt/transform/scale.py:93-98
- *   4. params += updates                 /root/reference/torchopt/update.py:71-74
- * With write_updates == 0 the updates array is left as it was (the fused GPU
- * step can skip that store); params, mu and nu are the same either way. */
-#define ORACLE_DEFINE_STEP(T, SFX, SQRT)                                                       \
+/* The classic in-place optimizer step as the reference chains perform it, their passes
+ * restated as statements per element (element-wise, so the order of passes and elements is
+ * immaterial); paths under /root/reference/torchopt:
+ *   1. [maximize] g = -g                          alias/utils.py:148
+ *   2. [decay == 1, adam]  g = g + wd * p         alias/utils.py:113-122
+ *   3. Adam forward_ in place                     adam_op_impl_cpu.cpp:32-91
+ *   4. [decay == 2, adamw] u = u + wd * p         transform/add_decayed_weights.py:232-239
+ *   5. updates *= -lr (scalar rounded to T)       transform/scale.py:93-98
+ *   6. params += updates                          update.py:71-74
+ * Steps 2 and 4 are Tensor.add_(p, alpha=wd), which torch evaluates as one fused multiply-add
+ * (a single rounding), hence fma() here.  With write_updates == 0 the updates array is left as
+ * it was (the fused GPU step can skip that store); params, mu and nu are the same either way. */
+#define ORACLE_DEFINE_STEP(T, SFX, SQRT, FMA)                                                  \
     void oracle_adam_fused_step_##SFX(T *params, T *updates, T *mu, T *nu, size_t n,           \
                                       double b1_, double b2_, double eps_, double eps_root_,   \
-                                      uint64_t count, double lr_, int maximize,                \
-                                      int write_updates) {                                     \
+                                      uint64_t count, double lr_, double wd_, int decay,       \
+                                      int maximize, int write_updates) {                       \
         double s[4];                                                                           \
         oracle_adam_host_scalars(b1_, b2_, eps_root_, count, s);                               \
         const T b1 = (T)b1_, b2 = (T)b2_, eps = (T)eps_, eps_root = (T)eps_root_;              \
-        const T c1 = (T)s[0], c2 = (T)s[1], neg_lr = (T)(-lr_);                                \
+        const T c1 = (T)s[0], c2 = (T)s[1], neg_lr = (T)(-lr_), wd = (T)wd_;                   \
         PAR_FOR(n)                                                                             \
         for (size_t i = 0; i < n; ++i) {                                                       \
-            const T g = maximize ? -updates[i] : updates[i];                                   \
+            T g = maximize ? -updates[i] : updates[i];                                         \
+            if (decay == 1) g = FMA(wd, params[i], g);                                         \
             const T m1 = b1 * mu[i] + (1 - b1) * g;                                            \
             const T v1 = b2 * nu[i] + (1 - b2) * g * g;                                        \
             const T mh = m1 * c1;                                                              \
             const T vh = v1 * c2;                                                              \
-            const T u1 = mh / (SQRT(vh + eps_root) + eps);                                     \
+            T u1 = mh / (SQRT(vh + eps_root) + eps);                                           \
+            if (decay == 2) u1 = FMA(wd, params[i], u1);                                       \
             const T step = u1 * neg_lr;                                                        \
             mu[i] = m1;                                                                        \
             nu[i] = v1;                                                                        \
@@ -186,8 +191,8 @@ void oracle_adam_host_scalars(double b1, double b2, double eps_root, uint64_t co
 
 ORACLE_DEFINE(float, f32, sqrtf)
 ORACLE_DEFINE(double, f64, sqrt)
-ORACLE_DEFINE_STEP(float, f32, sqrtf)
-ORACLE_DEFINE_STEP(double, f64, sqrt)
+ORACLE_DEFINE_STEP(float, f32, sqrtf, fmaf)
+ORACLE_DEFINE_STEP(double, f64, sqrt, fma)
 
 
 /* ---------------------------------------------------------------------------------------------

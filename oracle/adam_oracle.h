@@ -20,7 +20,8 @@
  *   plus closed forms in tests/test_oracle.py;
  *   oracle_adam_fused_step_*: bit-for-bit against the reference chain itself run
  *   on CPU -- the compiled reference forward_ followed by the two torch calls the
- *   reference makes (Tensor.mul_(-lr), Tensor.add_) -- in tests/test_oracle.py.
+ *   reference makes (Tensor.add_(p, alpha=wd), Tensor.mul_(-lr), Tensor.add_) -- in
+ *   tests/test_oracle.py.
  *   No function is "parity unpinned".
  */
 #ifndef ADAM_ORACLE_H
@@ -83,15 +84,18 @@ void oracle_adam_backward_updates_f64(const double *dupdates, const double *upda
                                       double eps_root, uint64_t count, double *dnew_mu_out,
                                       double *dnew_nu_out);
 
-/* The reference chain's classic in-place step: [negate], Adam forward_, updates *= -lr,
- * params += updates (alias/utils.py:148, adam_op_impl_cpu.cpp:32-91, transform/scale.py:93-98,
+/* The reference chains' classic in-place step: [negate], [g += wd*p (decay 1)], Adam forward_,
+ * [u += wd*p (decay 2)], updates *= -lr, params += updates (alias/utils.py:113-122,148,
+ * adam_op_impl_cpu.cpp:32-91, transform/add_decayed_weights.py:232-239, transform/scale.py:93-98,
  * update.py:71-74). */
 void oracle_adam_fused_step_f32(float *params, float *updates, float *mu, float *nu, size_t n,
                                 double b1, double b2, double eps, double eps_root,
-                                uint64_t count, double lr, int maximize, int write_updates);
+                                uint64_t count, double lr, double weight_decay, int decay,
+                                int maximize, int write_updates);
 void oracle_adam_fused_step_f64(double *params, double *updates, double *mu, double *nu, size_t n,
                                 double b1, double b2, double eps, double eps_root,
-                                uint64_t count, double lr, int maximize, int write_updates);
+                                uint64_t count, double lr, double weight_decay, int decay,
+                                int maximize, int write_updates);
 
 /* Host-side bias-correction scalars in double, before the cast to the element
  * type (adam_op_impl_cpu.cpp:73-74, 191-192, 328-329).

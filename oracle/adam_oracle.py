@@ -144,12 +144,14 @@ def backward_updates(dupdates, updates, new_mu, b1, b2, eps_root, count):
 
 
 def fused_step(params, updates, mu, nu, b1, b2, eps, eps_root, count, lr, maximize=False,
-               write_updates=True):
+               write_updates=True, weight_decay=0.0, decoupled=False):
     """Mutates params, mu, nu (and updates when write_updates), like the reference's classic
-    in-place chain: [negate], forward_, scale by -lr, apply."""
+    in-place chains: [negate], [L2 decay], forward_, [decoupled decay], scale by -lr, apply."""
+    decay = 0 if weight_decay == 0.0 else (2 if decoupled else 1)
     _fn('fused_step', params.dtype)(_ptr(params), _ptr(updates), _ptr(mu), _ptr(nu),
                                     _SZ(params.size), _D(b1), _D(b2), _D(eps), _D(eps_root),
-                                    _U64(count), _D(lr), ctypes.c_int(int(maximize)),
+                                    _U64(count), _D(lr), _D(weight_decay), ctypes.c_int(decay),
+                                    ctypes.c_int(int(maximize)),
                                     ctypes.c_int(int(write_updates)))
     return params, updates, mu, nu
 

@@ -10,7 +10,7 @@ import torch
 
 from conftest import assert_bit_equal
 from oracle import adam_oracle as O
-from torchopt_amd import FusedAdam
+from torchopt_amd import FusedAdam, FusedAdamW
 from torchopt_amd._C import adam_op
 from torchopt_amd.transform import scale_by_accelerated_adam
 
@@ -57,6 +57,40 @@ def test_single_tensor_against_oracle(dtype, maximize, write_updates):
         assert_bit_equal(host(gm), m, f'n={n} mu')
         assert_bit_equal(host(gv), v, f'n={n} nu')
         assert_bit_equal(host(gg), g, f'n={n} updates (untouched unless write_updates)')
+
+
+@pytest.mark.parametrize('dtype', [np.float32, np.float64], ids=['f32', 'f64'])
+@pytest.mark.parametrize('decoupled', [False, True], ids=['l2', 'decoupled'])
+def test_weight_decay_against_oracle(dtype, decoupled):
+    for k, n in enumerate([1, 257, 65537, (1 << 20) + 3]):
+        p, g, m, v = rand4(dtype, n, 500 + n)
+        gp, gg, gm, gv = dev(p), dev(g), dev(m), dev(v)
+        adam_op.fused_step_(gp, gg, gm, gv, B1, B2, EPS, 1e-8, 4, 0.01, maximize=bool(k % 2),
+                            write_updates=True, weight_decay=0.05, decoupled=decoupled)
+        O.fused_step(p, g, m, v, B1, B2, EPS, 1e-8, 4, 0.01, bool(k % 2), True, 0.05, decoupled)
+        for t, want, what in ((gp, p, 'params'), (gg, g, 'updates'), (gm, m, 'mu'), (gv, v, 'nu')):
+            assert_bit_equal(host(t), want, f'n={n} {what}')
+
+
+@pytest.mark.parametrize('decay', ['l2', 'decoupled'])
+def test_weight_decay_equals_the_unfused_chain_on_the_gpu(decay):
+    """With PyTorch's own GPU kernels for the neighbours (add_ with alpha, mul_, add_)."""
+    n, lr, wd, count = (1 << 21) + 1, 1e-3, 0.02, 9
+    g = torch.Generator(device='cuda').manual_seed(8)
+    p, u = (torch.randn(n, device='cuda', generator=g) for _ in range(2))
+    m = torch.randn(n, device='cuda', generator=g).mul_(0.1)
+    v = torch.randn(n, device='cuda', generator=g).mul_(0.01).abs_()
+    p2, u2, m2, v2 = p.clone(), u.clone(), m.clone(), v.clone()
+    if decay == 'l2':
+        u.add_(p, alpha=wd)
+    adam_op.forward_(u, m, v, B1, B2, EPS, 0.0, count)
+    if decay == 'decoupled':
+        u.add_(p, alpha=wd)
+    u.mul_(-lr)
+    p.add_(u)
+    adam_op.fused_step_(p2, u2, m2, v2, B1, B2, EPS, 0.0, count, lr, write_updates=True,
+                        weight_decay=wd, decoupled=decay == 'decoupled')
+    assert torch.equal(p, p2) and torch.equal(u, u2) and torch.equal(m, m2) and torch.equal(v, v2)
 
 
 @pytest.mark.parametrize('dtype', [torch.float32, torch.float64], ids=['f32', 'f64'])
@@ -130,15 +164,18 @@ def test_fused_adam_equals_the_transformation_chain(maximize):
     chain.update(tuple(torch.randn(s, device='cuda') for s in shapes), st, inplace=True)
 
 
-def test_fused_adam_tracks_torch_optim_adam():
+@pytest.mark.parametrize('cls,ref_cls,wd', [(FusedAdam, torch.optim.Adam, 0.0),
+                                            (FusedAdam, torch.optim.Adam, 0.05),
+                                            (FusedAdamW, torch.optim.AdamW, 0.05)])
+def test_fused_adam_tracks_torch_optim_adam(cls, ref_cls, wd):
     torch.manual_seed(0)
     net = torch.nn.Sequential(torch.nn.Linear(16, 32), torch.nn.ReLU(),
                               torch.nn.Linear(32, 4)).to('cuda', torch.float64)
     ref = torch.nn.Sequential(torch.nn.Linear(16, 32), torch.nn.ReLU(),
                               torch.nn.Linear(32, 4)).to('cuda', torch.float64)
     ref.load_state_dict(net.state_dict())
-    a = FusedAdam(net.parameters(), 1e-2)
-    b = torch.optim.Adam(ref.parameters(), 1e-2)
+    a = cls(net.parameters(), 1e-2, weight_decay=wd)
+    b = ref_cls(ref.parameters(), 1e-2, weight_decay=wd)
     for _ in range(10):
         x = torch.randn(32, 16, device='cuda', dtype=torch.float64)
         y = torch.randn(32, 4, device='cuda', dtype=torch.float64)

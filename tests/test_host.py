@@ -64,7 +64,7 @@ def test_abi_version_and_error_strings():
         _lib.check(-1, 'x')
     # the fused optimizer step serves float32 / float64 only
     assert lib.toa_adam_fused_step(_lib.TOA_F16, None, None, None, None, 0, 0.9, 0.999, 1e-8, 0.0, 1,
-                                   1e-3, 0, 0, None) == -1
+                                   1e-3, 0.0, 0, 0, 0, None) == -1
 
 
 def test_argument_errors_need_no_device():
@@ -180,7 +180,7 @@ def test_fused_adam_argument_validation():
 
     p = [torch.ones(3)]
     for kwargs in (dict(lr=-1.0), dict(eps=-1.0), dict(betas=(1.0, 0.9)), dict(betas=(0.9, 1.0)),
-                   dict(weight_decay=0.01), dict(lr=lambda c: 0.1)):
+                   dict(weight_decay=-0.01), dict(lr=lambda c: 0.1)):
         with pytest.raises(ValueError):
             FusedAdam(p, **kwargs)
     with pytest.raises(TypeError):

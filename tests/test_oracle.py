@@ -150,35 +150,61 @@ def test_c_oracle_equals_compiled_reference(dtype):
 
 @pytest.mark.parametrize('dtype', DTYPES, ids=['f32', 'f64'])
 @pytest.mark.parametrize('maximize', [False, True])
-def test_fused_step_is_the_reference_chain(dtype, maximize):
-    """The classic in-place step of the reference is three passes: [neg_], forward_,
-    Tensor.mul_(-lr) (transform/scale.py:93-98) and Tensor.add_ (update.py:71-74).  Run exactly
-    those calls on CPU tensors -- forward_ from the compiled reference where it is built, else
-    from the pinned C oracle -- and compare the one-pass oracle with them."""
+@pytest.mark.parametrize('decay', ['none', 'l2', 'decoupled'])
+def test_fused_step_is_the_reference_chain(dtype, maximize, decay):
+    """The classic in-place step of the reference is a chain of passes: [neg_],
+    [add_(p, alpha=wd)] (alias/utils.py:113-122), forward_, [add_(p, alpha=wd)]
+    (transform/add_decayed_weights.py:232-239), mul_(-lr) (transform/scale.py:93-98) and add_
+    (update.py:71-74).  Run exactly those calls on CPU tensors -- forward_ from the compiled
+    reference where it is built, else from the pinned C oracle -- and compare the one-pass
+    oracle with them."""
     import torch
 
     ref = O.load_reference()
     rng = np.random.default_rng(31)
+    wd = 0.0 if decay == 'none' else 0.03
     for n, lr, count, eps_root in [(1, 1e-3, 1, 0.0), (1003, 1e-3, 7, 0.0), (200_003, 0.05, 1000, 1e-8)]:
         g, m, v = _rand(dtype, n, n)
         p = rng.standard_normal(n).astype(dtype)
         tg, tm, tv, tp = (torch.from_numpy(x.copy()) for x in (g, m, v, p))
         if maximize:
             tg.neg_()
+        if decay == 'l2':
+            tg.add_(tp, alpha=wd)
         if ref is not None:
             ref.adam_op.forward_(tg, tm, tv, 0.9, 0.999, 1e-8, eps_root, count)
         else:
             O.forward_inplace(tg.numpy(), tm.numpy(), tv.numpy(), 0.9, 0.999, 1e-8, eps_root, count)
+        if decay == 'decoupled':
+            tg.add_(tp, alpha=wd)
         tg.mul_(-lr)
         tp.add_(tg)
         for write_updates in (True, False):
             op, og, om, ov = p.copy(), g.copy(), m.copy(), v.copy()
             O.fused_step(op, og, om, ov, 0.9, 0.999, 1e-8, eps_root, count, lr, maximize,
-                         write_updates)
+                         write_updates, wd, decay == 'decoupled')
             assert_bit_equal(op, tp.numpy(), 'params')
             assert_bit_equal(om, tm.numpy(), 'mu')
             assert_bit_equal(ov, tv.numpy(), 'nu')
             assert_bit_equal(og, tg.numpy() if write_updates else g, 'updates')
+
+
+def test_weight_decay_is_a_fused_multiply_add():
+    """Tensor.add_(p, alpha=wd) rounds once; g + round(wd*p) differs on a few percent of random
+    float32 inputs, so the distinction is observable and the oracle must be on the fma side."""
+    import torch
+
+    rng = np.random.default_rng(2)
+    n = 50_000
+    g, p = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+    torch_way = torch.from_numpy(g.copy()).add_(torch.from_numpy(p), alpha=0.01).numpy()
+    two_roundings = g + np.float32(0.01) * p
+    assert (torch_way != two_roundings).sum() > 100
+    # the oracle's decayed gradient shows in mu after one step from mu = 0 with b1 = 0: mu' = g'
+    mu = np.zeros(n, np.float32)
+    O.fused_step(p.copy(), g.copy(), mu, np.zeros(n, np.float32), 0.0, 0.0, 1e-8, 0.0, 1, 1e-3,
+                 False, False, 0.01, False)
+    assert_bit_equal(mu, torch_way)
 
 
 def test_fused_step_scales_by_the_rounded_learning_rate():

@@ -18,7 +18,7 @@ TOA_F32 = 0
 TOA_F64 = 1
 TOA_F16 = 2
 TOA_BF16 = 3
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _vp = ctypes.c_void_p
 _vpp = ctypes.POINTER(ctypes.c_void_p)
@@ -57,9 +57,10 @@ SIGNATURES = {
                               _vp, _vp],
     'toa_adam_backward_all_multi': [_i, _sz, _vpp, _vpp, _vpp, _vpp, _vpp, _vpp, _szp, _d, _d, _d,
                                     _u64p, _u64, _vpp, _vpp, _vpp, _vp],
-    'toa_adam_fused_step': [_i, _vp, _vp, _vp, _vp, _sz, _d, _d, _d, _d, _u64, _d, _i, _i, _vp],
+    'toa_adam_fused_step': [_i, _vp, _vp, _vp, _vp, _sz, _d, _d, _d, _d, _u64, _d, _d, _i, _i, _i,
+                            _vp],
     'toa_adam_fused_step_multi': [_i, _sz, _vpp, _vpp, _vpp, _vpp, _szp, _d, _d, _d, _d, _u64p,
-                                  _u64, _d, _i, _i, _vp],
+                                  _u64, _d, _d, _i, _i, _i, _vp],
 }
 
 _lib = None

@@ -353,30 +353,45 @@ struct BackwardAll {
     }
 };
 
-// The classic optimizer step in one pass: the in-place Adam step followed by what
-// the reference chain does next with its result -- scale by -lr
-// (/root/reference/torchopt/transform/scale.py:93-98 via alias/utils.py:226) and
-// add to the parameters (/root/reference/torchopt/update.py:71-74) -- each still
-// rounded on its own, so the result equals the three separate passes bit for
-// bit while streaming 28 (or 32) bytes per float32 element instead of 44.
-// `maximize` negates the gradient first (alias/utils.py:148).
+// The classic optimizer step in one pass: the in-place Adam step together with what
+// the reference chains do around it --
+//   [maximize]        g = -g                       alias/utils.py:148
+//   [L2 decay, adam]  g = g + wd * p               alias/utils.py:113-122
+//   Adam forward_                                  adam_op_impl_cpu.cpp:32-91
+//   [decay, adamw]    u = u + wd * p               transform/add_decayed_weights.py:232-239
+//   u = u * (-lr)                                  transform/scale.py:93-98
+//   p = p + u                                      update.py:71-74
+// (paths under /root/reference/torchopt) -- each still rounded as the separate
+// passes round it, so the result equals them bit for bit while streaming 28 (or
+// 32) bytes per float32 element instead of 44 and more.  The two "+ wd * p" are
+// single-rounding fused multiply-adds because that is what Tensor.add_(p,
+// alpha=wd) computes, on CPU and GPU alike; everything else is one rounding per
+// operation.
 // Slots: 0 updates (gradients), 1 mu, 2 nu, 3 params.
+enum : int { kNoDecay = 0, kDecayIntoGradient = 1, kDecayIntoUpdate = 2 };
+
+__device__ __forceinline__ float toa_fma(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ double toa_fma(double a, double b, double c) { return __builtin_fma(a, b, c); }
+
 template <typename T, bool WRITE_UPDATES>
 struct FusedStep {
     static constexpr int NIN = 4, NOUT = WRITE_UPDATES ? 4 : 3, NPTR = 4;
     static constexpr int kWavesPerCU = 13;
     // outputs: mu', nu', params', then the scaled update
     __device__ static constexpr int out_slot(int j) { return j == 3 ? 0 : j + 1; }
-    T b1, b2, c1, c2, eps, eps_root, neg_lr;
+    T b1, b2, c1, c2, eps, eps_root, neg_lr, wd;
+    int decay;
     bool maximize;
     __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
-        const T g = maximize ? -in[0] : in[0];
+        T g = maximize ? -in[0] : in[0];
         const T m = in[1], v = in[2], p = in[3];
+        if (decay == kDecayIntoGradient) g = toa_fma(wd, p, g);
         const T m1 = b1 * m + (1 - b1) * g;
         const T v1 = b2 * v + (1 - b2) * g * g;
         const T mh = m1 * c1;
         const T vh = v1 * c2;
-        const T u1 = mh / (toa_sqrt(vh + eps_root) + eps);
+        T u1 = mh / (toa_sqrt(vh + eps_root) + eps);
+        if (decay == kDecayIntoUpdate) u1 = toa_fma(wd, p, u1);
         const T step = u1 * neg_lr;
         out[0] = m1;
         out[1] = v1;

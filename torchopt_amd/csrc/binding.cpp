@@ -312,7 +312,7 @@ std::array<Tensor, 3> backwardAll(const Tensor &dnew_updates_in,
 std::array<Tensor, 4> fusedStep(const Tensor &params, const Tensor &updates, const Tensor &mu,
                                 const Tensor &nu, double b1, double b2, double eps,
                                 double eps_root, size_t count, double lr, bool maximize,
-                                bool write_updates) {
+                                bool write_updates, double weight_decay, bool decoupled) {
     const char *name = "adamFusedStep";
     size_t n;
     const int code = gate(name, updates, {&mu, &nu, &params}, &n);
@@ -326,7 +326,8 @@ std::array<Tensor, 4> fusedStep(const Tensor &params, const Tensor &updates, con
         const OnDeviceOf dev(updates);
         check(toa_adam_fused_step(code, params.data_ptr(), updates.data_ptr(), mu.data_ptr(),
                                   nu.data_ptr(), n, b1, b2, eps, eps_root, count, lr,
-                                  (int)maximize, (int)write_updates, dev.stream()),
+                                  weight_decay, (int)decoupled, (int)maximize,
+                                  (int)write_updates, dev.stream()),
               name);
     }
     return {params, updates, mu, nu};
@@ -614,7 +615,8 @@ std::tuple<TensorList, TensorList, TensorList> backwardAllMulti(
 py::tuple fusedStepMulti(const py::object &params_o, const py::object &updates_o,
                          const py::object &mu_o, const py::object &nu_o, double b1, double b2,
                          double eps, double eps_root, const py::object &counts, double lr,
-                         bool maximize, bool write_updates) {
+                         bool maximize, bool write_updates, double weight_decay,
+                         bool decoupled) {
     const char *name = "adamFusedStepMulti";
     const auto params = params_o.cast<TensorList>();
     const auto updates = updates_o.cast<TensorList>();
@@ -626,8 +628,9 @@ py::tuple fusedStepMulti(const py::object &params_o, const py::object &updates_o
         const OnDeviceOf dev(firstNonEmpty(updates));
         check(toa_adam_fused_step_multi(l.code, l.num, l.ptr[3].data(), l.ptr[0].data(),
                                         l.ptr[1].data(), l.ptr[2].data(), l.n.data(), b1, b2, eps,
-                                        eps_root, c.data(), c.all, lr, (int)maximize,
-                                        (int)write_updates, dev.stream()),
+                                        eps_root, c.data(), c.all, lr, weight_decay,
+                                        (int)decoupled, (int)maximize, (int)write_updates,
+                                        dev.stream()),
               name);
     }
     return py::make_tuple(params_o, updates_o, mu_o, nu_o);
@@ -689,8 +692,10 @@ PYBIND11_MODULE(_C, mod) {
     m.def("fused_step_", &fusedStep,
           "Adam + scale(-lr) + apply in one pass; returns [params, updates, mu, nu]", "params"_a,
           "updates"_a, "mu"_a, "nu"_a, "b1"_a, "b2"_a, "eps"_a, "eps_root"_a, "count"_a, "lr"_a,
-          py::kw_only(), "maximize"_a = false, "write_updates"_a = false);
+          py::kw_only(), "maximize"_a = false, "write_updates"_a = false,
+          "weight_decay"_a = 0.0, "decoupled"_a = false);
     m.def("fused_step_multi_", &fusedStepMulti, "fused_step_ over lists", "params"_a, "updates"_a,
           "mu"_a, "nu"_a, "b1"_a, "b2"_a, "eps"_a, "eps_root"_a, "counts"_a, "lr"_a,
-          py::kw_only(), "maximize"_a = false, "write_updates"_a = false);
+          py::kw_only(), "maximize"_a = false, "write_updates"_a = false,
+          "weight_decay"_a = 0.0, "decoupled"_a = false);
 }

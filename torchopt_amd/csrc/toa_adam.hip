@@ -277,7 +277,7 @@ int backward_all_multi(size_t num, const void *const *dnew_updates,
 
 extern "C" {
 
-int toa_adam_abi_version(void) { return 1; }
+int toa_adam_abi_version(void) { return 2; }
 
 int toa_adam_set_waves_per_cu(int waves) {
     const int prev = waves_override();
@@ -532,17 +532,20 @@ int toa_adam_backward_all_multi(int dtype, size_t num_tensors, const void *const
 
 int toa_adam_fused_step(int dtype, void *params, void *updates, void *mu, void *nu, size_t n,
                         double b1, double b2, double eps, double eps_root, uint64_t count,
-                        double lr, int maximize, int write_updates, void *stream) {
+                        double lr, double weight_decay, int decoupled, int maximize,
+                        int write_updates, void *stream) {
     const HostScalars s = host_scalars(b1, b2, eps_root, count);
+    const int decay = weight_decay == 0.0 ? kNoDecay
+                                          : (decoupled ? kDecayIntoUpdate : kDecayIntoGradient);
     TOA_DISPATCH(dtype, [&] {
         T *const p[4] = {(T *)updates, (T *)mu, (T *)nu, (T *)params};
         if (write_updates) {
-            const FusedStep<T, true> op{(T)b1,  (T)b2,       (T)s.c1,  (T)s.c2,
-                                        (T)eps, (T)eps_root, (T)(-lr), maximize != 0};
+            const FusedStep<T, true> op{(T)b1,       (T)b2,    (T)s.c1,         (T)s.c2, (T)eps,
+                                        (T)eps_root, (T)(-lr), (T)weight_decay, decay,   maximize != 0};
             return launch_single<T>(op, p, n, stream);
         }
-        const FusedStep<T, false> op{(T)b1,  (T)b2,       (T)s.c1,  (T)s.c2,
-                                     (T)eps, (T)eps_root, (T)(-lr), maximize != 0};
+        const FusedStep<T, false> op{(T)b1,       (T)b2,    (T)s.c1,         (T)s.c2, (T)eps,
+                                     (T)eps_root, (T)(-lr), (T)weight_decay, decay,   maximize != 0};
         return launch_single<T>(op, p, n, stream);
     });
 }
@@ -550,23 +553,28 @@ int toa_adam_fused_step(int dtype, void *params, void *updates, void *mu, void *
 int toa_adam_fused_step_multi(int dtype, size_t num_tensors, void *const *params,
                               void *const *updates, void *const *mu, void *const *nu,
                               const size_t *n, double b1, double b2, double eps, double eps_root,
-                              const uint64_t *counts, uint64_t count_all, double lr, int maximize,
+                              const uint64_t *counts, uint64_t count_all, double lr,
+                              double weight_decay, int decoupled, int maximize,
                               int write_updates, void *stream) {
+    const int decay = weight_decay == 0.0 ? kNoDecay
+                                          : (decoupled ? kDecayIntoUpdate : kDecayIntoGradient);
     TOA_DISPATCH(dtype, [&] {
         const void *const *const lists[4] = {CPP(updates), CPP(mu), CPP(nu), CPP(params)};
         if (write_updates) {
             auto make = [&](uint64_t c) {
                 const HostScalars s = host_scalars(b1, b2, eps_root, c);
-                return FusedStep<T, true>{(T)b1,  (T)b2,       (T)s.c1,  (T)s.c2,
-                                          (T)eps, (T)eps_root, (T)(-lr), maximize != 0};
+                return FusedStep<T, true>{(T)b1,       (T)b2,    (T)s.c1,         (T)s.c2, (T)eps,
+                                          (T)eps_root, (T)(-lr), (T)weight_decay, decay,
+                                          maximize != 0};
             };
             return launch_multi<T, FusedStep<T, true>>(make, num_tensors, lists, n, counts,
                                                        count_all, stream);
         }
         auto make = [&](uint64_t c) {
             const HostScalars s = host_scalars(b1, b2, eps_root, c);
-            return FusedStep<T, false>{(T)b1,  (T)b2,       (T)s.c1,  (T)s.c2,
-                                       (T)eps, (T)eps_root, (T)(-lr), maximize != 0};
+            return FusedStep<T, false>{(T)b1,       (T)b2,    (T)s.c1,         (T)s.c2, (T)eps,
+                                       (T)eps_root, (T)(-lr), (T)weight_decay, decay,
+                                       maximize != 0};
         };
         return launch_multi<T, FusedStep<T, false>>(make, num_tensors, lists, n, counts,
                                                     count_all, stream);

@@ -1,12 +1,12 @@
-"""`FusedAdam`: the classic `Adam(..., use_accelerated_op=True)` optimizer with its whole step
--- Adam scaling, multiplication by -lr and the addition to the parameters -- in one pass over
-memory.
+"""`FusedAdam` / `FusedAdamW`: the classic `Adam(..., use_accelerated_op=True)` and `AdamW`
+optimizers with their whole step -- sign flip, weight decay, Adam scaling, multiplication by -lr
+and the addition to the parameters -- in one pass over memory.
 
-Counterpart of /root/reference/torchopt/optim/adam.py:43-92 on top of
-/root/reference/torchopt/optim/base.py:30-135 for the case the fused kernel covers: constant
-learning rate, no weight decay.  What `step()` leaves in the parameters and in the moments is
-bit-identical to the reference chain (`scale_by_accelerated_adam` -> `scale(-lr)` ->
-`apply_updates`, all in place); the differences are mechanical:
+Counterparts of /root/reference/torchopt/optim/adam.py:43-92 and optim/adamw.py on top of
+/root/reference/torchopt/optim/base.py:30-135 for a constant learning rate.  What `step()` leaves in the parameters and in the moments is
+bit-identical to the reference chain (`flip_sign_and_add_weight_decay` ->
+`scale_by_accelerated_adam` [-> `add_decayed_weights`] -> `scale(-lr)` -> `apply_updates`, all in
+place); the differences are mechanical:
 
   * one multi-tensor launch per hundred-odd parameters instead of three passes per parameter
     (28 instead of 44 bytes of HBM traffic per float32 element);
@@ -27,11 +27,14 @@ from torchopt_amd.accelerated_op.adam_op import adam_op
 from torchopt_amd.transform.scale_by_adam import ScaleByAdamState, _inc_counts, _remember
 
 
-__all__ = ['FusedAdam']
+__all__ = ['FusedAdam', 'FusedAdamW']
 
 
 class FusedAdam:
-    """Classic Adam with the fused single-pass step (GPU tensors, float32 / float64)."""
+    """Classic Adam with the fused single-pass step (GPU tensors, float32 / float64).
+    `weight_decay` is the L2 kind: added to the gradient before the moments."""
+
+    _decoupled = False
 
     def __init__(
         self,
@@ -55,10 +58,9 @@ class FusedAdam:
             raise ValueError(f'Invalid beta parameter at index 0: {b1}')
         if not 0.0 <= b2 < 1.0:
             raise ValueError(f'Invalid beta parameter at index 1: {b2}')
-        if weight_decay != 0.0:
-            raise ValueError('FusedAdam does not fuse weight decay; chain '
-                             'scale_by_accelerated_adam with your own decay instead')
-        self.lr, self.b1, self.b2, self.eps = lr, b1, b2, eps
+        if not weight_decay >= 0.0:
+            raise ValueError(f'Invalid weight_decay value: {weight_decay}')
+        self.lr, self.b1, self.b2, self.eps, self.weight_decay = lr, b1, b2, eps, weight_decay
         self.eps_root, self.maximize = eps_root, maximize
         self.param_groups: list[tuple[torch.Tensor, ...]] = []
         self.state_groups: list[ScaleByAdamState | None] = []
@@ -119,6 +121,20 @@ class FusedAdam:
                     [group[k].data for k in ks], [grads[k] for k in ks],
                     [state.mu[k] for k in ks], [state.nu[k] for k in ks],
                     self.b1, self.b2, self.eps, self.eps_root, counts, self.lr,
-                    maximize=self.maximize, write_updates=False)
+                    maximize=self.maximize, write_updates=False,
+                    weight_decay=self.weight_decay, decoupled=self._decoupled)
             self.state_groups[i] = state._replace(count=tuple(new_counts))
         return loss
+
+
+class FusedAdamW(FusedAdam):
+    """Classic AdamW with the fused single-pass step: `weight_decay` is decoupled, added to the
+    Adam-scaled update (/root/reference/torchopt/alias/adamw.py:140-151)."""
+
+    _decoupled = True
+
+    def __init__(self, params, lr: float = 1e-3, betas=(0.9, 0.999), eps: float = 1e-8,
+                 weight_decay: float = 1e-2, *, eps_root: float = 0.0,
+                 maximize: bool = False) -> None:
+        super().__init__(params, lr, betas, eps, weight_decay, eps_root=eps_root,
+                         maximize=maximize)
