@@ -1,0 +1,131 @@
+"""Seeded random sweep: random lengths, alignments, hyper-parameters, element types and ops
+through the GPU path against the oracle, plus one tensor longer than 2^32 elements to cover
+64-bit indexing.  Everything bit for bit."""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import assert_bit_equal
+from oracle import adam_oracle as O
+from torchopt_amd._C import adam_op
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope='module', autouse=True)
+def _gpu():
+    assert torch.cuda.is_available(), 'these tests need a GPU; there is no fallback path'
+    yield
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+
+
+def to_fmt(x, tag):
+    if tag == 'bf16':
+        return O.bf16_bits(np.asarray(x, dtype=np.float32))
+    return np.asarray(x).astype({'f32': np.float32, 'f64': np.float64, 'f16': np.float16}[tag])
+
+
+def dev(a, tag):
+    a = np.ascontiguousarray(a)
+    if tag == 'bf16':
+        return torch.from_numpy(a.view(np.int16)).cuda().view(torch.bfloat16)
+    return torch.from_numpy(a).cuda()
+
+
+def host(t, tag):
+    if tag == 'bf16':
+        return t.detach().contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+    return t.detach().cpu().numpy()
+
+
+@pytest.mark.parametrize('seed', range(6))
+def test_random_cases(seed):
+    rng = np.random.default_rng(1234 + seed)
+    for case in range(40):
+        tag = ['f32', 'f64', 'f16', 'bf16'][int(rng.integers(4))]
+        n = int(rng.choice([rng.integers(0, 40), rng.integers(0, 3000), rng.integers(0, 200_000)]))
+        off = int(rng.integers(0, 9))
+        b1, b2 = float(rng.uniform(0, 0.999)), float(rng.uniform(0, 0.9999))
+        eps = float(10.0 ** rng.uniform(-8, -2)) if tag in ('f32', 'f64') else float(
+            10.0 ** rng.uniform(-4, -2))
+        er = float(rng.choice([0.0, 10.0 ** rng.uniform(-6, -3)]))
+        count = int(rng.choice([1, 2, 17, 1000, 10 ** 6]))
+        scale = float(10.0 ** rng.uniform(-3, 2))
+        raw = {k: to_fmt(scale * rng.standard_normal(n + off + 3), tag)
+               for k in ('updates', 'mu', 'dmu', 'dnu', 'dupdates')}
+        raw['nu'] = to_fmt(np.abs(scale * scale * rng.standard_normal(n + off + 3)), tag)
+        cut = {k: a[off:off + n].copy() for k, a in raw.items()}
+        g = {k: dev(a, tag)[off:off + n] for k, a in raw.items()}
+        label = f'seed {seed} case {case}: {tag} n={n} off={off} count={count}'
+        with np.errstate(all='ignore'):
+            e_mu = O.forward_mu(cut['updates'], cut['mu'], b1)
+            e_nu = O.forward_nu(cut['updates'], cut['nu'], b2)
+            e_u = O.forward_updates(e_mu, e_nu, b1, b2, eps, er, count)
+            bm, bv = O.backward_updates(cut['dupdates'], e_u, e_mu, b1, b2, er, count)
+        op = int(rng.integers(4))
+        if op == 0:  # the three split forwards and the fused in-place step
+            assert_bit_equal(host(adam_op.forward_mu(g['updates'], g['mu'], b1), tag), e_mu, label)
+            assert_bit_equal(host(adam_op.forward_nu(g['updates'], g['nu'], b2), tag), e_nu, label)
+            adam_op.forward_(g['updates'], g['mu'], g['nu'], b1, b2, eps, er, count)
+            assert_bit_equal(host(g['updates'], tag), e_u, label)
+            assert_bit_equal(host(g['nu'], tag), e_nu, label)
+        elif op == 1:  # one-pass forward
+            got = adam_op.forward_all(g['updates'], g['mu'], g['nu'], b1, b2, eps, er, count)
+            for t, want in zip(got, (e_mu, e_nu, e_u)):
+                assert_bit_equal(host(t, tag), want, label)
+        elif op == 2:  # the three split backwards
+            got = adam_op.backward_updates(g['dupdates'], dev(e_u, tag), dev(e_mu, tag),
+                                           dev(e_nu, tag), b1, b2, er, count)
+            assert_bit_equal(host(got[0], tag), bm, label)
+            assert_bit_equal(host(got[1], tag), bv, label)
+            got = adam_op.backward_mu(g['dmu'], g['updates'], g['mu'], b1)
+            want = O.backward_mu(cut['dmu'], b1)
+            assert_bit_equal(host(got[0], tag), want[0], label)
+            got = adam_op.backward_nu(g['dnu'], g['updates'], g['nu'], b2)
+            want = O.backward_nu(cut['dnu'], cut['updates'], b2)
+            assert_bit_equal(host(got[0], tag), want[0], label)
+            assert_bit_equal(host(got[1], tag), want[1], label)
+        else:  # one-pass backward without outside gradients
+            got = adam_op.backward_all(g['dupdates'], None, None, dev(e_u, tag), dev(e_mu, tag),
+                                       g['updates'], b1, b2, er, count)
+            with np.errstate(all='ignore'):
+                du1, dmu = O.backward_mu(bm, b1)
+                du2, dnu = O.backward_nu(bv, cut['updates'], b2)
+            assert_bit_equal(host(got[1], tag), dmu, label)
+            assert_bit_equal(host(got[2], tag), dnu, label)
+        # nothing outside the views was touched
+        for k in ('updates', 'mu', 'nu'):
+            full = host(g[k]._base if g[k]._base is not None else g[k], tag)
+            assert_bit_equal(full[:off], raw[k][:off], label + ' head guard')
+            assert_bit_equal(full[off + n:], raw[k][off + n:], label + ' tail guard')
+
+
+def test_tensor_longer_than_2_to_32_elements():
+    """2^32 + 777 float16 elements per array (8 GiB each): element indices and byte offsets pass
+    32 bits inside one launch.  Windows at the start, across the 2^32 boundary and at the ragged
+    end are checked against the oracle; the rest through the fused == split identity."""
+    n = (1 << 32) + 777
+    free, _ = torch.cuda.mem_get_info()
+    if free < 6 * n * 2 + (4 << 30):
+        pytest.skip('not enough free device memory for six 8 GiB arrays')
+    g = torch.Generator(device='cuda').manual_seed(99)
+    u = torch.empty(n, device='cuda', dtype=torch.float16).normal_(generator=g)
+    m = torch.empty(n, device='cuda', dtype=torch.float16).normal_(0, 0.1, generator=g)
+    v = torch.empty(n, device='cuda', dtype=torch.float16).normal_(0, 0.01, generator=g).abs_()
+    b1, b2, eps, er, count = 0.9, 0.999, 1e-3, 1e-4, 12
+    windows = [(0, 1 << 20), ((1 << 32) - (1 << 19), (1 << 32) + 777), (n - 4099, n)]
+    saved = [[t[a:b].cpu().numpy() for t in (u, m, v)] for a, b in windows]
+    m1 = adam_op.forward_mu(u, m, b1)
+    v1 = adam_op.forward_nu(u, v, b2)
+    u1 = adam_op.forward_updates(m1, v1, b1, b2, eps, er, count)
+    adam_op.forward_(u, m, v, b1, b2, eps, er, count)
+    assert torch.equal(u, u1) and torch.equal(m, m1) and torch.equal(v, v1)
+    for (a, b), (hu, hm, hv) in zip(windows, saved):
+        eu, em, ev = O.forward_inplace(hu, hm, hv, b1, b2, eps, er, count)
+        assert_bit_equal(u[a:b].cpu().numpy(), eu, f'updates[{a}:{b}]')
+        assert_bit_equal(m[a:b].cpu().numpy(), em, f'mu[{a}:{b}]')
+        assert_bit_equal(v[a:b].cpu().numpy(), ev, f'nu[{a}:{b}]')
