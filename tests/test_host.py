@@ -185,7 +185,12 @@ def test_fused_adam_argument_validation():
             FusedAdam(p, **kwargs)
     with pytest.raises(TypeError):
         FusedAdam([1.0])
-    opt = FusedAdam(p)
+    import torchopt_amd
+
+    # the reference's class names and its `use_accelerated_op` keyword carry over
+    assert torchopt_amd.Adam is FusedAdam and torchopt_amd.AdamW is torchopt_amd.FusedAdamW
+    assert torchopt_amd.AdamW(p, use_accelerated_op=True).weight_decay == 1e-2
+    opt = FusedAdam(p, use_accelerated_op=True)
     assert opt.state_dict() == (None,)
     opt.zero_grad()  # no grads yet: nothing to do
     assert opt.step() is None  # no grads: nothing is launched, counts stay at zero

@@ -12,7 +12,7 @@ from torchopt_amd.accelerated_op import AdamOp, MultiAdamOp
 from torchopt_amd.accelerated_op import is_available as accelerated_op_available
 from torchopt_amd.alias import adam, adamw, apply_updates, chain
 from torchopt_amd.meta import MetaAdam, MetaAdamW
-from torchopt_amd.optim import FusedAdam, FusedAdamW
+from torchopt_amd.optim import Adam, AdamW, FusedAdam, FusedAdamW
 
 # `import torchopt_amd._C.adam_op` should work like `from torchopt_amd._C import adam_op`
 from torchopt_amd import _C  # noqa: E402
@@ -21,5 +21,5 @@ _sys.modules.setdefault('torchopt_amd._C.adam_op', _C.adam_op)
 
 __version__ = '0.1.0'
 
-__all__ = ['AdamOp', 'FusedAdam', 'FusedAdamW', 'MetaAdam', 'MetaAdamW', 'MultiAdamOp', 'accelerated_op',
+__all__ = ['Adam', 'AdamOp', 'AdamW', 'FusedAdam', 'FusedAdamW', 'MetaAdam', 'MetaAdamW', 'MultiAdamOp', 'accelerated_op',
            'accelerated_op_available', 'adam', 'adamw', 'apply_updates', 'chain']

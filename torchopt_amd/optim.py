@@ -27,7 +27,7 @@ from torchopt_amd.accelerated_op.adam_op import adam_op
 from torchopt_amd.transform.scale_by_adam import ScaleByAdamState, _inc_counts, _remember
 
 
-__all__ = ['FusedAdam', 'FusedAdamW']
+__all__ = ['Adam', 'AdamW', 'FusedAdam', 'FusedAdamW']
 
 
 class FusedAdam:
@@ -46,7 +46,11 @@ class FusedAdam:
         *,
         eps_root: float = 0.0,
         maximize: bool = False,
+        use_accelerated_op: bool = True,
     ) -> None:
+        # `use_accelerated_op` is accepted so that the reference's constructor calls carry over
+        # (optim/adam.py:56-65); the fused operator is the only path here either way
+        del use_accelerated_op
         if callable(lr):
             raise ValueError('FusedAdam takes a constant learning rate; schedules are not fused')
         if not lr >= 0.0:
@@ -135,6 +139,11 @@ class FusedAdamW(FusedAdam):
 
     def __init__(self, params, lr: float = 1e-3, betas=(0.9, 0.999), eps: float = 1e-8,
                  weight_decay: float = 1e-2, *, eps_root: float = 0.0,
-                 maximize: bool = False) -> None:
+                 maximize: bool = False, use_accelerated_op: bool = True) -> None:
         super().__init__(params, lr, betas, eps, weight_decay, eps_root=eps_root,
-                         maximize=maximize)
+                         maximize=maximize, use_accelerated_op=use_accelerated_op)
+
+
+# the reference's class names (torchopt.Adam / torchopt.AdamW)
+Adam = FusedAdam
+AdamW = FusedAdamW
