@@ -258,7 +258,7 @@ def run_gpu(cfg_id, steps, warmup):
 
             def step():  # noqa: F811
                 rc = lib.toa_adam_fused_step_multi(code, num, pp, pu, pm, pv, ns, B1, B2, EPS,
-                                                   eps_root, None, count, lr, 0, 0, sptr)
+                                                   eps_root, None, count, lr, 0.0, 0, 0, 0, sptr)
                 if rc:
                     raise RuntimeError(lib.toa_adam_error_string(rc).decode())
             bytes_per_elem = 7 * esize  # reads g, mu, nu, p; writes mu, nu, p

@@ -1,0 +1,33 @@
+"""The benchmark's own configurations run end to end (few steps, no CPU leg) and report a
+plausible line: keeps bench.py in step with the C ABI."""
+
+from __future__ import annotations
+
+import json
+
+import pytest
+import torch
+
+import bench
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize('cfg', sorted(bench.CONFIGS))
+def test_bench_config_runs(cfg, capsys):
+    assert torch.cuda.is_available()
+    assert bench.main(['--config', str(cfg), '--steps', '3', '--warmup', '1',
+                       '--no-cpu-baseline']) == 0
+    line = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    assert line['n_gpus'] == 1 and line['steps'] == 3 and line['unit'] == 'elements/s'
+    assert line['value'] > 0 and line['ms_per_step'] > 0
+    assert line['config']['workload'] == bench.CONFIGS[cfg]['name']
+    roof = line['roofline']
+    assert roof['bound'] == 'hbm' and roof['peak'] == 8000.0 and roof['unit'] == 'GB/s'
+    assert roof['achieved'] > 0 and roof['frac'] > 0
+    torch.cuda.empty_cache()
+
+
+def test_bench_refuses_more_than_one_gpu(capsys):
+    assert bench.main(['--gpus', '2']) == 2
+    assert 'one GPU' in capsys.readouterr().err
