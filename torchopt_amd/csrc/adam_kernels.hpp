@@ -13,10 +13,12 @@
 //     waves run at once.  Coarser tiles, contiguous per-workgroup chunks and
 //     persistent grid-stride grids all measured 5-20 % slower on the
 //     read-modify-write stream;
-//   * residency is capped per op (kWavesPerCU, enforced through a dynamic-LDS
+//   * residency is capped per op (kWavesPerCU for the single-tensor kernel,
+//     kWavesPerCUMulti for the multi-tensor one, enforced through a dynamic-LDS
 //     reservation made at launch): more bytes in flight than the memory
-//     system needs only lengthens queues and widens the window.  The in-place
-//     step peaks at 13 waves per CU, the out-of-place ops at 24-32;
+//     system needs only lengthens queues and widens the window.  LDS granules
+//     make 32, 25, 21, 18, 16, 14, 12, 11, 10 ... the levels that exist; the
+//     in-place step peaks at 12 waves per CU, the out-of-place ops at 18-32;
 //   * every array is touched once, so loads and stores carry the
 //     non-temporal hint (worth ~10 %).
 //
@@ -185,9 +187,17 @@ __device__ __forceinline__ double toa_sqrt(double x) { return sqrt(x); }
 template <class F>
 __device__ __forceinline__ float toa_sqrt(R16<F> x) { return sqrtf((float)x); }
 
+// Residency level by element type: 4- and 8-byte types behave alike; the 16-bit types spend
+// twice the ALU time per byte on re-rounding and want more waves, bfloat16 (no native
+// arithmetic) the most.
+template <typename T>
+constexpr int waves_by_type(int wide, int half, int bfloat) {
+    return sizeof(T) != 2 ? wide : (__is_same(T, bfloat_t) ? bfloat : half);
+}
+
 // ---------------------------------------------------------------------------
 // Element-wise ops.  Pointer slots: inputs first, then outputs; an in-place op
-// writes output j back to input slot out_slot(j).  kWavesPerCU is the measured
+// writes output j back to input slot out_slot(j).  kWavesPerCU / kWavesPerCUMulti are the measured
 // best number of resident single-wave workgroups per compute unit.
 // ---------------------------------------------------------------------------
 
@@ -195,9 +205,9 @@ __device__ __forceinline__ float toa_sqrt(R16<F> x) { return sqrtf((float)x); }
 template <typename T>
 struct ForwardInplace {
     static constexpr int NIN = 3, NOUT = 3, NPTR = 3;
-    // read-modify-write: a tight window wins; the 16-bit types spend twice the ALU time per
-    // byte on conversions and want more waves to hide it
-    static constexpr int kWavesPerCU = sizeof(T) == 2 ? 22 : 13;
+    // read-modify-write: a tight window wins
+    static constexpr int kWavesPerCU = waves_by_type<T>(12, 18, 25);
+    static constexpr int kWavesPerCUMulti = waves_by_type<T>(16, 21, 32);
     // outputs are produced as (mu', nu', updates') and stored in that order
     __device__ static constexpr int out_slot(int j) { return j == 0 ? 1 : (j == 1 ? 2 : 0); }
     T b1, b2, c1, c2, eps, eps_root;
@@ -217,7 +227,8 @@ struct ForwardInplace {
 template <typename T>
 struct ForwardMu {
     static constexpr int NIN = 2, NOUT = 1, NPTR = 3;
-    static constexpr int kWavesPerCU = 24;
+    static constexpr int kWavesPerCU = waves_by_type<T>(25, 32, 32);
+    static constexpr int kWavesPerCUMulti = 32;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T b1;
     __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
@@ -229,7 +240,8 @@ struct ForwardMu {
 template <typename T>
 struct ForwardNu {
     static constexpr int NIN = 2, NOUT = 1, NPTR = 3;
-    static constexpr int kWavesPerCU = 24;
+    static constexpr int kWavesPerCU = waves_by_type<T>(25, 32, 32);
+    static constexpr int kWavesPerCUMulti = 32;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T b2;
     __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
@@ -243,6 +255,7 @@ template <typename T>
 struct ForwardUpdates {
     static constexpr int NIN = 2, NOUT = 1, NPTR = 3;
     static constexpr int kWavesPerCU = 32;  // sqrt and divide: needs the waves to hide ALU time
+    static constexpr int kWavesPerCUMulti = 32;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T c1, c2, eps, eps_root;
     __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
@@ -256,7 +269,8 @@ struct ForwardUpdates {
 template <typename T>
 struct BackwardMu {
     static constexpr int NIN = 1, NOUT = 2, NPTR = 3;
-    static constexpr int kWavesPerCU = 24;
+    static constexpr int kWavesPerCU = 21;
+    static constexpr int kWavesPerCUMulti = 25;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T b1;
     __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
@@ -269,7 +283,8 @@ struct BackwardMu {
 template <typename T>
 struct BackwardNu {
     static constexpr int NIN = 2, NOUT = 2, NPTR = 4;
-    static constexpr int kWavesPerCU = 24;
+    static constexpr int kWavesPerCU = 21;
+    static constexpr int kWavesPerCUMulti = 25;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T b2;
     __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
@@ -283,7 +298,8 @@ struct BackwardNu {
 template <typename T>
 struct BackwardUpdates {
     static constexpr int NIN = 3, NOUT = 2, NPTR = 5;
-    static constexpr int kWavesPerCU = 24;
+    static constexpr int kWavesPerCU = 18;
+    static constexpr int kWavesPerCUMulti = 25;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T p1, q2;
     __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
@@ -306,7 +322,8 @@ struct BackwardUpdates {
 template <typename T>
 struct ForwardAll {
     static constexpr int NIN = 3, NOUT = 3, NPTR = 6;
-    static constexpr int kWavesPerCU = 16;  // six streams per wave: few waves fill the queues
+    static constexpr int kWavesPerCU = waves_by_type<T>(14, 18, 18);  // six streams per wave: few waves fill the queues
+    static constexpr int kWavesPerCUMulti = waves_by_type<T>(18, 21, 21);
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T b1, b2, c1, c2, eps, eps_root;
     __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
@@ -333,7 +350,8 @@ template <typename T, bool HAS_DM, bool HAS_DV>
 struct BackwardAll {
     static constexpr int NIN = 4 + (HAS_DM ? 1 : 0) + (HAS_DV ? 1 : 0), NOUT = 3,
                          NPTR = NIN + NOUT;
-    static constexpr int kWavesPerCU = 14;  // seven to nine streams per wave
+    static constexpr int kWavesPerCU = waves_by_type<T>(11, 14, 14);  // seven to nine streams per wave
+    static constexpr int kWavesPerCUMulti = waves_by_type<T>(14, 16, 16);
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T b1, b2, p1, q2;
     __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
@@ -376,7 +394,8 @@ __device__ __forceinline__ double toa_fma(double a, double b, double c) { return
 template <typename T, bool WRITE_UPDATES>
 struct FusedStep {
     static constexpr int NIN = 4, NOUT = WRITE_UPDATES ? 4 : 3, NPTR = 4;
-    static constexpr int kWavesPerCU = 13;
+    static constexpr int kWavesPerCU = 12;
+    static constexpr int kWavesPerCUMulti = 16;
     // outputs: mu', nu', params', then the scaled update
     __device__ static constexpr int out_slot(int j) { return j == 3 ? 0 : j + 1; }
     T b1, b2, c1, c2, eps, eps_root, neg_lr, wd;

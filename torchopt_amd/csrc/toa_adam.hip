@@ -25,10 +25,14 @@ using namespace toa;
 constexpr int kUnroll = 1;           // one 16-byte access per lane per stream
 constexpr bool kNonTemporal = true;  // every array is touched once
 constexpr unsigned kMaxGrid = 1u << 25;  // default cap on workgroups per launch
-constexpr int kLdsPerCU = 160 * 1024;    // gfx950
-// The multi-tensor kernel spends three dependent scalar loads finding its tensor
-// before any memory traffic starts; a few more resident waves cover that.
-constexpr int kMultiExtraWaves = 4;
+// LDS of a gfx950 compute unit: 160 KiB handed out in granules of 1280 bytes (128 per CU).  A
+// single-wave workgroup that reserves g granules therefore limits residency to floor(128 / g)
+// workgroups per CU: 32 (no reservation; the wave-slot limit), 25, 21, 18, 16, 14, 12, 11, 10,
+// 9, 8 ...  Measured on MI355X with a kernel that counts its concurrently resident workgroups:
+// 12 800 bytes -> 12 per CU, 12 801 -> 11; 6 400 -> 25, 6 401 -> 21.
+constexpr int kLdsGranule = 1280;
+constexpr int kLdsGranulesPerCU = 128;
+constexpr int kMaxWavesPerCU = 32;
 
 // Global override of the per-op resident-wave cap: -1 = not yet initialised,
 // 0 = use each op's own kWavesPerCU, 1..32 = that many for every op.  Set by
@@ -42,21 +46,34 @@ int waves_override() {
         w = 0;
         if (const char *env = std::getenv("TOA_ADAM_WAVES_PER_CU")) {
             const int v = std::atoi(env);
-            if (v >= 1 && v <= 32) w = v;
+            if (v >= 1 && v <= kMaxWavesPerCU) w = v;
         }
         g_waves_override.store(w, std::memory_order_relaxed);
     }
     return w;
 }
 
-// Dynamic LDS bytes that let exactly `waves` single-wave workgroups fit on a CU.
-// The kernels never touch LDS; the reservation only bounds residency.
+// Dynamic LDS bytes that hold residency to the largest achievable level not above `waves`
+// single-wave workgroups per CU.  The kernels never touch LDS; the reservation only bounds
+// residency.
+constexpr unsigned lds_for_waves(int waves) {
+    if (waves >= kMaxWavesPerCU) return 0;
+    if (waves < 1) waves = 1;
+    // smallest g with floor(128 / g) <= waves
+    return (unsigned)((kLdsGranulesPerCU / (waves + 1) + 1) * kLdsGranule);
+}
+static_assert(lds_for_waves(12) == 12800 && lds_for_waves(13) == 12800, "12 per CU");
+static_assert(lds_for_waves(14) == 11520 && lds_for_waves(16) == 10240, "14 and 16 per CU");
+static_assert(lds_for_waves(25) == 6400 && lds_for_waves(24) == 7680, "25 and 21 per CU");
+static_assert(lds_for_waves(31) == 6400 && lds_for_waves(32) == 0, "25, then no reservation");
+static_assert(lds_for_waves(1) == 65 * 1280, "one per CU: more than half of the LDS");
+
+// The multi-tensor kernel spends three dependent scalar loads finding its tensor before any
+// memory traffic starts, so its best level sits one or two steps above the single-tensor one.
 template <class Op>
-unsigned lds_reservation(int extra_waves = 0) {
+unsigned lds_reservation(bool multi) {
     const int o = waves_override();
-    const int w = o ? o : Op::kWavesPerCU + extra_waves;
-    if (w >= 32) return 0;  // 32 waves per CU is the hardware limit anyway
-    return (unsigned)((kLdsPerCU / w) & ~1023);
+    return lds_for_waves(o ? o : (multi ? Op::kWavesPerCUMulti : Op::kWavesPerCU));
 }
 
 // Workgroups per launch are capped; a tensor with more tiles than the cap is covered by the
@@ -91,7 +108,7 @@ int launch_single(const Op &op, T *const (&ptrs)[Op::NPTR], size_t n, void *stre
     constexpr size_t tile = Tile<T, kUnroll>::ELEMS;
     const size_t num_tiles = (n + tile - 1) / tile;
     hipLaunchKernelGGL((stream_kernel<T, Op, kUnroll, kNonTemporal>), dim3(grid_for(num_tiles)),
-                       dim3(kBlock), lds_reservation<Op>(), (hipStream_t)stream, op, tp, n,
+                       dim3(kBlock), lds_reservation<Op>(false), (hipStream_t)stream, op, tp, n,
                        num_tiles);
     return (int)hipGetLastError();
 }
@@ -148,7 +165,7 @@ int launch_multi(MakeOp make_op, size_t num_tensors,
             tab.total = next_tile;
             hipLaunchKernelGGL((multi_stream_kernel<T, Op, kUnroll, kNonTemporal>),
                                dim3(grid_for(next_tile)), dim3(kBlock),
-                               lds_reservation<Op>(kMultiExtraWaves), (hipStream_t)stream, op,
+                               lds_reservation<Op>(true), (hipStream_t)stream, op,
                                tab);
             reset();
             return (int)hipGetLastError();
@@ -281,7 +298,7 @@ int toa_adam_abi_version(void) { return 2; }
 
 int toa_adam_set_waves_per_cu(int waves) {
     const int prev = waves_override();
-    g_waves_override.store(waves >= 1 && waves <= 32 ? waves : 0, std::memory_order_relaxed);
+    g_waves_override.store(waves >= 1 && waves <= kMaxWavesPerCU ? waves : 0, std::memory_order_relaxed);
     return prev;
 }
 
