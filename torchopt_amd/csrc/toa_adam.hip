@@ -70,10 +70,17 @@ static_assert(lds_for_waves(1) == 65 * 1280, "one per CU: more than half of the 
 
 // The multi-tensor kernel spends three dependent scalar loads finding its tensor before any
 // memory traffic starts, so its best level sits one or two steps above the single-tensor one.
+// A launch that fits on the chip in one round (256 CUs x 32 wave slots) is latency-bound, not
+// bandwidth-bound: capping residency would only add rounds (2^21 float32 elements in place:
+// 8.8 us capped, 6.5 us uncapped), so such launches run without a reservation.
+constexpr size_t kOneRoundTiles = 256 * kMaxWavesPerCU;
+
 template <class Op>
-unsigned lds_reservation(bool multi) {
+unsigned lds_reservation(bool multi, size_t num_tiles) {
     const int o = waves_override();
-    return lds_for_waves(o ? o : (multi ? Op::kWavesPerCUMulti : Op::kWavesPerCU));
+    if (o) return lds_for_waves(o);
+    if (num_tiles <= kOneRoundTiles) return 0;
+    return lds_for_waves(multi ? Op::kWavesPerCUMulti : Op::kWavesPerCU);
 }
 
 // Workgroups per launch are capped; a tensor with more tiles than the cap is covered by the
@@ -108,7 +115,8 @@ int launch_single(const Op &op, T *const (&ptrs)[Op::NPTR], size_t n, void *stre
     constexpr size_t tile = Tile<T, kUnroll>::ELEMS;
     const size_t num_tiles = (n + tile - 1) / tile;
     hipLaunchKernelGGL((stream_kernel<T, Op, kUnroll, kNonTemporal>), dim3(grid_for(num_tiles)),
-                       dim3(kBlock), lds_reservation<Op>(false), (hipStream_t)stream, op, tp, n,
+                       dim3(kBlock), lds_reservation<Op>(false, num_tiles), (hipStream_t)stream, op, tp,
+                       n,
                        num_tiles);
     return (int)hipGetLastError();
 }
@@ -165,7 +173,7 @@ int launch_multi(MakeOp make_op, size_t num_tensors,
             tab.total = next_tile;
             hipLaunchKernelGGL((multi_stream_kernel<T, Op, kUnroll, kNonTemporal>),
                                dim3(grid_for(next_tile)), dim3(kBlock),
-                               lds_reservation<Op>(true), (hipStream_t)stream, op,
+                               lds_reservation<Op>(true, next_tile), (hipStream_t)stream, op,
                                tab);
             reset();
             return (int)hipGetLastError();
