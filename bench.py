@@ -16,6 +16,11 @@ Beside the headline `value` (elements per second) the line carries
   cpu_baseline  the reference's CPU op (or this repo's bit-identical C port of it) timed on the
                 host's cores on a bounded sample of the same workload.
 
+`--ceiling` measures, instead of the operator, what this machine's HBM delivers to streaming
+kernels of the same launch shape that do next to no arithmetic (bench_probe.hip: R arrays read,
+W arrays written, at every residency level), and prints those ceilings as one JSON line: the
+context for `roofline.frac`.
+
 Everything on one GPU: `--gpus N` with N > 1 is refused.
 """
 
@@ -325,6 +330,78 @@ def run_gpu(cfg_id, steps, warmup):
     }
 
 
+# ----------------------------------------------------------------------------- HBM ceilings
+
+PROBE_SRC = os.path.join(REPO, 'bench_probe.hip')
+PROBE_LIB = os.path.join(REPO, 'bench_probe.so')
+RESIDENCY_LEVELS = (32, 25, 21, 18, 16, 14, 12, 11, 10, 9, 8)  # floor(128 / LDS granules)
+
+
+def build_probe():
+    """hipcc -> bench_probe.so (cross-compiles without a GPU)."""
+    import subprocess
+
+    subprocess.run(['hipcc', '-O3', '-std=c++17', '--offload-arch=gfx950', '-fPIC', '-shared',
+                    '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
+                    '-fvisibility=hidden', '-o', PROBE_LIB, PROBE_SRC], check=True,
+                   stderr=subprocess.DEVNULL)
+    return PROBE_LIB
+
+
+def lds_for_waves(waves):
+    """Dynamic LDS per single-wave workgroup that caps a gfx950 CU (128 granules of 1280 B) at
+    `waves` resident workgroups."""
+    return 0 if waves >= 32 else (128 // (waves + 1) + 1) * 1280
+
+
+def run_ceiling(array_bytes=1 << 30, reps=20):
+    import ctypes
+
+    import torch
+
+    if not os.path.exists(PROBE_LIB):
+        build_probe()
+    probe = ctypes.CDLL(PROBE_LIB)
+    probe.bench_probe_stream.restype = ctypes.c_int
+    probe.bench_probe_stream.argtypes = [ctypes.c_int, ctypes.c_int,
+                                         ctypes.POINTER(ctypes.c_void_p), ctypes.c_size_t,
+                                         ctypes.c_uint, ctypes.c_void_p]
+    stream = torch.cuda.current_stream()
+    arrays = [torch.rand(array_bytes // 4, device='cuda') for _ in range(7)]
+    torch.cuda.synchronize()
+    out = {}
+    shapes = [(r, w, False) for r, w in ((1, 0), (3, 0), (0, 1), (0, 3), (1, 1), (2, 1), (3, 3),
+                                         (4, 3))]
+    shapes += [(3, 3, True), (4, 3, True)]  # written back over the arrays just read, as forward_
+    for reads, writes, in_place in shapes:
+        order = list(range(reads)) + (list(range(reads - writes, reads)) if in_place
+                                      else list(range(reads, reads + writes)))
+        ptrs = (ctypes.c_void_p * (reads + writes))(*[arrays[k].data_ptr() for k in order])
+        best = (0.0, None)
+        for waves in RESIDENCY_LEVELS:
+            def launch():
+                rc = probe.bench_probe_stream(reads, writes, ptrs, array_bytes,
+                                              lds_for_waves(waves), stream.cuda_stream)
+                if rc:
+                    raise RuntimeError(f'bench_probe_stream({reads}, {writes}) returned {rc}')
+            for _ in range(4):
+                launch()
+            ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            ev0.record(stream)
+            for _ in range(reps):
+                launch()
+            ev1.record(stream)
+            torch.cuda.synchronize()
+            gbs = (reads + writes) * array_bytes / (ev0.elapsed_time(ev1) / reps * 1e-3) / 1e9
+            if gbs > best[0]:
+                best = (gbs, waves)
+        out[f'{reads}R{writes}W' + (' in place' if in_place else '')] = {'GB/s': round(best[0], 1), 'frac_of_peak': round(
+            best[0] / HBM_PEAK_GBS, 4), 'waves_per_cu': best[1]}
+    return {'metric': 'hbm_streaming_ceiling', 'unit': 'GB/s', 'peak': HBM_PEAK_GBS,
+            'array_bytes': array_bytes, 'launches_timed': reps,
+            'device': torch.cuda.get_device_name(0), 'ceilings': out}
+
+
 # ----------------------------------------------------------------------------- CPU baseline
 
 
@@ -408,6 +485,9 @@ def main(argv=None):
                     help='after the timed region also run 5 plain device copies of 1 GiB, so a '
                          'rocprofv3 --pmc run holds a kernel of known traffic to scale '
                          'FETCH_SIZE / WRITE_SIZE by')
+    ap.add_argument('--ceiling', action='store_true',
+                    help='measure the streaming ceilings of this machine (probe kernels with '
+                         'the operator\'s launch shape) instead of the operator')
     args = ap.parse_args(argv)
 
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
@@ -415,6 +495,10 @@ def main(argv=None):
               'GPUs; each would run the same kernel on its shard). Run with --gpus 1.',
               file=sys.stderr)
         return 2
+
+    if args.ceiling:
+        print(json.dumps(run_ceiling()), flush=True)
+        return 0
 
     gpu = run_gpu(args.config, args.steps, args.warmup)
     cfg = CONFIGS[args.config]

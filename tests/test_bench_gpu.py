@@ -31,3 +31,13 @@ def test_bench_config_runs(cfg, capsys):
 def test_bench_refuses_more_than_one_gpu(capsys):
     assert bench.main(['--gpus', '2']) == 2
     assert 'one GPU' in capsys.readouterr().err
+
+
+def test_ceiling_probe_runs():
+    """The arithmetic-free probes behind `bench.py --ceiling`, on small arrays."""
+    out = bench.run_ceiling(array_bytes=1 << 26, reps=3)
+    assert out['unit'] == 'GB/s' and out['peak'] == 8000.0
+    assert {'3R0W', '0R3W', '1R1W', '3R3W', '3R3W in place', '4R3W in place'} <= set(out['ceilings'])
+    for row in out['ceilings'].values():
+        assert row['GB/s'] > 0 and row['waves_per_cu'] in bench.RESIDENCY_LEVELS
+    torch.cuda.empty_cache()
