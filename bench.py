@@ -14,7 +14,8 @@ Beside the headline `value` (elements per second) the line carries
                 float32 element for forward_) over the average launch duration, measured with
                 events on the launch stream across the timed region, against 8 TB/s;
   cpu_baseline  the reference's CPU op (or this repo's bit-identical C port of it) timed on the
-                host's cores on a bounded sample of the same workload.
+                host's cores on a bounded sample of the same workload, and with it the parity of
+                the GPU's result with the CPU's on that sample (differing elements, max ulp).
 
 `--ceiling` measures, instead of the operator, what this machine's HBM delivers to streaming
 kernels of the same launch shape that do next to no arithmetic (bench_probe.hip: R arrays read,
@@ -454,7 +455,32 @@ def run_cpu_baseline(cfg_id, budget_s=12.0):
             adam_oracle.forward_inplace(u, mu, nu, B1, B2, EPS, cfg['eps_root'], cfg['count'])
         kind = 'port'
 
-    one()  # warm-up (threads, page faults)
+    # Parity on this sample: the GPU's first application from the seeded state against the
+    # CPU's (which doubles as the CPU warm-up: threads, page faults).
+    import torch
+
+    from torchopt_amd import _lib
+
+    dev = [torch.from_numpy(a).cuda() for a in (u, mu, nu)]
+    rc = _lib.load().toa_adam_forward_inplace(
+        _lib.TOA_F32 if cfg['dtype'] == 'f32' else _lib.TOA_F64, dev[0].data_ptr(),
+        dev[1].data_ptr(), dev[2].data_ptr(), n, B1, B2, EPS, cfg['eps_root'], cfg['count'],
+        torch.cuda.current_stream().cuda_stream)
+    if rc:
+        raise RuntimeError(f'toa_adam_forward_inplace returned {rc}')
+    one()
+    itype = np.int32 if np_dtype is np.float32 else np.int64
+    worst, differing = 0, 0
+    for got, want in zip(dev, (u, mu, nu)):
+        a = got.cpu().numpy().view(itype).astype(np.int64)
+        b = want.view(itype).astype(np.int64)
+        lo = np.iinfo(itype).min
+        a, b = np.where(a < 0, lo - a, a), np.where(b < 0, lo - b, b)  # monotone integer line
+        d = np.abs(a - b)
+        worst, differing = max(worst, int(d.max())), differing + int(np.count_nonzero(d))
+    del dev
+    parity = {'elements_checked': 3 * n, 'differing': differing, 'max_ulp': worst}
+
     times = []
     t_end = time.perf_counter() + budget_s
     while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 25):
@@ -468,6 +494,7 @@ def run_cpu_baseline(cfg_id, budget_s=12.0):
         'sample': f'{n} of {full} elements ({cfg["dtype"]}), forward_ in place, '
                   f'median of {len(times)} passes after 1 warm-up',
         'gb_per_s': round(BYTES_PER_ELEM['forward_'] * esize * n / med / 1e9, 2),
+        'parity_gpu_vs_cpu': parity,
     }
 
 
