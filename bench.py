@@ -311,6 +311,21 @@ def run_gpu(cfg_id, steps, warmup):
     torch.cuda.synchronize()
     t1 = time.perf_counter()
 
+    # per-step spread, from a second short pass with one pair of events per step (outside the
+    # timed region; event overhead makes it meaningless for microsecond steps)
+    spread = {}
+    if (t1 - t0) * 1e3 / steps > 0.05:
+        pairs = []
+        for _ in range(min(steps, 20)):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(stream)
+            step()
+            b.record(stream)
+            pairs.append((a, b))
+        torch.cuda.synchronize()
+        each = sorted(a.elapsed_time(b) for a, b in pairs)
+        spread = {'step_ms_min': round(each[0], 5), 'step_ms_median': round(each[len(each) // 2], 5)}
+
     wall_ms = (t1 - t0) * 1e3 / steps
     kern_ms = ev0.elapsed_time(ev1) / steps  # stream time per launch (launches are back to back)
     alg_bytes = bytes_per_elem * total
@@ -324,7 +339,7 @@ def run_gpu(cfg_id, steps, warmup):
             'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
             'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': traffic,
             'kernel_ms': round(kern_ms, 5), 'algorithmic_bytes_per_launch': alg_bytes,
-            'bytes_per_element': bytes_per_elem,
+            'bytes_per_element': bytes_per_elem, **spread,
         },
         'extra': extra,
         'device': torch.cuda.get_device_name(0),
