@@ -269,3 +269,42 @@ def test_chain_reduces_to_torch_optim_adam(inplace):
         optim_ref.step()
     for p, q, p0 in zip(model.parameters(), ref.parameters(), base):
         torch.testing.assert_close(p - p0, q - p0, rtol=25 * 1e-7, atol=25 * 1e-7)
+
+
+def test_expanded_and_permuted_gradients_on_the_differentiable_branch():
+    """Gradients straight out of `torch.autograd.grad` may be expanded (stride 0, as the
+    gradient of a sum is) or laid out differently from the moments; the list ops bring them to
+    the moments' memory order instead of misreading them."""
+    torch.manual_seed(5)
+    shapes = [(6, 40), (33,), (4, 3, 5, 5)]
+    mu = [0.1 * torch.randn(s, device='cuda', dtype=torch.float64) for s in shapes]
+    nu = [(0.01 * torch.randn(s, device='cuda', dtype=torch.float64)).abs_() for s in shapes]
+    grads = [torch.tensor(0.5, device='cuda', dtype=torch.float64).expand(shapes[0]),  # stride 0
+             torch.randn(66, device='cuda', dtype=torch.float64)[::2],  # strided slice
+             torch.randn(shapes[2], device='cuda', dtype=torch.float64).contiguous(
+                 memory_format=torch.channels_last)]
+    assert not grads[0].is_contiguous() and not grads[1].is_contiguous()
+    leaves = [g.detach().clone().requires_grad_(True) for g in grads]  # dense stand-ins
+    op = MultiAdamOp(B1, B2, EPS, eps_root=1e-8, inplace=False)
+    want = op([m.clone() for m in mu], [v.clone() for v in nu], leaves, 4)
+    got = op([m.clone() for m in mu], [v.clone() for v in nu], grads, 4)
+    for a, b in zip(sum(map(list, got), []), sum(map(list, want), [])):
+        assert a.shape == b.shape
+        assert_bit_equal(host(a.contiguous()), host(b.contiguous()), 'values')
+    # and the backward pass reads the saved non-dense gradients correctly
+    gl = [g.detach().requires_grad_(True) for g in grads]
+    out = op([m.clone() for m in mu], [v.clone() for v in nu], gl, 4)
+    total = sum((u * u).sum() for u in out[2])
+    dg = torch.autograd.grad(total, gl)
+    total_ref = sum((u * u).sum() for u in want[2])
+    dg_ref = torch.autograd.grad(total_ref, leaves)
+    for a, b in zip(dg, dg_ref):
+        assert_bit_equal(host(a.contiguous()), host(b.contiguous()), 'gradients')
+
+
+def test_inplace_branch_refuses_gradients_it_cannot_overwrite():
+    mu = [torch.zeros(6, 40, device='cuda')]
+    nu = [torch.zeros(6, 40, device='cuda')]
+    g = [torch.tensor(0.5, device='cuda').expand(6, 40)]
+    with pytest.raises(RuntimeError, match='dense'):
+        MultiAdamOp(inplace=True)(mu, nu, g, 1)

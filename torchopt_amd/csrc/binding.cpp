@@ -87,6 +87,8 @@ bool sameLayout(const Tensor &a, const Tensor &b) {
 // (The reference makes incoming gradients .contiguous(), adam_op.cpp:107,123,143.)
 Tensor asLayoutOf(const Tensor &x, const Tensor &donor) {
     if (x.numel() <= 1 || (x.is_contiguous() && donor.is_contiguous())) return x;
+    // a wrong device or dtype is the gate's to report, not to be papered over by a copy
+    if (x.device() != donor.device() || x.scalar_type() != donor.scalar_type()) return x;
     if (x.sizes() == donor.sizes())
         return x.strides() == donor.strides() ? x : at::empty_like(donor).copy_(x);
     TORCH_CHECK(donor.is_contiguous(), "operands of different shapes must be contiguous");
@@ -441,7 +443,8 @@ TensorList asLayoutOfEach(const TensorList &xs, const TensorList &donors, const 
     return out;
 }
 
-const Tensor &firstNonEmpty(const TensorList &l) { return l[0]; }
+// Any member names the device of a list call (gateLists has checked they agree).
+const Tensor &deviceDonor(const TensorList &l) { return l[0]; }
 
 py::tuple forwardMultiInplace(const py::object &updates_o, const py::object &mu_o,
                               const py::object &nu_o, double b1, double b2, double eps,
@@ -453,7 +456,7 @@ py::tuple forwardMultiInplace(const py::object &updates_o, const py::object &mu_
     Lists l = gateLists(name, {&updates, &mu, &nu});
     if (l.num) {
         const Counts c = parseCounts(counts, l.num);
-        const OnDeviceOf dev(firstNonEmpty(updates));
+        const OnDeviceOf dev(deviceDonor(updates));
         check(toa_adam_forward_inplace_multi(l.code, l.num, l.ptr[0].data(), l.ptr[1].data(),
                                              l.ptr[2].data(), l.n.data(), b1, b2, eps, eps_root,
                                              c.data(), c.all, dev.stream()),
@@ -462,40 +465,43 @@ py::tuple forwardMultiInplace(const py::object &updates_o, const py::object &mu_
     return py::make_tuple(updates_o, mu_o, nu_o);  // the caller's own lists, mutated in place
 }
 
-TensorList forwardMuMulti(const TensorList &updates, const TensorList &mu, double b1) {
+TensorList forwardMuMulti(const TensorList &updates_in, const TensorList &mu, double b1) {
     const char *name = "adamForwardMuMulti";
     TensorList out = emptyLike(mu);
-    Lists l = gateLists(name, {&updates, &mu, &out});
+    const TensorList updates = asLayoutOfEach(updates_in, mu, name);
+    Lists l = gateLists(name, {&mu, &updates, &out});
     if (l.num) {
-        const OnDeviceOf dev(firstNonEmpty(mu));
-        check(toa_adam_forward_mu_multi(l.code, l.num, l.ptr[0].data(), l.ptr[1].data(),
+        const OnDeviceOf dev(deviceDonor(mu));
+        check(toa_adam_forward_mu_multi(l.code, l.num, l.ptr[1].data(), l.ptr[0].data(),
                                         l.n.data(), b1, l.ptr[2].data(), dev.stream()),
               name);
     }
     return out;
 }
 
-TensorList forwardNuMulti(const TensorList &updates, const TensorList &nu, double b2) {
+TensorList forwardNuMulti(const TensorList &updates_in, const TensorList &nu, double b2) {
     const char *name = "adamForwardNuMulti";
     TensorList out = emptyLike(nu);
-    Lists l = gateLists(name, {&updates, &nu, &out});
+    const TensorList updates = asLayoutOfEach(updates_in, nu, name);
+    Lists l = gateLists(name, {&nu, &updates, &out});
     if (l.num) {
-        const OnDeviceOf dev(firstNonEmpty(nu));
-        check(toa_adam_forward_nu_multi(l.code, l.num, l.ptr[0].data(), l.ptr[1].data(),
+        const OnDeviceOf dev(deviceDonor(nu));
+        check(toa_adam_forward_nu_multi(l.code, l.num, l.ptr[1].data(), l.ptr[0].data(),
                                         l.n.data(), b2, l.ptr[2].data(), dev.stream()),
               name);
     }
     return out;
 }
 
-TensorList forwardUpdatesMulti(const TensorList &new_mu, const TensorList &new_nu, double b1,
+TensorList forwardUpdatesMulti(const TensorList &new_mu, const TensorList &new_nu_in, double b1,
                                double b2, double eps, double eps_root, const py::object &counts) {
     const char *name = "adamForwardUpdatesMulti";
     TensorList out = emptyLike(new_mu);
+    const TensorList new_nu = asLayoutOfEach(new_nu_in, new_mu, name);
     Lists l = gateLists(name, {&new_mu, &new_nu, &out});
     if (l.num) {
         const Counts c = parseCounts(counts, l.num);
-        const OnDeviceOf dev(firstNonEmpty(new_mu));
+        const OnDeviceOf dev(deviceDonor(new_mu));
         check(toa_adam_forward_updates_multi(l.code, l.num, l.ptr[0].data(), l.ptr[1].data(),
                                              l.n.data(), b1, b2, eps, eps_root, c.data(), c.all,
                                              l.ptr[2].data(), dev.stream()),
@@ -508,27 +514,29 @@ std::tuple<TensorList, TensorList> backwardMuMulti(const TensorList &dmu_in,
                                                    const TensorList &updates,
                                                    const TensorList &mu, double b1) {
     const char *name = "adamBackwardMuMulti";
-    TensorList dupdates_out = emptyLike(updates), dmu_out = emptyLike(mu);
+    TORCH_CHECK(updates.size() == mu.size(), name, ": tensor lists differ in length");
+    TensorList dupdates_out = emptyLike(mu), dmu_out = emptyLike(mu);
     const TensorList dmu = asLayoutOfEach(dmu_in, dmu_out, name);
-    Lists l = gateLists(name, {&dmu, &dupdates_out, &dmu_out});
+    Lists l = gateLists(name, {&dmu_out, &dmu, &dupdates_out});
     if (l.num) {
-        const OnDeviceOf dev(firstNonEmpty(dmu));
-        check(toa_adam_backward_mu_multi(l.code, l.num, l.ptr[0].data(), l.n.data(), b1,
-                                         l.ptr[1].data(), l.ptr[2].data(), dev.stream()),
+        const OnDeviceOf dev(deviceDonor(dmu));
+        check(toa_adam_backward_mu_multi(l.code, l.num, l.ptr[1].data(), l.n.data(), b1,
+                                         l.ptr[2].data(), l.ptr[0].data(), dev.stream()),
               name);
     }
     return {dupdates_out, dmu_out};
 }
 
 std::tuple<TensorList, TensorList> backwardNuMulti(const TensorList &dnu_in,
-                                                   const TensorList &updates,
+                                                   const TensorList &updates_in,
                                                    const TensorList &nu, double b2) {
     const char *name = "adamBackwardNuMulti";
-    TensorList dupdates_out = emptyLike(updates), dnu_out = emptyLike(nu);
+    TensorList dupdates_out = emptyLike(nu), dnu_out = emptyLike(nu);
     const TensorList dnu = asLayoutOfEach(dnu_in, dnu_out, name);
+    const TensorList updates = asLayoutOfEach(updates_in, nu, name);
     Lists l = gateLists(name, {&dnu, &updates, &dupdates_out, &dnu_out});
     if (l.num) {
-        const OnDeviceOf dev(firstNonEmpty(dnu));
+        const OnDeviceOf dev(deviceDonor(dnu));
         check(toa_adam_backward_nu_multi(l.code, l.num, l.ptr[0].data(), l.ptr[1].data(),
                                          l.n.data(), b2, l.ptr[2].data(), l.ptr[3].data(),
                                          dev.stream()),
@@ -538,15 +546,17 @@ std::tuple<TensorList, TensorList> backwardNuMulti(const TensorList &dnu_in,
 }
 
 std::tuple<TensorList, TensorList> backwardUpdatesMulti(
-    const TensorList &dupdates_in, const TensorList &updates, const TensorList &new_mu,
+    const TensorList &dupdates_in, const TensorList &updates_in, const TensorList &new_mu,
     const TensorList &new_nu, double b1, double b2, double eps_root, const py::object &counts) {
     const char *name = "adamBackwardUpdatesMulti";
-    TensorList dmu_out = emptyLike(new_mu), dnu_out = emptyLike(new_nu);
+    TORCH_CHECK(new_nu.size() == new_mu.size(), name, ": tensor lists differ in length");
+    TensorList dmu_out = emptyLike(new_mu), dnu_out = emptyLike(new_mu);
     const TensorList dupdates = asLayoutOfEach(dupdates_in, dmu_out, name);
+    const TensorList updates = asLayoutOfEach(updates_in, new_mu, name);
     Lists l = gateLists(name, {&dupdates, &updates, &new_mu, &dmu_out, &dnu_out});
     if (l.num) {
         const Counts c = parseCounts(counts, l.num);
-        const OnDeviceOf dev(firstNonEmpty(dupdates));
+        const OnDeviceOf dev(deviceDonor(dupdates));
         check(toa_adam_backward_updates_multi(l.code, l.num, l.ptr[0].data(), l.ptr[1].data(),
                                               l.ptr[2].data(), l.n.data(), b1, b2, eps_root,
                                               c.data(), c.all, l.ptr[3].data(), l.ptr[4].data(),
@@ -557,14 +567,17 @@ std::tuple<TensorList, TensorList> backwardUpdatesMulti(
 }
 
 std::tuple<TensorList, TensorList, TensorList> forwardAllMulti(
-    const TensorList &updates, const TensorList &mu, const TensorList &nu, double b1, double b2,
-    double eps, double eps_root, const py::object &counts) {
+    const TensorList &updates_in, const TensorList &mu, const TensorList &nu_in, double b1,
+    double b2, double eps, double eps_root, const py::object &counts) {
     const char *name = "adamForwardAllMulti";
     TensorList new_mu = emptyLike(mu), new_nu = emptyLike(mu), new_updates = emptyLike(mu);
+    // gradients may arrive expanded or in another memory order: bring them to mu's
+    const TensorList updates = asLayoutOfEach(updates_in, mu, name);
+    const TensorList nu = asLayoutOfEach(nu_in, mu, name);
     Lists l = gateLists(name, {&updates, &mu, &nu, &new_mu, &new_nu, &new_updates});
     if (l.num) {
         const Counts c = parseCounts(counts, l.num);
-        const OnDeviceOf dev(firstNonEmpty(mu));
+        const OnDeviceOf dev(deviceDonor(mu));
         check(toa_adam_forward_all_multi(l.code, l.num, l.ptr[0].data(), l.ptr[1].data(),
                                          l.ptr[2].data(), l.n.data(), b1, b2, eps, eps_root,
                                          c.data(), c.all, l.ptr[3].data(), l.ptr[4].data(),
@@ -575,15 +588,17 @@ std::tuple<TensorList, TensorList, TensorList> forwardAllMulti(
 }
 
 // dnew_mu / dnew_nu: a list of outside gradients, or None when there are none at all (a list
-// may not mix tensors and None: the caller substitutes zeros for the missing members).
+// may not mix tensors and None: the caller substitutes -0.0 for the missing members).
 std::tuple<TensorList, TensorList, TensorList> backwardAllMulti(
     const TensorList &dnew_updates_in, const c10::optional<TensorList> &dnew_mu_in,
-    const c10::optional<TensorList> &dnew_nu_in, const TensorList &new_updates,
-    const TensorList &new_mu, const TensorList &updates, double b1, double b2, double eps_root,
-    const py::object &counts) {
+    const c10::optional<TensorList> &dnew_nu_in, const TensorList &new_updates_in,
+    const TensorList &new_mu, const TensorList &updates_in, double b1, double b2,
+    double eps_root, const py::object &counts) {
     const char *name = "adamBackwardAllMulti";
     TensorList dupdates = emptyLike(new_mu), dmu = emptyLike(new_mu), dnu = emptyLike(new_mu);
     const TensorList du = asLayoutOfEach(dnew_updates_in, new_mu, name);
+    const TensorList new_updates = asLayoutOfEach(new_updates_in, new_mu, name);
+    const TensorList updates = asLayoutOfEach(updates_in, new_mu, name);
     Lists l = gateLists(name, {&du, &new_updates, &new_mu, &updates, &dupdates, &dmu, &dnu});
     // outside gradients, brought to new_mu's layout; the (possibly copied) tensors live until
     // the launch below has been enqueued
@@ -600,7 +615,7 @@ std::tuple<TensorList, TensorList, TensorList> backwardAllMulti(
     collect(dnew_nu_in, &ext_v, &pv);
     if (l.num) {
         const Counts c = parseCounts(counts, l.num);
-        const OnDeviceOf dev(firstNonEmpty(new_mu));
+        const OnDeviceOf dev(deviceDonor(new_mu));
         check(toa_adam_backward_all_multi(
                   l.code, l.num, l.ptr[0].data(), l.ptr[1].data(), l.ptr[2].data(),
                   l.ptr[3].data(), dnew_mu_in.has_value() ? pm.data() : nullptr,
@@ -625,7 +640,7 @@ py::tuple fusedStepMulti(const py::object &params_o, const py::object &updates_o
     Lists l = gateLists(name, {&updates, &mu, &nu, &params});
     if (l.num) {
         const Counts c = parseCounts(counts, l.num);
-        const OnDeviceOf dev(firstNonEmpty(updates));
+        const OnDeviceOf dev(deviceDonor(updates));
         check(toa_adam_fused_step_multi(l.code, l.num, l.ptr[3].data(), l.ptr[0].data(),
                                         l.ptr[1].data(), l.ptr[2].data(), l.n.data(), b1, b2, eps,
                                         eps_root, c.data(), c.all, lr, weight_decay,
