@@ -186,3 +186,34 @@ def test_fused_adam_tracks_torch_optim_adam(cls, ref_cls, wd):
             opt.step()
     for p, q in zip(net.parameters(), ref.parameters()):
         torch.testing.assert_close(p, q, rtol=25e-7, atol=25e-7)
+
+
+def test_fused_adam_reads_gradients_in_any_layout():
+    """`p.grad` may be channels-last, expanded or a strided slice while the parameter is
+    contiguous: the step only reads it, so it is brought to the parameter's memory order."""
+    torch.manual_seed(11)
+    ps = [torch.randn(4, 3, 5, 5, device='cuda'), torch.randn(6, 40, device='cuda'),
+          torch.randn(33, device='cuda')]
+    grads = [torch.randn(4, 3, 5, 5, device='cuda').contiguous(memory_format=torch.channels_last),
+             torch.tensor(0.25, device='cuda').expand(6, 40),
+             torch.randn(66, device='cuda')[::2]]
+    a = [p.clone().requires_grad_(True) for p in ps]
+    b = [p.clone().requires_grad_(True) for p in ps]
+    opt_a, opt_b = FusedAdam(a, lr=0.01), FusedAdam(b, lr=0.01)
+    for _ in range(3):
+        for p, q, g in zip(a, b, grads):
+            p.grad, q.grad = g, g.contiguous()
+        opt_a.step()
+        opt_b.step()
+    for p, q in zip(a, b):
+        assert torch.equal(p, q)
+    # the single-tensor entry point likewise
+    p1, p2 = ps[0].clone(), ps[0].clone()
+    m, v = torch.zeros_like(p1), torch.zeros_like(p1)
+    adam_op.fused_step_(p1, grads[0], m, v, B1, B2, EPS, 0.0, 1, 0.01)
+    adam_op.fused_step_(p2, grads[0].contiguous(), torch.zeros_like(p2), torch.zeros_like(p2), B1,
+                        B2, EPS, 0.0, 1, 0.01)
+    assert torch.equal(p1, p2)
+    with pytest.raises(RuntimeError):  # a gradient that must be overwritten has to be dense
+        adam_op.fused_step_(p1, torch.tensor(0.25, device='cuda').expand(4, 3, 5, 5), m, v, B1,
+                            B2, EPS, 0.0, 2, 0.01, write_updates=True)

@@ -311,13 +311,16 @@ std::array<Tensor, 3> backwardAll(const Tensor &dnew_updates_in,
     return {dupdates, dmu, dnu};
 }
 
-std::array<Tensor, 4> fusedStep(const Tensor &params, const Tensor &updates, const Tensor &mu,
+std::array<Tensor, 4> fusedStep(const Tensor &params, const Tensor &updates_in, const Tensor &mu,
                                 const Tensor &nu, double b1, double b2, double eps,
                                 double eps_root, size_t count, double lr, bool maximize,
                                 bool write_updates, double weight_decay, bool decoupled) {
     const char *name = "adamFusedStep";
     size_t n;
-    const int code = gate(name, updates, {&mu, &nu, &params}, &n);
+    const int code = gate(name, params, {&mu, &nu, &updates_in}, &n);
+    // a gradient that is only read may come in any layout
+    const Tensor updates = (n && !write_updates && params.is_non_overlapping_and_dense())
+                               ? asLayoutOf(updates_in, params) : updates_in;
     if (n) {
         requireDense(name, "params", params);
         requireDense(name, "updates", updates);
@@ -325,14 +328,14 @@ std::array<Tensor, 4> fusedStep(const Tensor &params, const Tensor &updates, con
         requireDense(name, "nu", nu);
         TORCH_CHECK(sameLayout(params, updates) && sameLayout(params, mu) && sameLayout(params, nu),
                     name, ": params, updates, mu and nu must share one memory layout");
-        const OnDeviceOf dev(updates);
+        const OnDeviceOf dev(params);
         check(toa_adam_fused_step(code, params.data_ptr(), updates.data_ptr(), mu.data_ptr(),
                                   nu.data_ptr(), n, b1, b2, eps, eps_root, count, lr,
                                   weight_decay, (int)decoupled, (int)maximize,
                                   (int)write_updates, dev.stream()),
               name);
     }
-    return {params, updates, mu, nu};
+    return {params, updates_in, mu, nu};
 }
 
 // ---- lists of tensors ----------------------------------------------------------------------
@@ -634,14 +637,16 @@ py::tuple fusedStepMulti(const py::object &params_o, const py::object &updates_o
                          bool decoupled) {
     const char *name = "adamFusedStepMulti";
     const auto params = params_o.cast<TensorList>();
-    const auto updates = updates_o.cast<TensorList>();
+    auto updates = updates_o.cast<TensorList>();
     const auto mu = mu_o.cast<TensorList>();
     const auto nu = nu_o.cast<TensorList>();
-    Lists l = gateLists(name, {&updates, &mu, &nu, &params});
+    // gradients that are only read may come in any layout (channels-last, expanded, sliced)
+    if (!write_updates) updates = asLayoutOfEach(updates, params, name);
+    Lists l = gateLists(name, {&params, &mu, &nu, &updates});
     if (l.num) {
         const Counts c = parseCounts(counts, l.num);
-        const OnDeviceOf dev(deviceDonor(updates));
-        check(toa_adam_fused_step_multi(l.code, l.num, l.ptr[3].data(), l.ptr[0].data(),
+        const OnDeviceOf dev(deviceDonor(params));
+        check(toa_adam_fused_step_multi(l.code, l.num, l.ptr[0].data(), l.ptr[3].data(),
                                         l.ptr[1].data(), l.ptr[2].data(), l.n.data(), b1, b2, eps,
                                         eps_root, c.data(), c.all, lr, weight_decay,
                                         (int)decoupled, (int)maximize, (int)write_updates,
