@@ -217,3 +217,28 @@ def test_fused_adam_reads_gradients_in_any_layout():
     with pytest.raises(RuntimeError):  # a gradient that must be overwritten has to be dense
         adam_op.fused_step_(p1, torch.tensor(0.25, device='cuda').expand(4, 3, 5, 5), m, v, B1,
                             B2, EPS, 0.0, 2, 0.01, write_updates=True)
+
+
+def test_fused_adam_with_a_learning_rate_schedule():
+    """The schedule sees the number of steps already taken (0 on the first step); checked step
+    by step against the oracle with the same host-computed rate, and loosely against
+    `torch.optim.Adam` under a `LambdaLR`."""
+    schedule = lambda count: 0.05 / (1.0 + 0.5 * count)  # noqa: E731
+    rng = np.random.default_rng(21)
+    p0 = rng.standard_normal(3001).astype(np.float32)
+    p = dev(p0).requires_grad_(True)
+    q = dev(p0).requires_grad_(True)
+    opt = FusedAdam([p], lr=schedule)
+    ref = torch.optim.Adam([q], lr=1.0)
+    sched = torch.optim.lr_scheduler.LambdaLR(ref, schedule)
+    hp, hm, hv = p0.copy(), np.zeros_like(p0), np.zeros_like(p0)
+    for step in range(4):
+        g = rng.standard_normal(3001).astype(np.float32)
+        p.grad, q.grad = dev(g), dev(g)
+        opt.step()
+        ref.step()
+        sched.step()
+        O.fused_step(hp, g.copy(), hm, hv, B1, B2, EPS, 0.0, step + 1, schedule(step),
+                     write_updates=False)
+        assert_bit_equal(host(p), hp, f'step {step}')
+    np.testing.assert_allclose(host(p), host(q), rtol=2e-5, atol=1e-6)

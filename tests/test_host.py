@@ -180,7 +180,7 @@ def test_fused_adam_argument_validation():
 
     p = [torch.ones(3)]
     for kwargs in (dict(lr=-1.0), dict(eps=-1.0), dict(betas=(1.0, 0.9)), dict(betas=(0.9, 1.0)),
-                   dict(weight_decay=-0.01), dict(lr=lambda c: 0.1)):
+                   dict(weight_decay=-0.01)):
         with pytest.raises(ValueError):
             FusedAdam(p, **kwargs)
     with pytest.raises(TypeError):

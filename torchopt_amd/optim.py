@@ -3,7 +3,7 @@ optimizers with their whole step -- sign flip, weight decay, Adam scaling, multi
 and the addition to the parameters -- in one pass over memory.
 
 Counterparts of /root/reference/torchopt/optim/adam.py:43-92 and optim/adamw.py on top of
-/root/reference/torchopt/optim/base.py:30-135 for a constant learning rate.  What `step()` leaves in the parameters and in the moments is
+/root/reference/torchopt/optim/base.py:30-135.  What `step()` leaves in the parameters and in the moments is
 bit-identical to the reference chain (`flip_sign_and_add_weight_decay` ->
 `scale_by_accelerated_adam` [-> `add_decayed_weights`] -> `scale(-lr)` -> `apply_updates`, all in
 place); the differences are mechanical:
@@ -11,7 +11,12 @@ place); the differences are mechanical:
   * one multi-tensor launch per hundred-odd parameters instead of three passes per parameter
     (28 instead of 44 bytes of HBM traffic per float32 element);
   * `p.grad` is left untouched (the reference's in-place chain overwrites it with the update);
-  * the step count lives on the host next to the 0-dim device tensors the state carries.
+  * the step count lives on the host next to the 0-dim device tensors the state carries;
+  * a learning-rate schedule (a callable of the step count) is evaluated on the host with the
+    integer number of steps already taken, as `scale_by_schedule` feeds it the count before the
+    increment (/root/reference/torchopt/transform/scale_by_schedule.py:93-123); the reference
+    hands the schedule a 0-dim device tensor, so a schedule that computes in tensor arithmetic
+    there may round the rate differently in the last place.
 
 State per parameter group is a `ScaleByAdamState(mu, nu, count)` of tuples, as the
 transformation's own state, so it can be handed to `scale_by_accelerated_adam(...).update`.
@@ -39,7 +44,7 @@ class FusedAdam:
     def __init__(
         self,
         params: Iterable[torch.Tensor],
-        lr: float = 1e-3,
+        lr: float | Callable[[int], float] = 1e-3,
         betas: tuple[float, float] = (0.9, 0.999),
         eps: float = 1e-8,
         weight_decay: float = 0.0,
@@ -51,9 +56,7 @@ class FusedAdam:
         # `use_accelerated_op` is accepted so that the reference's constructor calls carry over
         # (optim/adam.py:56-65); the fused operator is the only path here either way
         del use_accelerated_op
-        if callable(lr):
-            raise ValueError('FusedAdam takes a constant learning rate; schedules are not fused')
-        if not lr >= 0.0:
+        if not callable(lr) and not lr >= 0.0:
             raise ValueError(f'Invalid learning rate: {lr}')
         if not eps >= 0.0:
             raise ValueError(f'Invalid epsilon value: {eps}')
@@ -114,17 +117,21 @@ class FusedAdam:
                 state = self._init_state(group)
             grads = [p.grad for p in group]
             new_counts, values = _inc_counts(state.count, grads)
+            scheduled = callable(self.lr)
             buckets: dict[tuple, list[int]] = {}
             for k, (p, g) in enumerate(zip(group, grads)):
                 if g is not None:
-                    buckets.setdefault((p.device, p.dtype), []).append(k)
+                    # a schedule makes the rate depend on the leaf's own step count
+                    key = (p.device, p.dtype, values[k] if scheduled else None)
+                    buckets.setdefault(key, []).append(k)
             for ks in buckets.values():
                 vals = [values[k] for k in ks]
                 counts = vals[0] if len(set(vals)) == 1 else vals
+                lr = float(self.lr(vals[0] - 1)) if scheduled else self.lr
                 adam_op.fused_step_multi_(
                     [group[k].data for k in ks], [grads[k] for k in ks],
                     [state.mu[k] for k in ks], [state.nu[k] for k in ks],
-                    self.b1, self.b2, self.eps, self.eps_root, counts, self.lr,
+                    self.b1, self.b2, self.eps, self.eps_root, counts, lr,
                     maximize=self.maximize, write_updates=False,
                     weight_decay=self.weight_decay, decoupled=self._decoupled)
             self.state_groups[i] = state._replace(count=tuple(new_counts))
