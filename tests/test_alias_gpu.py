@@ -192,3 +192,31 @@ def test_meta_adamw_and_unused_parameters():
     opt.step(net(x).pow(2).mean())
     st = opt.state_dict()[0][1]
     assert [int(c) for c in st.count] == [2, 2, 0, 0]
+
+
+def test_func_optimizer_inner_loop_matches_plain_autograd():
+    """`FuncOptimizer(adam(...)).step(loss, params)` on a dict of parameters: two differentiable
+    steps, outer gradient against the hand-written inner loop (eps = eps_root = 0, where the
+    op's backward is the exact derivative)."""
+    torch.manual_seed(9)
+    dt = torch.float64
+    w0 = torch.randn(4, 6, device='cuda', dtype=dt, requires_grad=True)
+    b0 = torch.randn(4, device='cuda', dtype=dt, requires_grad=True)
+    x = torch.randn(20, 6, device='cuda', dtype=dt)
+    y = torch.randn(20, 4, device='cuda', dtype=dt)
+    lr, b1, b2 = 0.05, 0.9, 0.999
+    opt = topt.FuncOptimizer(topt.adam(lr, (b1, b2), 0.0))
+    params = {'w': w0, 'b': b0, 'frozen': None}
+    for _ in range(2):
+        loss = ((x @ params['w'].t() + params['b'] - y) ** 2).mean()
+        params = opt.step(loss, params)
+    assert set(params) == {'w', 'b', 'frozen'} and params['frozen'] is None
+    outer = (params['w'] ** 2).sum() + (params['b'] ** 2).sum()
+    got = torch.autograd.grad(outer, (w0, b0))
+    w, b = inner_loop_plain(w0, b0, x, y, 2, lr, b1, b2, 0.0, 0.0)
+    want = torch.autograd.grad((w ** 2).sum() + (b ** 2).sum(), (w0, b0))
+    torch.testing.assert_close(params['w'], w, rtol=1e-9, atol=1e-12)
+    for g, r in zip(got, want):
+        torch.testing.assert_close(g, r, rtol=1e-8, atol=1e-11)
+    with pytest.raises(TypeError):
+        topt.FuncOptimizer(object())

@@ -11,6 +11,7 @@ from torchopt_amd import accelerated_op
 from torchopt_amd.accelerated_op import AdamOp, MultiAdamOp
 from torchopt_amd.accelerated_op import is_available as accelerated_op_available
 from torchopt_amd.alias import adam, adamw, apply_updates, chain
+from torchopt_amd.func import FuncOptimizer
 from torchopt_amd.meta import MetaAdam, MetaAdamW
 from torchopt_amd.optim import Adam, AdamW, FusedAdam, FusedAdamW
 
@@ -21,5 +22,5 @@ _sys.modules.setdefault('torchopt_amd._C.adam_op', _C.adam_op)
 
 __version__ = '0.1.0'
 
-__all__ = ['Adam', 'AdamOp', 'AdamW', 'FusedAdam', 'FusedAdamW', 'MetaAdam', 'MetaAdamW', 'MultiAdamOp', 'accelerated_op',
+__all__ = ['Adam', 'AdamOp', 'AdamW', 'FuncOptimizer', 'FusedAdam', 'FusedAdamW', 'MetaAdam', 'MetaAdamW', 'MultiAdamOp', 'accelerated_op',
            'accelerated_op_available', 'adam', 'adamw', 'apply_updates', 'chain']
