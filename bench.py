@@ -117,6 +117,38 @@ def make_state(torch, n, dtype, seed):
     return u, mu, nu
 
 
+def python_level_differentiable_step(torch, shapes, eps_root, count, wall_ms):
+    """What a meta-learning loop pays per inner step, from Python through autograd: the Adam
+    transformation's differentiable `update` over the tree plus the backward through it, next to
+    the same mathematics written as per-leaf PyTorch tensor expressions (the route a build
+    without the fused operator takes)."""
+    from torchopt_amd.transform import scale_by_accelerated_adam
+
+    grads = tuple(torch.randn(s, device='cuda', requires_grad=True) for s in shapes)
+    transform = scale_by_accelerated_adam(B1, B2, EPS, eps_root, moment_requires_grad=True)
+    state = transform.init(grads)
+    c1, c2 = 1 / (1 - B1 ** count), 1 / (1 - B2 ** count)
+
+    def fused():
+        updates, _ = transform.update(grads, state, inplace=False)
+        torch.autograd.grad(sum((u * u).sum() for u in updates), grads)
+
+    def per_leaf_expressions():
+        updates = []
+        for g, m, v in zip(grads, state.mu, state.nu):
+            m1 = m * B1 + g * (1 - B1)
+            v1 = v * B2 + g * g * (1 - B2)
+            updates.append((m1 * c1) / (torch.sqrt(v1 * c2 + eps_root) + EPS))
+        torch.autograd.grad(sum((u * u).sum() for u in updates), grads)
+
+    def loss_alone():  # the part of both that is not Adam
+        torch.autograd.grad(sum((g * g).sum() for g in grads), grads)
+
+    base = wall_ms(loss_alone)
+    return {'python_update_plus_backward_ms': round(wall_ms(fused) - base, 5),
+            'python_per_leaf_tensor_expressions_ms': round(wall_ms(per_leaf_expressions) - base, 5)}
+
+
 def run_gpu(cfg_id, steps, warmup):
     import torch
 
@@ -209,7 +241,9 @@ def run_gpu(cfg_id, steps, warmup):
         extra = {'tensors': num, 'launches_per_step': 2,
                  'six_list_launches_ms_per_step': round(six_ms, 5),
                  'per_leaf_loop_ms_per_step': round(per_leaf_ms, 5),
-                 'per_leaf_loop_launches_per_step': 6 * num}
+                 'per_leaf_loop_launches_per_step': 6 * num,
+                 **python_level_differentiable_step(torch, cfg['shapes'], eps_root, count,
+                                                    wall_ms)}
     elif 'shapes' in cfg:
         import ctypes
 
