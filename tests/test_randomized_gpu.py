@@ -53,7 +53,7 @@ def test_random_cases(seed):
         eps = float(10.0 ** rng.uniform(-8, -2)) if tag in ('f32', 'f64') else float(
             10.0 ** rng.uniform(-4, -2))
         er = float(rng.choice([0.0, 10.0 ** rng.uniform(-6, -3)]))
-        count = int(rng.choice([1, 2, 17, 1000, 10 ** 6]))
+        count = int(rng.choice([0, 1, 2, 17, 1000, 10 ** 6, 2 ** 40]))
         scale = float(10.0 ** rng.uniform(-3, 2))
         raw = {k: to_fmt(scale * rng.standard_normal(n + off + 3), tag)
                for k in ('updates', 'mu', 'dmu', 'dnu', 'dupdates')}
