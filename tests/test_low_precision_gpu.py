@@ -99,6 +99,19 @@ def test_sizes_against_oracle(tag):
 
 
 @pytest.mark.parametrize('tag', ['f16', 'bf16'])
+@pytest.mark.parametrize('operand', ['updates', 'mu', 'nu', 'dmu', 'dnu', 'dupdates'])
+def test_every_bit_pattern_of_one_operand(tag, operand):
+    """All 65 536 values of the type (every denormal, infinity and NaN included) in one operand,
+    the others drawn at random: every conversion and rounding case of that operand's paths."""
+    n = 1 << 16
+    inp = draw(tag, n, 900 + len(operand))
+    every = np.arange(n, dtype=np.uint16)
+    inp[operand] = every if tag == 'bf16' else every.view(np.float16)
+    with np.errstate(all='ignore'):
+        check_all_seven(tag, inp, (0.9, 0.999, 1e-3, 1e-4, 3), f'{tag}/all {operand}')
+
+
+@pytest.mark.parametrize('tag', ['f16', 'bf16'])
 def test_misaligned_views(tag):
     n = 30_001
     inp = draw(tag, n + 8, 5)
