@@ -93,8 +93,9 @@ CONFIGS = {
     2: dict(name='config2: fused forward_ in place, 268 435 456 float32 elements '
                  '(1 GiB per state array), count=1000',
             dtype='f32', n=1 << 28, eps_root=0.0, count=1000),
-    3: dict(name='config3: fused forward_ in place, 67 108 864 float64 elements, count=3',
-            dtype='f64', n=1 << 26, eps_root=1e-8, count=3),
+    3: dict(name='config3: fused forward_ in place, 67 108 864 float64 elements, count=3; beside '
+                 'it the backward ops on the same shapes',
+            dtype='f64', n=1 << 26, eps_root=1e-8, count=3, backward=True),
     4: dict(name='config4: multi-tensor forward_ in place over the GPT-2-medium parameter list '
                  '(float32), count=1',
             dtype='f32', shapes=gpt2_medium_shapes(), eps_root=0.0, count=1),
@@ -147,6 +148,43 @@ def python_level_differentiable_step(torch, shapes, eps_root, count, wall_ms):
     base = wall_ms(loss_alone)
     return {'python_update_plus_backward_ms': round(wall_ms(fused) - base, 5),
             'python_per_leaf_tensor_expressions_ms': round(wall_ms(per_leaf_expressions) - base, 5)}
+
+
+def time_backward_ops(torch, lib, code, dtype, n, esize, eps_root, count, stream, reps=20):
+    """backward_mu, backward_nu, backward_updates and the one-pass backward_all on flat arrays of
+    n elements: ms per launch and achieved GB/s (algorithmic bytes: 3, 4, 5 and 9 arrays)."""
+    g = torch.Generator(device='cuda')
+    g.manual_seed(77)
+    arrays = [torch.randn(n, device='cuda', dtype=dtype, generator=g) for _ in range(9)]
+    arrays[2].mul_(0.1)
+    p = [a.data_ptr() for a in arrays]
+    s = stream.cuda_stream
+    # slots: 0 updates / dupdates, 1 new_updates, 2 new_mu, 3 dmu, 4 dnu, 5..8 outputs
+    ops = {
+        'backward_mu': (3, lambda: lib.toa_adam_backward_mu(code, p[3], n, B1, p[5], p[6], s)),
+        'backward_nu': (4, lambda: lib.toa_adam_backward_nu(code, p[4], p[0], n, B2, p[5], p[6],
+                                                            s)),
+        'backward_updates': (5, lambda: lib.toa_adam_backward_updates(
+            code, p[0], p[1], p[2], n, B1, B2, eps_root, count, p[5], p[6], s)),
+        'backward_all': (9, lambda: lib.toa_adam_backward_all(
+            code, p[0], p[1], p[2], p[8], p[3], p[4], n, B1, B2, eps_root, count, p[5], p[6],
+            p[7], s)),
+    }
+    out = {}
+    for name, (streams, fn) in ops.items():
+        for _ in range(5):
+            rc = fn()
+            if rc:
+                raise RuntimeError(f'{name}: {lib.toa_adam_error_string(rc).decode()}')
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(reps):
+            fn()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        out[name] = {'ms': round(ms, 5), 'GB/s': round(streams * esize * n / ms / 1e6, 1)}
+    return out
 
 
 def run_gpu(cfg_id, steps, warmup):
@@ -315,6 +353,9 @@ def run_gpu(cfg_id, steps, warmup):
             if rc:
                 raise RuntimeError(lib.toa_adam_error_string(rc).decode())
         extra = {}
+        if cfg.get('backward'):
+            extra['backward_ops'] = time_backward_ops(torch, lib, code, dtype, total, esize,
+                                                      eps_root, count, stream)
         if alg_small(total * esize):
             # The timed loop below re-runs on state that stays in the 256 MB Infinity Cache; a
             # real optimizer step finds its state in HBM.  Time single launches after sweeping
