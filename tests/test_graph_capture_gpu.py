@@ -102,3 +102,46 @@ def test_split_ops_and_fused_step_under_graph_replay():
         assert_bit_equal(host(p), hp, f'replay {replay} params')
         assert_bit_equal(host(m), hm, f'replay {replay} mu')
         assert_bit_equal(host(g), f, f'replay {replay} gradient left alone')
+
+
+def test_concurrent_callers_on_their_own_streams():
+    """The library keeps no per-call state: threads launching on separate streams at the same
+    time (as autograd's worker threads do for the backward ops) get independent, correct
+    results."""
+    import threading
+
+    rng = np.random.default_rng(3)
+    n, rounds = 200_003, 25
+    jobs = []
+    for k in range(4):
+        g = rng.standard_normal(n).astype(np.float32)
+        m = (0.1 * rng.standard_normal(n)).astype(np.float32)
+        v = np.abs(0.01 * rng.standard_normal(n)).astype(np.float32)
+        jobs.append({'host': (g, m, v), 'count': k + 1, 'out': None, 'err': None})
+
+    def worker(job):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                dev = [torch.from_numpy(a).cuda() for a in job['host']]
+                for _ in range(rounds):  # out-of-place ops: same inputs, same outputs, every time
+                    mu1 = adam_op.forward_mu(dev[0], dev[1], 0.9)
+                    nu1 = adam_op.forward_nu(dev[0], dev[2], 0.999)
+                    up = adam_op.forward_updates(mu1, nu1, 0.9, 0.999, 1e-8, 0.0, job['count'])
+                stream.synchronize()
+                job['out'] = (mu1.cpu().numpy(), nu1.cpu().numpy(), up.cpu().numpy())
+        except Exception as exc:  # noqa: BLE001
+            job['err'] = exc
+
+    threads = [threading.Thread(target=worker, args=(j,)) for j in jobs]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for k, job in enumerate(jobs):
+        assert job['err'] is None, job['err']
+        g, m, v = job['host']
+        e_mu, e_nu = O.forward_mu(g, m, 0.9), O.forward_nu(g, v, 0.999)
+        e_up = O.forward_updates(e_mu, e_nu, 0.9, 0.999, 1e-8, 0.0, job['count'])
+        for got, want, what in zip(job['out'], (e_mu, e_nu, e_up), ('mu', 'nu', 'updates')):
+            assert_bit_equal(got, want, f'thread {k} {what}')
