@@ -26,7 +26,9 @@
 // rounding: every product and sum is rounded on its own (build with
 // -ffp-contract=off), (1-b) is formed in the element type, bias corrections
 // are pre-rounded reciprocals that multiply, sqrt and divide are the
-// correctly rounded ones, and the tail of backward_updates runs in double.
+// correctly rounded ones (bfloat16 reaches the same bits through a checked
+// shortcut, see adam_direction_quick), and the tail of backward_updates runs in
+// double.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -187,6 +189,63 @@ __device__ __forceinline__ double toa_sqrt(double x) { return sqrt(x); }
 template <class F>
 __device__ __forceinline__ float toa_sqrt(R16<F> x) { return sqrtf((float)x); }
 
+// The step direction mu_hat / (sqrt(nu_hat + eps_root) + eps) as the reference writes it
+// (adam_op_impl_cpu.cpp:58-60, 177-179).
+template <typename T>
+__device__ __forceinline__ T adam_direction(T mh, T vh, T eps_root, T eps) {
+    return mh / (toa_sqrt(vh + eps_root) + eps);
+}
+
+// bfloat16: the root, the sum with eps and the quotient run in float and only the quotient is
+// rounded to 8 significant bits, so the correctly rounded float root and quotient (ten and
+// twelve instructions each) are needed only when the quotient lands next to a rounding boundary
+// of the 16-bit result.  The quick route takes the hardware's 1-ulp root and reciprocal:
+//     s' = sqrt~(x), d' = s' + eps, q' = mu_hat * rcp~(d')
+// q' is within 9 float ulps of the exact chain's quotient (1 + 0.5 ulp from the root carried
+// through the sum, one rounding of each sum, 1 ulp of the reciprocal, the rounding of each
+// product and quotient: 4.5 * 2^-23 relative).  If q' is further than 16 float ulps from the
+// midpoint between two bfloat16 values, both round to the same bfloat16 and `ok` is set.
+// Otherwise -- about one element in two thousand -- or when an operand is outside the range
+// where the 1-ulp claims hold (denormal, zero divisor, infinity, NaN, negative), the caller
+// runs the exact chain for that element.  Checked against the exact chain for every
+// (mu_hat, nu_hat + eps_root) pair of bit patterns.
+template <typename T>
+struct HasQuickDirection {
+    static constexpr bool value = false;
+};
+template <>
+struct HasQuickDirection<bfloat_t> {
+    static constexpr bool value = true;
+};
+
+__device__ __forceinline__ bfloat_t adam_direction_quick(bfloat_t mh, bfloat_t vh,
+                                                         bfloat_t eps_root, bfloat_t eps,
+                                                         bool &ok) {
+    const bfloat_t x16 = vh + eps_root;
+    const float x = (float)x16, m = (float)mh, e = (float)eps;
+    const float d = __builtin_amdgcn_sqrtf(x) + e;
+    const float q = m * __builtin_amdgcn_rcpf(d);
+    const uint32_t low = __builtin_bit_cast(uint32_t, q) & 0xffffu;
+    const float aq = __builtin_fabsf(q);
+    ok = (x == 0.0f || x >= 1.17549435e-38f) &&          // normal or zero radicand
+         d >= 5.42101086e-20f && d <= 1.84467441e19f &&  // 2^-64 .. 2^64
+         ((aq >= 7.88860905e-31f && aq <= 1.26765060e30f) || m == 0.0f) &&  // 2^-100 .. 2^100
+         (low - 0x7ff0u > 0x20u);  // not within 16 ulps of the midpoint 0x8000
+    return bfloat_t(q);
+}
+
+// An op is speculative when it offers `quick(in, out) -> bool` beside the exact operator():
+// the whole-tile path runs quick() on every element and repeats only the elements that
+// returned false with the exact operator.
+template <class Op, class = void>
+struct IsSpeculative {
+    static constexpr bool value = false;
+};
+template <class Op>
+struct IsSpeculative<Op, decltype((void)Op::kSpeculative)> {
+    static constexpr bool value = Op::kSpeculative;
+};
+
 // Residency level by element type: 4- and 8-byte types behave alike; the 16-bit types spend
 // twice the ALU time per byte on re-rounding and want more waves, bfloat16 (no native
 // arithmetic) the most.
@@ -210,8 +269,10 @@ struct ForwardInplace {
     static constexpr int kWavesPerCUMulti = waves_by_type<T>(16, 21, 32);
     // outputs are produced as (mu', nu', updates') and stored in that order
     __device__ static constexpr int out_slot(int j) { return j == 0 ? 1 : (j == 1 ? 2 : 0); }
+    static constexpr bool kSpeculative = HasQuickDirection<T>::value;
     T b1, b2, c1, c2, eps, eps_root;
-    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
+    template <bool QUICK>
+    __device__ __forceinline__ bool run(const T (&in)[NIN], T (&out)[NOUT]) const {
         const T g = in[0], m = in[1], v = in[2];
         const T m1 = b1 * m + (1 - b1) * g;
         const T v1 = b2 * v + (1 - b2) * g * g;
@@ -219,7 +280,18 @@ struct ForwardInplace {
         const T vh = v1 * c2;
         out[0] = m1;
         out[1] = v1;
-        out[2] = mh / (toa_sqrt(vh + eps_root) + eps);
+        bool ok = true;
+        if constexpr (QUICK)
+            out[2] = adam_direction_quick(mh, vh, eps_root, eps, ok);
+        else
+            out[2] = adam_direction(mh, vh, eps_root, eps);
+        return ok;
+    }
+    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
+        run<false>(in, out);
+    }
+    __device__ __forceinline__ bool quick(const T (&in)[NIN], T (&out)[NOUT]) const {
+        return run<true>(in, out);
     }
 };
 
@@ -257,11 +329,24 @@ struct ForwardUpdates {
     static constexpr int kWavesPerCU = 32;  // sqrt and divide: needs the waves to hide ALU time
     static constexpr int kWavesPerCUMulti = 32;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
+    static constexpr bool kSpeculative = HasQuickDirection<T>::value;
     T c1, c2, eps, eps_root;
-    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
+    template <bool QUICK>
+    __device__ __forceinline__ bool run(const T (&in)[NIN], T (&out)[NOUT]) const {
         const T mh = in[0] * c1;
         const T vh = in[1] * c2;
-        out[0] = mh / (toa_sqrt(vh + eps_root) + eps);
+        bool ok = true;
+        if constexpr (QUICK)
+            out[0] = adam_direction_quick(mh, vh, eps_root, eps, ok);
+        else
+            out[0] = adam_direction(mh, vh, eps_root, eps);
+        return ok;
+    }
+    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
+        run<false>(in, out);
+    }
+    __device__ __forceinline__ bool quick(const T (&in)[NIN], T (&out)[NOUT]) const {
+        return run<true>(in, out);
     }
 };
 
@@ -322,11 +407,13 @@ struct BackwardUpdates {
 template <typename T>
 struct ForwardAll {
     static constexpr int NIN = 3, NOUT = 3, NPTR = 6;
-    static constexpr int kWavesPerCU = waves_by_type<T>(14, 18, 18);  // six streams per wave: few waves fill the queues
-    static constexpr int kWavesPerCUMulti = waves_by_type<T>(18, 21, 21);
+    static constexpr int kWavesPerCU = waves_by_type<T>(14, 18, 25);  // six streams per wave: few waves fill the queues
+    static constexpr int kWavesPerCUMulti = waves_by_type<T>(18, 21, 32);
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
+    static constexpr bool kSpeculative = HasQuickDirection<T>::value;
     T b1, b2, c1, c2, eps, eps_root;
-    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
+    template <bool QUICK>
+    __device__ __forceinline__ bool run(const T (&in)[NIN], T (&out)[NOUT]) const {
         const T g = in[0], m = in[1], v = in[2];
         const T m1 = b1 * m + (1 - b1) * g;
         const T v1 = b2 * v + (1 - b2) * g * g;
@@ -334,7 +421,18 @@ struct ForwardAll {
         const T vh = v1 * c2;
         out[0] = m1;
         out[1] = v1;
-        out[2] = mh / (toa_sqrt(vh + eps_root) + eps);
+        bool ok = true;
+        if constexpr (QUICK)
+            out[2] = adam_direction_quick(mh, vh, eps_root, eps, ok);
+        else
+            out[2] = adam_direction(mh, vh, eps_root, eps);
+        return ok;
+    }
+    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
+        run<false>(in, out);
+    }
+    __device__ __forceinline__ bool quick(const T (&in)[NIN], T (&out)[NOUT]) const {
+        return run<true>(in, out);
     }
 };
 
@@ -409,7 +507,7 @@ struct FusedStep {
         const T v1 = b2 * v + (1 - b2) * g * g;
         const T mh = m1 * c1;
         const T vh = v1 * c2;
-        T u1 = mh / (toa_sqrt(vh + eps_root) + eps);
+        T u1 = adam_direction(mh, vh, eps_root, eps);
         if (decay == kDecayIntoUpdate) u1 = toa_fma(wd, p, u1);
         const T step = u1 * neg_lr;
         out[0] = m1;
@@ -451,6 +549,8 @@ __device__ __forceinline__ void tile_full(const Op &op, const TensorPtrs<T, Op> 
             in[i][k] = ld<NT>(reinterpret_cast<const V *>(tp.p[i]) + v0 + (size_t)k * kBlock);
 
     V out[Op::NOUT][UNROLL];
+    static_assert(UNROLL * VN <= 32, "one redo bit per element of a lane");
+    [[maybe_unused]] uint32_t redo = 0;
 #pragma unroll
     for (int k = 0; k < UNROLL; ++k)
 #pragma unroll
@@ -458,10 +558,31 @@ __device__ __forceinline__ void tile_full(const Op &op, const TensorPtrs<T, Op> 
             T a[Op::NIN], r[Op::NOUT];
 #pragma unroll
             for (int i = 0; i < Op::NIN; ++i) a[i] = Vec<T>::get(in[i][k], e);
-            op(a, r);
+            if constexpr (IsSpeculative<Op>::value) {
+                if (!op.quick(a, r)) redo |= 1u << (k * VN + e);
+            } else {
+                op(a, r);
+            }
 #pragma unroll
             for (int j = 0; j < Op::NOUT; ++j) Vec<T>::set(out[j][k], e, r[j]);
         }
+
+    if constexpr (IsSpeculative<Op>::value) {
+        if (redo != 0) {  // rare: some lane has an element the quick route could not settle
+#pragma unroll
+            for (int k = 0; k < UNROLL; ++k)
+#pragma unroll
+                for (int e = 0; e < VN; ++e)
+                    if (redo & (1u << (k * VN + e))) {
+                        T a[Op::NIN], r[Op::NOUT];
+#pragma unroll
+                        for (int i = 0; i < Op::NIN; ++i) a[i] = Vec<T>::get(in[i][k], e);
+                        op(a, r);
+#pragma unroll
+                        for (int j = 0; j < Op::NOUT; ++j) Vec<T>::set(out[j][k], e, r[j]);
+                    }
+        }
+    }
 
 #pragma unroll
     for (int k = 0; k < UNROLL; ++k)
