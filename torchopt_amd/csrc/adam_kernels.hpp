@@ -26,7 +26,7 @@
 // rounding: every product and sum is rounded on its own (build with
 // -ffp-contract=off), (1-b) is formed in the element type, bias corrections
 // are pre-rounded reciprocals that multiply, sqrt and divide are the
-// correctly rounded ones (bfloat16 reaches the same bits through a checked
+// correctly rounded ones (the 16-bit types reach the same bits through a checked
 // shortcut, see adam_direction_quick), and the tail of backward_updates runs in
 // double.
 #pragma once
@@ -217,6 +217,10 @@ template <>
 struct HasQuickDirection<bfloat_t> {
     static constexpr bool value = true;
 };
+template <>
+struct HasQuickDirection<half_t> {
+    static constexpr bool value = true;
+};
 
 __device__ __forceinline__ bfloat_t adam_direction_quick(bfloat_t mh, bfloat_t vh,
                                                          bfloat_t eps_root, bfloat_t eps,
@@ -232,6 +236,22 @@ __device__ __forceinline__ bfloat_t adam_direction_quick(bfloat_t mh, bfloat_t v
          ((aq >= 7.88860905e-31f && aq <= 1.26765060e30f) || m == 0.0f) &&  // 2^-100 .. 2^100
          (low - 0x7ff0u > 0x20u);  // not within 16 ulps of the midpoint 0x8000
     return bfloat_t(q);
+}
+
+// float16 likewise: 11 significant bits, so the midpoints lie 0x2000 float ulps apart (the
+// quick route settles fewer elements), and the result must be a normal float16.
+__device__ __forceinline__ half_t adam_direction_quick(half_t mh, half_t vh, half_t eps_root,
+                                                       half_t eps, bool &ok) {
+    const half_t x16 = vh + eps_root;
+    const float x = (float)x16, m = (float)mh, e = (float)eps;
+    const float d = __builtin_amdgcn_sqrtf(x) + e;
+    const float q = m * __builtin_amdgcn_rcpf(d);
+    const uint32_t low = __builtin_bit_cast(uint32_t, q) & 0x1fffu;
+    const float aq = __builtin_fabsf(q);
+    ok = x >= 0.0f && d >= 5.42101086e-20f && d <= 1.84467441e19f &&
+         ((aq >= 6.10351562e-05f && aq <= 32768.0f) || m == 0.0f) &&  // 2^-14 .. 2^15
+         (low - 0x0ff0u > 0x20u);  // not within 16 ulps of the midpoint 0x1000
+    return half_t(q);
 }
 
 // An op is speculative when it offers `quick(in, out) -> bool` beside the exact operator():
