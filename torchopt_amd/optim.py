@@ -11,7 +11,8 @@ place); the differences are mechanical:
   * one multi-tensor launch per hundred-odd parameters instead of three passes per parameter
     (28 instead of 44 bytes of HBM traffic per float32 element);
   * `p.grad` is left untouched (the reference's in-place chain overwrites it with the update);
-  * the step count lives on the host next to the 0-dim device tensors the state carries;
+  * the step count lives on the host; the 0-dim device tensors the state carries are brought up
+    to date when the state is asked for (`state_dict()`);
   * a learning-rate schedule (a callable of the step count) is evaluated on the host with the
     integer number of steps already taken, as `scale_by_schedule` feeds it the count before the
     increment (/root/reference/torchopt/transform/scale_by_schedule.py:93-123); the reference
@@ -29,7 +30,8 @@ from typing import Callable, Iterable, Sequence
 import torch
 
 from torchopt_amd.accelerated_op.adam_op import adam_op
-from torchopt_amd.transform.scale_by_adam import ScaleByAdamState, _inc_counts, _remember
+from torchopt_amd.transform.scale_by_adam import (INT64_MAX, ScaleByAdamState, _host_value,
+                                                 _remember)
 
 
 __all__ = ['Adam', 'AdamW', 'FusedAdam', 'FusedAdamW']
@@ -71,6 +73,9 @@ class FusedAdam:
         self.eps_root, self.maximize = eps_root, maximize
         self.param_groups: list[tuple[torch.Tensor, ...]] = []
         self.state_groups: list[ScaleByAdamState | None] = []
+        self._kinds: list[list[tuple]] = []       # (device, dtype) per parameter
+        self._steps: list[list[int] | None] = []  # host-side step numbers per parameter
+        self._stale: list[bool] = []              # device count tensors lag the host numbers
         self.add_param_group(params)
 
     def add_param_group(self, params: Iterable[torch.Tensor]) -> None:
@@ -80,6 +85,9 @@ class FusedAdam:
                 raise TypeError(f'expected tensors, got {type(p).__name__}')
         self.param_groups.append(group)
         self.state_groups.append(None)  # built on the first step, like the reference
+        self._kinds.append([(p.device, p.dtype) for p in group])
+        self._steps.append(None)
+        self._stale.append(False)
 
     def zero_grad(self, set_to_none: bool = False) -> None:
         for group in self.param_groups:
@@ -94,47 +102,81 @@ class FusedAdam:
                     p.grad.zero_()
 
     def state_dict(self) -> tuple:
+        """Per group a `ScaleByAdamState` (or None before the first step)."""
+        for i in range(len(self.state_groups)):
+            self._sync_counts(i)
         return tuple(self.state_groups)
 
     def load_state_dict(self, state_dict: Sequence) -> None:
         self.state_groups[:] = list(state_dict)
+        self._steps = [None if s is None else [_host_value(c) for c in s.count]
+                       for s in self.state_groups]
+        self._stale = [False] * len(self.state_groups)
 
-    @staticmethod
-    def _init_state(group: tuple[torch.Tensor, ...]) -> ScaleByAdamState:
+    def _init_state(self, i: int) -> ScaleByAdamState:
+        group = self.param_groups[i]
         count = tuple(_remember(torch.zeros(1, dtype=torch.int64, device=p.device).squeeze_(), 0)
                       for p in group)
+        self._steps[i] = [0] * len(group)
+        self._stale[i] = False
         return ScaleByAdamState(mu=tuple(torch.zeros_like(p) for p in group),
                                 nu=tuple(torch.zeros_like(p) for p in group), count=count)
 
+    def _sync_counts(self, i: int) -> None:
+        """Bring the 0-dim device count tensors of group `i` up to the host's step numbers.
+        `step()` advances only the host numbers; the tensors are rebuilt (one upload per
+        device) when somebody asks for the state."""
+        if not self._stale[i]:
+            return
+        state, steps = self.state_groups[i], self._steps[i]
+        by_device: dict[torch.device, list[int]] = {}
+        for k, c in enumerate(state.count):
+            by_device.setdefault(c.device, []).append(k)
+        counts = list(state.count)
+        for device, ks in by_device.items():
+            fresh = torch.tensor([steps[k] for k in ks], dtype=torch.int64, device=device).unbind(0)
+            for k, t in zip(ks, fresh):
+                counts[k] = _remember(t, steps[k])
+        self.state_groups[i] = state._replace(count=tuple(counts))
+        self._stale[i] = False
+
+    @torch.no_grad()
     def step(self, closure: Callable[[], torch.Tensor] | None = None):
         loss = None
         if closure is not None:
             with torch.enable_grad():
                 loss = closure()
+        scheduled = callable(self.lr)
         for i, group in enumerate(self.param_groups):
-            state = self.state_groups[i]
-            if state is None:
-                state = self._init_state(group)
+            if self.state_groups[i] is None:
+                self.state_groups[i] = self._init_state(i)
+            state, steps = self.state_groups[i], self._steps[i]
             grads = [p.grad for p in group]
-            new_counts, values = _inc_counts(state.count, grads)
-            scheduled = callable(self.lr)
+            live = [k for k, g in enumerate(grads) if g is not None]
+            if not live:
+                continue
+            for k in live:
+                if steps[k] != INT64_MAX:
+                    steps[k] += 1
+            self._stale[i] = True
             buckets: dict[tuple, list[int]] = {}
-            for k, (p, g) in enumerate(zip(group, grads)):
-                if g is not None:
-                    # a schedule makes the rate depend on the leaf's own step count
-                    key = (p.device, p.dtype, values[k] if scheduled else None)
-                    buckets.setdefault(key, []).append(k)
+            for k in live:
+                # a schedule makes the rate depend on the leaf's own step count
+                key = (self._kinds[i][k], steps[k] if scheduled else None)
+                buckets.setdefault(key, []).append(k)
             for ks in buckets.values():
-                vals = [values[k] for k in ks]
-                counts = vals[0] if len(set(vals)) == 1 else vals
+                vals = [steps[k] for k in ks]
+                counts = vals[0] if vals.count(vals[0]) == len(vals) else vals
                 lr = float(self.lr(vals[0] - 1)) if scheduled else self.lr
+                whole = len(ks) == len(group)
                 adam_op.fused_step_multi_(
-                    [group[k].data for k in ks], [grads[k] for k in ks],
-                    [state.mu[k] for k in ks], [state.nu[k] for k in ks],
+                    list(group) if whole else [group[k] for k in ks],
+                    grads if whole else [grads[k] for k in ks],
+                    list(state.mu) if whole else [state.mu[k] for k in ks],
+                    list(state.nu) if whole else [state.nu[k] for k in ks],
                     self.b1, self.b2, self.eps, self.eps_root, counts, lr,
                     maximize=self.maximize, write_updates=False,
                     weight_decay=self.weight_decay, decoupled=self._decoupled)
-            self.state_groups[i] = state._replace(count=tuple(new_counts))
         return loss
 
 
