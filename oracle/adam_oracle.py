@@ -7,7 +7,8 @@ CPU-baseline leg of the benchmark may import this module.  The shipped operator
 `load_reference()` additionally loads, where it has been built, the reference's
 own compiled CPU op (oracle/_ref/_C*.so, built by `make -C oracle ref` from the
 sources under /root/reference) as a Python module exposing `adam_op.forward_`
-and friends on CPU torch tensors.
+and friends on CPU torch tensors.  `load_dropin()` loads the reference's extension
+built with its device branch routed to libtoa_adam.so (oracle/_ref/dropin/).
 """
 
 from __future__ import annotations
@@ -161,14 +162,29 @@ def reference_path():
     return hits[0] if hits else None
 
 
-def load_reference():
-    """Import the compiled reference CPU op, or return None if it was not built."""
-    path = reference_path()
-    if path is None:
-        return None
+def _load_extension(path):
     import torch  # noqa: F401  (libtorch must be loaded first)
 
     spec = importlib.util.spec_from_file_location('_C', path)
     mod = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mod)
     return mod
+
+
+def load_reference():
+    """Import the compiled reference CPU op, or return None if it was not built."""
+    path = reference_path()
+    return None if path is None else _load_extension(path)
+
+
+def dropin_path():
+    hits = sorted(glob.glob(os.path.join(_HERE, '_ref', 'dropin', '_C*.so')))
+    return hits[0] if hits else None
+
+
+def load_dropin():
+    """Import the reference's own extension built with its device branch on libtoa_adam.so
+    (`make -C oracle dropin`), or return None if it was not built.  This is the object under
+    test of the drop-in boundary, not a checker."""
+    path = dropin_path()
+    return None if path is None else _load_extension(path)
