@@ -29,14 +29,19 @@ def ref_ext():
 
 
 def dev(a):
-    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.uint16:  # bfloat16 bit patterns
+        return torch.from_numpy(a.view(np.int16)).cuda().view(torch.bfloat16)
+    return torch.from_numpy(a).cuda()
 
 
 def host(t):
+    if t.dtype == torch.bfloat16:
+        return t.detach().contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
     return t.detach().cpu().numpy()
 
 
-@pytest.mark.parametrize('tag', ['f32', 'f64'])
+@pytest.mark.parametrize('tag', ['f32', 'f64', 'f16', 'bf16'])
 def test_golden_vectors_through_the_reference_dispatcher(ref_ext, tag):
     for name, case in sorted(load_golden(tag).items()):
         b1, b2, eps, er, c = hyper_of(case)
