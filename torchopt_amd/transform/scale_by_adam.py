@@ -40,6 +40,8 @@ __all__ = ['ScaleByAdamState', 'scale_by_accelerated_adam']
 
 INT64_MAX = torch.iinfo(torch.int64).max
 _MIRROR = '_toa_host_value'
+# exact leaf types a flat list may hold to count as already flattened (checked in C, per call)
+_PLAIN_LEAVES = frozenset({torch.Tensor, torch.nn.Parameter, type(None)})
 
 
 class ScaleByAdamState(NamedTuple):
@@ -71,19 +73,42 @@ def _host_value(t: torch.Tensor) -> int:
 
 def _inc_counts(counts: Sequence[torch.Tensor | None], grads: Sequence[Any]):
     """``c + (c != INT64_MAX)`` for leaves with a gradient, the same tensor otherwise.
-    Returns (new count leaves, host values of the new counts)."""
-    values = [None if c is None else _host_value(c) for c in counts]
-    todo = [k for k, (c, g) in enumerate(zip(counts, grads))
-            if c is not None and g is not None and values[k] != INT64_MAX]
-    new = list(counts)
+    Returns (new count leaves, host values of the new counts).
+
+    Leaves that hold the very same count tensor (as the leaves of one `init` do, see there) are
+    advanced together: one addition, one new tensor, shared again by all of them."""
+    values = [None] * len(counts)
+    seen: dict[int, int] = {}      # id(count tensor) -> its host value
+    bump: dict[int, torch.Tensor] = {}  # id -> tensor to advance
+    for k, c in enumerate(counts):
+        if c is None:
+            continue
+        key = id(c)
+        v = seen.get(key)
+        if v is None:
+            v = seen[key] = _host_value(c)
+        values[k] = v
+        if grads[k] is not None and v != INT64_MAX:
+            bump[key] = c
+    if not bump:
+        return list(counts), values
+    olds = list(bump.values())
     by_device: dict[torch.device, list[int]] = {}
-    for k in todo:
-        by_device.setdefault(counts[k].device, []).append(k)
-    for ks in by_device.values():
-        bumped = torch._foreach_add([counts[k] for k in ks], 1)  # one fused launch per device
-        for k, t in zip(ks, bumped):
-            values[k] += 1
-            new[k] = _remember(t, values[k])
+    for j, c in enumerate(olds):
+        by_device.setdefault(c.device, []).append(j)
+    fresh: dict[int, torch.Tensor] = {}
+    for js in by_device.values():
+        bumped = torch._foreach_add([olds[j] for j in js], 1)  # one fused launch per device
+        for j, t in zip(js, bumped):
+            key = id(olds[j])
+            fresh[key] = _remember(t, seen[key] + 1)
+    new = list(counts)
+    for k, c in enumerate(counts):
+        if c is not None and grads[k] is not None:
+            t = fresh.get(id(c))
+            if t is not None:
+                new[k] = t
+                values[k] += 1
     return new, values
 
 
@@ -143,8 +168,8 @@ def _scale_by_accelerated_adam(
     def flatten(tree):
         # a plain list / tuple of tensors and Nones is its own flattening; the general walk
         # (pure Python in torch.utils._pytree) costs ~3 us per leaf per tree
-        if already_flattened or (type(tree) in (list, tuple) and all(
-                t is None or isinstance(t, torch.Tensor) for t in tree)):
+        if already_flattened or (type(tree) in (list, tuple)
+                                 and _PLAIN_LEAVES.issuperset(map(type, tree))):
             return list(tree), None
         return pytree.tree_flatten(tree)
 
@@ -156,12 +181,21 @@ def _scale_by_accelerated_adam(
     def init_fn(params):
         leaves, spec = flatten(params)
         count, mu, nu = [], [], []
+        # The leaves of one device start from ONE 0-dim count tensor and keep sharing the
+        # tensors `update` returns for as long as they step together (a leaf that misses a
+        # gradient falls behind and goes its own way from there).  The values are what the
+        # reference's per-leaf tensors hold; what is saved is a tensor object and an addition per
+        # leaf per step.  Counts are never modified in place here.
+        zeros: dict[torch.device, torch.Tensor] = {}
         for t in leaves:
             if t is None:
                 count.append(None), mu.append(None), nu.append(None)
                 continue
-            zero = torch.zeros(1, dtype=torch.int64, device=t.device).squeeze_()
-            count.append(_remember(zero, 0))
+            zero = zeros.get(t.device)
+            if zero is None:
+                zero = zeros[t.device] = _remember(
+                    torch.zeros(1, dtype=torch.int64, device=t.device).squeeze_(), 0)
+            count.append(zero)
             mu.append(torch.zeros_like(t, requires_grad=moment_requires_grad))
             nu.append(torch.zeros_like(t, requires_grad=moment_requires_grad))
         return ScaleByAdamState(mu=rebuild(mu, params, spec), nu=rebuild(nu, params, spec),
