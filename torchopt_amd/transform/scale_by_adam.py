@@ -6,7 +6,9 @@ Counterpart of /root/reference/torchopt/transform/scale_by_adam.py:225-420 and o
   * validates ``eps >= 0`` and ``0 <= b1, b2 < 1`` (:293-298);
   * ``init(params)`` -> ``ScaleByAdamState(mu, nu, count)`` with, per leaf, zero moments shaped
     like the parameter (``requires_grad=moment_requires_grad``) and a 0-dim int64 count on the
-    leaf's device (:401-414); ``None`` parameters give ``None`` state leaves;
+    leaf's device (:401-414; the leaves of one device share one count tensor for as long as they
+    step together, which the reference's per-leaf tensors of equal value cannot be told from
+    unless somebody writes into one in place); ``None`` parameters give ``None`` state leaves;
   * ``update(updates, state, *, params=None, inplace=True)`` increments the count of every leaf
     whose gradient is not ``None`` (saturating at INT64_MAX), applies the Adam op and returns
     ``(new_updates, ScaleByAdamState(new_mu, new_nu, count_inc))`` with the container types of
