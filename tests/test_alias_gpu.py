@@ -220,3 +220,29 @@ def test_func_optimizer_inner_loop_matches_plain_autograd():
         torch.testing.assert_close(g, r, rtol=1e-8, atol=1e-11)
     with pytest.raises(TypeError):
         topt.FuncOptimizer(object())
+
+
+@pytest.mark.parametrize('inplace', [True, False])
+def test_adamw_mask_decays_only_the_chosen_leaves(inplace):
+    """`mask` as the reference's adamw takes it (alias/adamw.py:62): weights decay, biases do
+    not -- against torch.optim.AdamW with two parameter groups."""
+    model, ref = make_models()
+    lr, wd = 1e-2, 5e-2
+    params = tuple(model.parameters())
+    mask = lambda ps: tuple(p.dim() > 1 for p in ps)  # noqa: E731
+    optim = topt.adamw(lr, weight_decay=wd, mask=mask, use_accelerated_op=True)
+    state = optim.init(params)
+    optim_ref = torch.optim.AdamW([
+        {'params': [p for p in ref.parameters() if p.dim() > 1], 'weight_decay': wd},
+        {'params': [p for p in ref.parameters() if p.dim() <= 1], 'weight_decay': 0.0}], lr)
+    for x, y in batches(4):
+        grads = torch.autograd.grad(((model(x) - y) ** 2).mean(), params)
+        updates, state = optim.update(grads, state, params=params, inplace=inplace)
+        with torch.no_grad():
+            for p, u in zip(params, updates):
+                p.add_(u)
+        optim_ref.zero_grad()
+        ((ref(x) - y) ** 2).mean().backward()
+        optim_ref.step()
+    for p, q in zip(model.parameters(), ref.parameters()):
+        torch.testing.assert_close(p, q, **TOL)

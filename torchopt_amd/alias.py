@@ -117,8 +117,11 @@ def _flip_sign_and_add_weight_decay(weight_decay: float, maximize: bool) -> Grad
     return _stateless(update)
 
 
-def _add_decayed_weights(weight_decay: float) -> GradientTransformation:
-    """``u + wd * p`` after the Adam scaling (transform/add_decayed_weights.py:195-258)."""
+def _add_decayed_weights(weight_decay: float, mask: Any = None) -> GradientTransformation:
+    """``u + wd * p`` after the Adam scaling (transform/add_decayed_weights.py:195-258).  `mask`
+    is a tree of booleans shaped like the parameters, or a callable that makes one from them:
+    leaves marked ``False`` pass through undecayed (transform/add_decayed_weights.py:252-258 via
+    the masked wrapper)."""
     if not weight_decay >= 0.0:
         raise ValueError(f'Invalid weight_decay value: {weight_decay}')
 
@@ -128,12 +131,27 @@ def _add_decayed_weights(weight_decay: float) -> GradientTransformation:
         if params is None:
             raise AssertionError('Parameters are required for weight decay. '
                                  'Call `update(updates, state, params=params)` instead.')
+        if mask is None:
+            chosen = None
+        else:
+            chosen = pytree.tree_flatten(mask(params) if callable(mask) else mask)[0]
         if inplace:
             gs, (ps,) = _tensors(updates, params)
+            if chosen is not None:
+                keep = [k for k, x in enumerate(pytree.tree_flatten(updates)[0]) if x is not None]
+                picked = [j for j, k in enumerate(keep) if chosen[k]]
+                gs, ps = [gs[j] for j in picked], [ps[j] for j in picked]
             if gs:
                 torch._foreach_add_(gs, [p.detach() for p in ps], alpha=weight_decay)
             return updates
-        return _map_leaves(lambda g, p: g.add(p, alpha=weight_decay), updates, params)
+        if chosen is None:
+            return _map_leaves(lambda g, p: g.add(p, alpha=weight_decay), updates, params)
+        marks = iter(chosen)
+        leaves, spec = pytree.tree_flatten(updates)
+        p_leaves = pytree.tree_flatten(params)[0]
+        out = [g if (g is None or not m) else g.add(p, alpha=weight_decay)
+               for g, p, m in zip(leaves, p_leaves, marks)]
+        return pytree.tree_unflatten(out, spec)
 
     return _stateless(update)
 
@@ -193,8 +211,10 @@ def adam(
     eps_root: float = 0.0,
     moment_requires_grad: bool = False,
     maximize: bool = False,
+    use_accelerated_op: bool = True,  # accepted for the reference's call sites; always the case
 ) -> GradientTransformation:
     """Functional Adam on the fused operator (L2 weight decay is added to the gradient)."""
+    del use_accelerated_op
     b1, b2 = betas
     _check(lr, b1, b2, eps, weight_decay)
     return chain(
@@ -211,16 +231,20 @@ def adamw(
     weight_decay: float = 1e-2,
     *,
     eps_root: float = 0.0,
+    mask: Any = None,
     moment_requires_grad: bool = False,
     maximize: bool = False,
+    use_accelerated_op: bool = True,  # accepted for the reference's call sites; always the case
 ) -> GradientTransformation:
-    """Functional AdamW on the fused operator (decoupled decay is added to the scaled update)."""
+    """Functional AdamW on the fused operator (decoupled decay is added to the scaled update;
+    `mask` selects the leaves that decay)."""
+    del use_accelerated_op
     b1, b2 = betas
     _check(lr, b1, b2, eps, weight_decay)
     return chain(
         _flip_sign_and_add_weight_decay(0.0, maximize),
         scale_by_accelerated_adam(b1, b2, eps, eps_root, moment_requires_grad),
-        _add_decayed_weights(weight_decay),
+        _add_decayed_weights(weight_decay, mask),
         _scale_by_neg_lr(lr),
     )
 

@@ -70,7 +70,9 @@ class MetaAdam(_MetaOptimizer):
 
     def __init__(self, module: nn.Module, lr=1e-3, betas=(0.9, 0.999), eps: float = 1e-8,
                  weight_decay: float = 0.0, *, eps_root: float = 0.0,
-                 moment_requires_grad: bool = True, maximize: bool = False) -> None:
+                 moment_requires_grad: bool = True, maximize: bool = False,
+                 use_accelerated_op: bool = True) -> None:
+        del use_accelerated_op  # the reference's keyword; the fused operator is the only path
         super().__init__(module, alias.adam(lr, betas, eps, weight_decay, eps_root=eps_root,
                                             moment_requires_grad=moment_requires_grad,
                                             maximize=maximize))
@@ -80,8 +82,11 @@ class MetaAdamW(_MetaOptimizer):
     """Differentiable AdamW over a module's parameters."""
 
     def __init__(self, module: nn.Module, lr=1e-3, betas=(0.9, 0.999), eps: float = 1e-8,
-                 weight_decay: float = 1e-2, *, eps_root: float = 0.0,
-                 moment_requires_grad: bool = False, maximize: bool = False) -> None:
+                 weight_decay: float = 1e-2, *, eps_root: float = 0.0, mask=None,
+                 moment_requires_grad: bool = False, maximize: bool = False,
+                 use_accelerated_op: bool = True) -> None:
+        del use_accelerated_op
         super().__init__(module, alias.adamw(lr, betas, eps, weight_decay, eps_root=eps_root,
+                                             mask=mask,
                                              moment_requires_grad=moment_requires_grad,
                                              maximize=maximize))
