@@ -242,3 +242,24 @@ def test_fused_adam_with_a_learning_rate_schedule():
                      write_updates=False)
         assert_bit_equal(host(p), hp, f'step {step}')
     np.testing.assert_allclose(host(p), host(q), rtol=2e-5, atol=1e-6)
+
+
+def test_fused_adamw_mask():
+    """Biases exempt from the decay: against torch.optim.AdamW with two parameter groups."""
+    torch.manual_seed(4)
+    net = torch.nn.Sequential(torch.nn.Linear(7, 5), torch.nn.Tanh(), torch.nn.Linear(5, 3)).cuda()
+    ref = torch.nn.Sequential(torch.nn.Linear(7, 5), torch.nn.Tanh(), torch.nn.Linear(5, 3)).cuda()
+    ref.load_state_dict(net.state_dict())
+    opt = FusedAdamW(net.parameters(), lr=1e-2, weight_decay=0.1,
+                     mask=lambda ps: [p.dim() > 1 for p in ps])
+    opt_ref = torch.optim.AdamW([
+        {'params': [p for p in ref.parameters() if p.dim() > 1], 'weight_decay': 0.1},
+        {'params': [p for p in ref.parameters() if p.dim() <= 1], 'weight_decay': 0.0}], lr=1e-2)
+    for _ in range(4):
+        x = torch.randn(16, 7, device='cuda')
+        for model, o in ((net, opt), (ref, opt_ref)):
+            o.zero_grad()
+            model(x).pow(2).mean().backward()
+            o.step()
+    for p, q in zip(net.parameters(), ref.parameters()):
+        torch.testing.assert_close(p, q, rtol=2e-5, atol=1e-6)

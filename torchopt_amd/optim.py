@@ -42,6 +42,7 @@ class FusedAdam:
     `weight_decay` is the L2 kind: added to the gradient before the moments."""
 
     _decoupled = False
+    _mask = None  # FusedAdamW: which parameters decay
 
     def __init__(
         self,
@@ -74,6 +75,7 @@ class FusedAdam:
         self.param_groups: list[tuple[torch.Tensor, ...]] = []
         self.state_groups: list[ScaleByAdamState | None] = []
         self._kinds: list[list[tuple]] = []       # (device, dtype) per parameter
+        self._decays: list[list[bool]] = []       # whether weight decay applies, per parameter
         self._steps: list[list[int] | None] = []  # host-side step numbers per parameter
         self._stale: list[bool] = []              # device count tensors lag the host numbers
         self.add_param_group(params)
@@ -86,6 +88,10 @@ class FusedAdam:
         self.param_groups.append(group)
         self.state_groups.append(None)  # built on the first step, like the reference
         self._kinds.append([(p.device, p.dtype) for p in group])
+        mask = self._mask(group) if callable(self._mask) else self._mask
+        self._decays.append([True] * len(group) if mask is None else [bool(m) for m in mask])
+        if len(self._decays[-1]) != len(group):
+            raise ValueError('mask and parameters differ in length')
         self._steps.append(None)
         self._stale.append(False)
 
@@ -162,9 +168,9 @@ class FusedAdam:
             buckets: dict[tuple, list[int]] = {}
             for k in live:
                 # a schedule makes the rate depend on the leaf's own step count
-                key = (self._kinds[i][k], steps[k] if scheduled else None)
+                key = (self._kinds[i][k], steps[k] if scheduled else None, self._decays[i][k])
                 buckets.setdefault(key, []).append(k)
-            for ks in buckets.values():
+            for key, ks in buckets.items():
                 vals = [steps[k] for k in ks]
                 counts = vals[0] if vals.count(vals[0]) == len(vals) else vals
                 lr = float(self.lr(vals[0] - 1)) if scheduled else self.lr
@@ -176,7 +182,8 @@ class FusedAdam:
                     list(state.nu) if whole else [state.nu[k] for k in ks],
                     self.b1, self.b2, self.eps, self.eps_root, counts, lr,
                     maximize=self.maximize, write_updates=False,
-                    weight_decay=self.weight_decay, decoupled=self._decoupled)
+                    weight_decay=self.weight_decay if key[2] else 0.0,
+                    decoupled=self._decoupled)
         return loss
 
 
@@ -187,8 +194,11 @@ class FusedAdamW(FusedAdam):
     _decoupled = True
 
     def __init__(self, params, lr: float = 1e-3, betas=(0.9, 0.999), eps: float = 1e-8,
-                 weight_decay: float = 1e-2, *, eps_root: float = 0.0,
+                 weight_decay: float = 1e-2, *, eps_root: float = 0.0, mask=None,
                  maximize: bool = False, use_accelerated_op: bool = True) -> None:
+        # `mask`: a sequence of booleans, one per parameter, or a callable that makes one from
+        # the parameters; False exempts a parameter from the decay (optim/adamw.py:60-63)
+        self._mask = mask
         super().__init__(params, lr, betas, eps, weight_decay, eps_root=eps_root,
                          maximize=maximize, use_accelerated_op=use_accelerated_op)
 
