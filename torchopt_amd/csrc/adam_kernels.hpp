@@ -266,12 +266,16 @@ struct IsSpeculative<Op, decltype((void)Op::kSpeculative)> {
     static constexpr bool value = Op::kSpeculative;
 };
 
-// Residency level by element type: 4- and 8-byte types behave alike; the 16-bit types spend
-// twice the ALU time per byte on re-rounding and want more waves, bfloat16 (no native
-// arithmetic) the most.
+// Residency level by element type, measured per op: float32, float64, float16, bfloat16.  (The
+// 16-bit types spend more ALU time per byte on re-rounding, bfloat16 the most.)
+template <typename T>
+constexpr int waves_by_type(int f32, int f64, int half, int bfloat) {
+    return sizeof(T) == 4 ? f32 : sizeof(T) == 8 ? f64 : (__is_same(T, bfloat_t) ? bfloat : half);
+}
+// The multi-tensor kernel's levels were measured on their own: float32 / float64, float16, bfloat16.
 template <typename T>
 constexpr int waves_by_type(int wide, int half, int bfloat) {
-    return sizeof(T) != 2 ? wide : (__is_same(T, bfloat_t) ? bfloat : half);
+    return waves_by_type<T>(wide, wide, half, bfloat);
 }
 
 // ---------------------------------------------------------------------------
@@ -285,7 +289,7 @@ template <typename T>
 struct ForwardInplace {
     static constexpr int NIN = 3, NOUT = 3, NPTR = 3;
     // read-modify-write: a tight window wins
-    static constexpr int kWavesPerCU = waves_by_type<T>(12, 18, 25);
+    static constexpr int kWavesPerCU = waves_by_type<T>(12, 10, 16, 32);
     static constexpr int kWavesPerCUMulti = waves_by_type<T>(16, 21, 32);
     // outputs are produced as (mu', nu', updates') and stored in that order
     __device__ static constexpr int out_slot(int j) { return j == 0 ? 1 : (j == 1 ? 2 : 0); }
@@ -319,7 +323,7 @@ struct ForwardInplace {
 template <typename T>
 struct ForwardMu {
     static constexpr int NIN = 2, NOUT = 1, NPTR = 3;
-    static constexpr int kWavesPerCU = waves_by_type<T>(25, 32, 32);
+    static constexpr int kWavesPerCU = 25;
     static constexpr int kWavesPerCUMulti = 32;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T b1;
@@ -332,7 +336,7 @@ struct ForwardMu {
 template <typename T>
 struct ForwardNu {
     static constexpr int NIN = 2, NOUT = 1, NPTR = 3;
-    static constexpr int kWavesPerCU = waves_by_type<T>(25, 32, 32);
+    static constexpr int kWavesPerCU = waves_by_type<T>(21, 21, 32, 32);
     static constexpr int kWavesPerCUMulti = 32;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T b2;
@@ -346,7 +350,8 @@ struct ForwardNu {
 template <typename T>
 struct ForwardUpdates {
     static constexpr int NIN = 2, NOUT = 1, NPTR = 3;
-    static constexpr int kWavesPerCU = 32;  // sqrt and divide: needs the waves to hide ALU time
+    // root and quotient: the 16-bit types need every wave to hide the ALU time
+    static constexpr int kWavesPerCU = waves_by_type<T>(21, 18, 32, 32);
     static constexpr int kWavesPerCUMulti = 32;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     static constexpr bool kSpeculative = HasQuickDirection<T>::value;
@@ -374,7 +379,7 @@ struct ForwardUpdates {
 template <typename T>
 struct BackwardMu {
     static constexpr int NIN = 1, NOUT = 2, NPTR = 3;
-    static constexpr int kWavesPerCU = 21;
+    static constexpr int kWavesPerCU = 18;
     static constexpr int kWavesPerCUMulti = 25;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T b1;
@@ -388,7 +393,7 @@ struct BackwardMu {
 template <typename T>
 struct BackwardNu {
     static constexpr int NIN = 2, NOUT = 2, NPTR = 4;
-    static constexpr int kWavesPerCU = 21;
+    static constexpr int kWavesPerCU = 16;
     static constexpr int kWavesPerCUMulti = 25;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T b2;
@@ -403,7 +408,7 @@ struct BackwardNu {
 template <typename T>
 struct BackwardUpdates {
     static constexpr int NIN = 3, NOUT = 2, NPTR = 5;
-    static constexpr int kWavesPerCU = 18;
+    static constexpr int kWavesPerCU = waves_by_type<T>(18, 12, 16, 16);
     static constexpr int kWavesPerCUMulti = 25;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T p1, q2;
@@ -427,7 +432,7 @@ struct BackwardUpdates {
 template <typename T>
 struct ForwardAll {
     static constexpr int NIN = 3, NOUT = 3, NPTR = 6;
-    static constexpr int kWavesPerCU = waves_by_type<T>(14, 18, 25);  // six streams per wave: few waves fill the queues
+    static constexpr int kWavesPerCU = waves_by_type<T>(11, 10, 16, 18);  // six streams per wave: few waves fill the queues
     static constexpr int kWavesPerCUMulti = waves_by_type<T>(18, 21, 32);
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     static constexpr bool kSpeculative = HasQuickDirection<T>::value;
@@ -468,7 +473,7 @@ template <typename T, bool HAS_DM, bool HAS_DV>
 struct BackwardAll {
     static constexpr int NIN = 4 + (HAS_DM ? 1 : 0) + (HAS_DV ? 1 : 0), NOUT = 3,
                          NPTR = NIN + NOUT;
-    static constexpr int kWavesPerCU = waves_by_type<T>(11, 14, 14);  // seven to nine streams per wave
+    static constexpr int kWavesPerCU = waves_by_type<T>(10, 10, 11, 14);  // seven to nine streams per wave
     static constexpr int kWavesPerCUMulti = waves_by_type<T>(14, 16, 16);
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T b1, b2, p1, q2;
@@ -512,7 +517,7 @@ __device__ __forceinline__ double toa_fma(double a, double b, double c) { return
 template <typename T, bool WRITE_UPDATES>
 struct FusedStep {
     static constexpr int NIN = 4, NOUT = WRITE_UPDATES ? 4 : 3, NPTR = 4;
-    static constexpr int kWavesPerCU = 12;
+    static constexpr int kWavesPerCU = waves_by_type<T>(12, 10, 12, 12);
     static constexpr int kWavesPerCUMulti = 16;
     // outputs: mu', nu', params', then the scaled update
     __device__ static constexpr int out_slot(int j) { return j == 3 ? 0 : j + 1; }
@@ -715,6 +720,15 @@ __global__ __launch_bounds__(kBlock) void stream_kernel(const Op op, const Tenso
     const bool aligned = all_aligned16<T, Op>(tp);
     for (size_t tile = blockIdx.x; tile < num_tiles; tile += gridDim.x)
         process_tile<T, Op, UNROLL, NT>(op, tp, n, tile, aligned);
+}
+
+// The common case without its branches: every pointer 16-byte aligned and only whole tiles,
+// one workgroup per tile.  The host launches this over the whole tiles of a tensor and hands a
+// ragged last tile to stream_kernel.
+template <typename T, class Op, int UNROLL, bool NT>
+__global__ __launch_bounds__(kBlock) void full_tiles_kernel(const Op op,
+                                                            const TensorPtrs<T, Op> tp) {
+    tile_full<T, Op, UNROLL, NT>(op, tp, (size_t)blockIdx.x * Tile<T, UNROLL>::VECS);
 }
 
 // ---------------------------------------------------------------------------

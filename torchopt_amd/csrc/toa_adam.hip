@@ -113,6 +113,21 @@ int launch_single(const Op &op, T *const (&ptrs)[Op::NPTR], size_t n, void *stre
         tp.p[i] = ptrs[i];
     }
     constexpr size_t tile = Tile<T, kUnroll>::ELEMS;
+    // Aligned operands: the whole tiles go to the branch-free kernel, one workgroup each; a
+    // ragged last tile (or a tensor beyond the grid cap, or unaligned operands) to the general one.
+    uintptr_t bits = 0;
+    for (int i = 0; i < Op::NPTR; ++i) bits |= reinterpret_cast<uintptr_t>(ptrs[i]);
+    const size_t whole = n / tile;
+    if ((bits & 15u) == 0 && whole > 0 && whole <= g_max_grid.load(std::memory_order_relaxed)) {
+        hipLaunchKernelGGL((full_tiles_kernel<T, Op, kUnroll, kNonTemporal>), dim3((unsigned)whole),
+                           dim3(kBlock), lds_reservation<Op>(false, whole), (hipStream_t)stream,
+                           op, tp);
+        if (const int rc = (int)hipGetLastError()) return rc;
+        const size_t done = whole * tile;
+        if (done == n) return 0;
+        for (int i = 0; i < Op::NPTR; ++i) tp.p[i] += done;
+        n -= done;
+    }
     const size_t num_tiles = (n + tile - 1) / tile;
     hipLaunchKernelGGL((stream_kernel<T, Op, kUnroll, kNonTemporal>), dim3(grid_for(num_tiles)),
                        dim3(kBlock), lds_reservation<Op>(false, num_tiles), (hipStream_t)stream, op, tp,
