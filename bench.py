@@ -49,7 +49,7 @@ BYTES_PER_ELEM = {  # op -> number of arrays streamed (multiply by the element s
 # each scaled by what the same counter reads for a plain 1 GiB copy: x1.99996 and x1.0); the
 # commands and raw readings are in profiles/*pmc_traffic*.md.  Not measured live: a counter run
 # serialises the kernels, so it cannot share a process with the timed region.
-MEASURED_TRAFFIC_BYTES = {2: 6442486906, 4: 8516628944}
+MEASURED_TRAFFIC_BYTES = {2: 6442431962, 4: 8516628944}
 
 B1, B2, EPS = 0.9, 0.999, 1e-8
 

@@ -28,7 +28,8 @@ NP = {'f32': np.float32, 'f64': np.float64}
 CODE = {'f32': _lib.TOA_F32, 'f64': _lib.TOA_F64}
 HYPERS = [(0.9, 0.999, 1e-8, 0.0, 10), (0.9, 0.999, 1e-8, 1e-8, 5), (0.8, 0.95, 1e-6, 1e-10, 77)]
 SIZES = [1, 2, 3, 4, 5, 7, 255, 256, 1023, 1024, 1025, 4095, 4096, 4097, 8191, 12289, 65537,
-         1 << 20, (1 << 20) + 3]
+         1 << 20, (1 << 20) + 3,
+         (1 << 22) + 777]  # whole tiles to the branch-free kernel, the ragged tail to the general one
 
 
 @pytest.fixture(scope='module', autouse=True)

@@ -94,7 +94,8 @@ def test_golden_vectors(tag):
 def test_sizes_against_oracle(tag):
     """Eight elements per 128-bit access, 512 per tile: sizes around those boundaries."""
     hypers = [(0.9, 0.999, 1e-3, 0.0, 10), (0.9, 0.999, 1e-3, 1e-4, 5), (0.8, 0.95, 1e-2, 1e-3, 77)]
-    for k, n in enumerate([1, 7, 8, 9, 511, 512, 513, 4095, 4097, 65537, (1 << 20) + 5]):
+    for k, n in enumerate([1, 7, 8, 9, 511, 512, 513, 4095, 4097, 65537, (1 << 20) + 5,
+                           (1 << 23) + 777]):  # the last: whole-tile kernel plus a ragged tail
         check_all_seven(tag, draw(tag, n, 700 + n), hypers[k % 3], f'{tag}/n={n}')
 
 

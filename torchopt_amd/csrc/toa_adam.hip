@@ -113,12 +113,15 @@ int launch_single(const Op &op, T *const (&ptrs)[Op::NPTR], size_t n, void *stre
         tp.p[i] = ptrs[i];
     }
     constexpr size_t tile = Tile<T, kUnroll>::ELEMS;
-    // Aligned operands: the whole tiles go to the branch-free kernel, one workgroup each; a
-    // ragged last tile (or a tensor beyond the grid cap, or unaligned operands) to the general one.
+    // Bandwidth-bound launches with aligned operands: the whole tiles go to the branch-free
+    // kernel, one workgroup each, and a ragged last tile to the general kernel.  Launches of one
+    // round of workgroups (latency-bound: a second launch would cost more than the branches),
+    // tensors beyond the grid cap and unaligned operands take the general kernel alone.
     uintptr_t bits = 0;
     for (int i = 0; i < Op::NPTR; ++i) bits |= reinterpret_cast<uintptr_t>(ptrs[i]);
     const size_t whole = n / tile;
-    if ((bits & 15u) == 0 && whole > 0 && whole <= g_max_grid.load(std::memory_order_relaxed)) {
+    if ((bits & 15u) == 0 && whole > kOneRoundTiles &&
+        whole <= g_max_grid.load(std::memory_order_relaxed)) {
         hipLaunchKernelGGL((full_tiles_kernel<T, Op, kUnroll, kNonTemporal>), dim3((unsigned)whole),
                            dim3(kBlock), lds_reservation<Op>(false, whole), (hipStream_t)stream,
                            op, tp);
