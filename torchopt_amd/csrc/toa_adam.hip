@@ -133,9 +133,8 @@ int launch_single(const Op &op, T *const (&ptrs)[Op::NPTR], size_t n, void *stre
     }
     const size_t num_tiles = (n + tile - 1) / tile;
     hipLaunchKernelGGL((stream_kernel<T, Op, kUnroll, kNonTemporal>), dim3(grid_for(num_tiles)),
-                       dim3(kBlock), lds_reservation<Op>(false, num_tiles), (hipStream_t)stream, op, tp,
-                       n,
-                       num_tiles);
+                       dim3(kBlock), lds_reservation<Op>(false, num_tiles), (hipStream_t)stream,
+                       op, tp, n, num_tiles);
     return (int)hipGetLastError();
 }
 
