@@ -308,3 +308,17 @@ def test_inplace_branch_refuses_gradients_it_cannot_overwrite():
     g = [torch.tensor(0.5, device='cuda').expand(6, 40)]
     with pytest.raises(RuntimeError, match='dense'):
         MultiAdamOp(inplace=True)(mu, nu, g, 1)
+
+
+def test_availability_probe_on_the_gpu():
+    """tests/test_accelerated_op.py:47-54 of the reference, for the devices this build serves."""
+    from torchopt_amd import accelerated_op_available
+
+    assert accelerated_op_available()
+    assert accelerated_op_available('cuda')
+    assert accelerated_op_available('cuda:0')
+    assert accelerated_op_available(0)
+    assert accelerated_op_available(torch.device('cuda', 0))
+    assert accelerated_op_available(['cuda', 'cuda:0', 0])
+    assert not accelerated_op_available(['cuda', 'meta'])
+    assert not accelerated_op_available(['cpu', 'cuda'])  # the CPU is not served here
