@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused Adam operator on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config {0,1,2,3,4,5}]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config {0,...,7}]
 
 A "step" is one pass of the hot path over one batch of synthetic state that is already
 resident in HBM: for the default workload (config 2) one fused in-place `forward_` over three
@@ -102,7 +102,16 @@ CONFIGS = {
     5: dict(name='config5: classic optimizer step (Adam + scale(-lr) + apply) in one pass over the '
                  'GPT-2-medium parameter list (float32), count=1; beside it the three-pass chain',
             dtype='f32', shapes=gpt2_medium_shapes(), eps_root=0.0, count=1, fused_step=True),
+    6: dict(name='config6: fused forward_ in place, 268 435 456 float16 elements (arithmetic of '
+                 'the reference CPU op on at::Half: every operation rounded to 16 bits), '
+                 'eps=1e-3, count=1000, a fresh gradient array every step',
+            dtype='f16', n=1 << 28, eps=1e-3, eps_root=0.0, count=1000, fresh_gradients=True),
+    7: dict(name='config7: fused forward_ in place, 268 435 456 bfloat16 elements (arithmetic of '
+                 'the reference CPU op on at::BFloat16), eps=1e-3, count=1000, a fresh gradient array '
+                 'every step',
+            dtype='bf16', n=1 << 28, eps=1e-3, eps_root=0.0, count=1000, fresh_gradients=True),
 }
+ESIZE = {'f32': 4, 'f64': 8, 'f16': 2, 'bf16': 2}
 
 
 # ----------------------------------------------------------------------------- GPU side
@@ -112,9 +121,10 @@ def make_state(torch, n, dtype, seed):
     """updates ~ N(0,1), mu ~ 0.1 N(0,1), nu ~ |0.01 N(0,1)|, generated on the GPU."""
     g = torch.Generator(device='cuda')
     g.manual_seed(seed)
-    u = torch.randn(n, device='cuda', dtype=dtype, generator=g)
-    mu = torch.randn(n, device='cuda', dtype=dtype, generator=g).mul_(0.1)
-    nu = torch.randn(n, device='cuda', dtype=dtype, generator=g).mul_(0.01).abs_()
+    wide = torch.float32 if dtype in (torch.float16, torch.bfloat16) else dtype
+    u = torch.randn(n, device='cuda', dtype=wide, generator=g).to(dtype)
+    mu = torch.randn(n, device='cuda', dtype=wide, generator=g).mul_(0.1).to(dtype)
+    nu = torch.randn(n, device='cuda', dtype=wide, generator=g).mul_(0.01).abs_().to(dtype)
     return u, mu, nu
 
 
@@ -196,9 +206,12 @@ def run_gpu(cfg_id, steps, warmup):
         raise SystemExit('bench.py needs a GPU: the fused Adam op has no CPU path')
     lib = _lib.load()
     cfg = CONFIGS[cfg_id]
-    dtype = torch.float32 if cfg['dtype'] == 'f32' else torch.float64
-    code = _lib.TOA_F32 if cfg['dtype'] == 'f32' else _lib.TOA_F64
-    esize = 4 if cfg['dtype'] == 'f32' else 8
+    dtype = {'f32': torch.float32, 'f64': torch.float64, 'f16': torch.float16,
+             'bf16': torch.bfloat16}[cfg['dtype']]
+    code = {'f32': _lib.TOA_F32, 'f64': _lib.TOA_F64, 'f16': _lib.TOA_F16,
+            'bf16': _lib.TOA_BF16}[cfg['dtype']]
+    esize = ESIZE[cfg['dtype']]
+    eps = cfg.get('eps', EPS)
     stream = torch.cuda.current_stream()
     sptr = stream.cuda_stream
     eps_root, count = cfg['eps_root'], cfg['count']
@@ -347,12 +360,33 @@ def run_gpu(cfg_id, steps, warmup):
         u, mu, nu = make_state(torch, total, dtype, 1000 * cfg_id)
         pu, pm, pv = u.data_ptr(), mu.data_ptr(), nu.data_ptr()
 
-        def step():
-            rc = lib.toa_adam_forward_inplace(code, pu, pm, pv, total, B1, B2, EPS, eps_root,
-                                              count, sptr)
-            if rc:
-                raise RuntimeError(lib.toa_adam_error_string(rc).decode())
         extra = {}
+        if cfg.get('fresh_gradients'):
+            # A training loop hands the step a new gradient every time; re-applying the step to
+            # its own output instead drives every element towards one fixed point, which no real
+            # run does and which the 16-bit kernels' data-dependent quick route would be timed
+            # on.  So each step gets its own freshly drawn gradient array (as many as the step
+            # count, at most 64 of them in rotation).
+            g = torch.Generator(device='cuda')
+            g.manual_seed(1000 * cfg_id + 1)
+            fresh = [torch.randn(total, device='cuda', generator=g).to(dtype)
+                     for _ in range(min(steps + warmup, 64))]
+            ptrs, turn = [t.data_ptr() for t in fresh], [0]
+            extra['gradient_arrays'] = len(fresh)
+
+            def step():
+                k = turn[0]
+                turn[0] = (k + 1) % len(ptrs)
+                rc = lib.toa_adam_forward_inplace(code, ptrs[k], pm, pv, total, B1, B2, eps,
+                                                  eps_root, count, sptr)
+                if rc:
+                    raise RuntimeError(lib.toa_adam_error_string(rc).decode())
+        else:
+            def step():
+                rc = lib.toa_adam_forward_inplace(code, pu, pm, pv, total, B1, B2, eps, eps_root,
+                                                  count, sptr)
+                if rc:
+                    raise RuntimeError(lib.toa_adam_error_string(rc).decode())
         if cfg.get('backward'):
             extra['backward_ops'] = time_backward_ops(torch, lib, code, dtype, total, esize,
                                                       eps_root, count, stream)
@@ -506,7 +540,9 @@ def run_cpu_baseline(cfg_id, budget_s=12.0):
     from oracle import adam_oracle
 
     cfg = CONFIGS[cfg_id]
-    np_dtype = np.float32 if cfg['dtype'] == 'f32' else np.float64
+    tag = cfg['dtype']
+    np_dtype = {'f32': np.float32, 'f64': np.float64, 'f16': np.float16, 'bf16': np.float32}[tag]
+    eps = cfg.get('eps', EPS)
     full = cfg['n'] if 'n' in cfg else sum(numel(s) for s in cfg['shapes'])
     n = min(full, 1 << 26)
 
@@ -525,6 +561,12 @@ def run_cpu_baseline(cfg_id, budget_s=12.0):
     u = np.tile(rng.standard_normal(block).astype(np_dtype), reps)[:n].copy()
     mu = np.tile((0.1 * rng.standard_normal(block)).astype(np_dtype), reps)[:n].copy()
     nu = np.tile(np.abs(0.01 * rng.standard_normal(block)).astype(np_dtype), reps)[:n].copy()
+    if tag == 'bf16':  # bfloat16 travels as uint16 bit patterns on the NumPy side
+        u, mu, nu = (adam_oracle.bf16_bits(a) for a in (u, mu, nu))
+
+    def as_torch(a):
+        t = torch.from_numpy(a.view(np.int16) if tag == 'bf16' else a)
+        return t.view(torch.bfloat16) if tag == 'bf16' else t
 
     ref = None
     try:
@@ -532,36 +574,36 @@ def run_cpu_baseline(cfg_id, budget_s=12.0):
     except Exception as exc:  # noqa: BLE001
         print(f'[bench] compiled reference not usable ({exc}); timing the C port',
               file=sys.stderr)
-    if ref is not None:
-        import torch
-
-        tu, tm, tv = torch.from_numpy(u), torch.from_numpy(mu), torch.from_numpy(nu)
-
-        def one():
-            ref.adam_op.forward_(tu, tm, tv, B1, B2, EPS, cfg['eps_root'], cfg['count'])
-        kind = 'reference'
-    else:
-        def one():
-            adam_oracle.forward_inplace(u, mu, nu, B1, B2, EPS, cfg['eps_root'], cfg['count'])
-        kind = 'port'
-
-    # Parity on this sample: the GPU's first application from the seeded state against the
-    # CPU's (which doubles as the CPU warm-up: threads, page faults).
     import torch
 
     from torchopt_amd import _lib
 
-    dev = [torch.from_numpy(a).cuda() for a in (u, mu, nu)]
+    if ref is not None:
+        tu, tm, tv = as_torch(u), as_torch(mu), as_torch(nu)  # share memory with u, mu, nu
+
+        def one():
+            ref.adam_op.forward_(tu, tm, tv, B1, B2, eps, cfg['eps_root'], cfg['count'])
+        kind = 'reference'
+    else:
+        def one():
+            adam_oracle.forward_inplace(u, mu, nu, B1, B2, eps, cfg['eps_root'], cfg['count'])
+        kind = 'port'
+
+    # Parity on this sample: the GPU's first application from the seeded state against the
+    # CPU's (which doubles as the CPU warm-up: threads, page faults).
+    dev = [as_torch(a).cuda() for a in (u, mu, nu)]
+    code = {'f32': _lib.TOA_F32, 'f64': _lib.TOA_F64, 'f16': _lib.TOA_F16,
+            'bf16': _lib.TOA_BF16}[tag]
     rc = _lib.load().toa_adam_forward_inplace(
-        _lib.TOA_F32 if cfg['dtype'] == 'f32' else _lib.TOA_F64, dev[0].data_ptr(),
-        dev[1].data_ptr(), dev[2].data_ptr(), n, B1, B2, EPS, cfg['eps_root'], cfg['count'],
-        torch.cuda.current_stream().cuda_stream)
+        code, dev[0].data_ptr(), dev[1].data_ptr(), dev[2].data_ptr(), n, B1, B2, eps,
+        cfg['eps_root'], cfg['count'], torch.cuda.current_stream().cuda_stream)
     if rc:
         raise RuntimeError(f'toa_adam_forward_inplace returned {rc}')
     one()
-    itype = np.int32 if np_dtype is np.float32 else np.int64
+    itype = {2: np.int16, 4: np.int32, 8: np.int64}[ESIZE[tag]]
     worst, differing = 0, 0
     for got, want in zip(dev, (u, mu, nu)):
+        got = got.view(torch.int16) if tag == 'bf16' else got
         a = got.cpu().numpy().view(itype).astype(np.int64)
         b = want.view(itype).astype(np.int64)
         lo = np.iinfo(itype).min
@@ -578,7 +620,7 @@ def run_cpu_baseline(cfg_id, budget_s=12.0):
         one()
         times.append(time.perf_counter() - t0)
     med = sorted(times)[len(times) // 2]
-    esize = np.dtype(np_dtype).itemsize
+    esize = ESIZE[tag]
     return {
         'value': n / med, 'unit': 'elements/s', 'cores': cores, 'kind': kind,
         'sample': f'{n} of {full} elements ({cfg["dtype"]}), forward_ in place, '
@@ -644,7 +686,7 @@ def main(argv=None):
         'dtype': cfg['dtype'],
         'data': 'synthetic',
         'config': {'workload': cfg['name'], 'elements': gpu['elements'], 'b1': B1, 'b2': B2,
-                   'eps': EPS, 'eps_root': cfg['eps_root'], 'count': cfg['count'],
+                   'eps': cfg.get('eps', EPS), 'eps_root': cfg['eps_root'], 'count': cfg['count'],
                    'device': gpu['device'], **gpu['extra']},
         'roofline': gpu['roofline'],
     }
