@@ -1,0 +1,165 @@
+"""The two memory schedules of the in-place step -- plain (all loads, then all stores) and staged
+(load g | load mu | store mu', load nu | store nu', store u') -- against the CPU oracle, bit for
+bit, on tensors large enough to take the bandwidth-bound kernels; the fallback to the plain
+schedule when the arrays of a tensor overlap; lists whose arrays lie 16 MiB apart (the layout that
+collides in DRAM and makes a list pick the staged schedule by itself)."""
+
+from __future__ import annotations
+
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import assert_bit_equal
+from oracle import adam_oracle as O
+from torchopt_amd import _lib
+
+pytestmark = pytest.mark.gpu
+
+B1, B2 = 0.9, 0.999
+CODE = {'f32': _lib.TOA_F32, 'f64': _lib.TOA_F64, 'f16': _lib.TOA_F16, 'bf16': _lib.TOA_BF16}
+TORCH = {'f32': torch.float32, 'f64': torch.float64, 'f16': torch.float16, 'bf16': torch.bfloat16}
+# elements per 1 KiB tile, times more tiles than one round of workgroups (8192), plus a ragged tail
+BIG = {'f32': 256 * 9000 + 77, 'f64': 128 * 9000 + 5, 'f16': 512 * 9000 + 301, 'bf16': 512 * 9000 + 301}
+
+
+@pytest.fixture(scope='module', autouse=True)
+def _gpu():
+    assert torch.cuda.is_available(), 'these tests need a GPU; there is no fallback path'
+    lib = _lib.load()
+    yield
+    lib.toa_adam_set_schedule(0)
+    lib.toa_adam_set_waves_per_cu(0)
+    torch.cuda.synchronize()
+
+
+def draw(tag, n, seed):
+    rng = np.random.default_rng(seed)
+
+    def fmt(x):
+        if tag == 'bf16':
+            return O.bf16_bits(x.astype(np.float32))
+        return x.astype({'f32': np.float32, 'f64': np.float64, 'f16': np.float16}[tag])
+
+    return [fmt(rng.standard_normal(n)), fmt(0.1 * rng.standard_normal(n)),
+            fmt(np.abs(0.01 * rng.standard_normal(n)))]
+
+
+def dev(a, tag):
+    a = np.ascontiguousarray(a)
+    if tag == 'bf16':
+        return torch.from_numpy(a.view(np.int16)).cuda().view(torch.bfloat16)
+    return torch.from_numpy(a).cuda()
+
+
+def host(t, tag):
+    if tag == 'bf16':
+        return t.detach().contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+    return t.detach().cpu().numpy()
+
+
+@pytest.mark.parametrize('tag', ['f32', 'f64', 'f16', 'bf16'])
+@pytest.mark.parametrize('schedule', [0, 1, 2])
+def test_both_schedules_match_the_oracle(tag, schedule):
+    lib = _lib.load()
+    n = BIG[tag]
+    eps, eps_root, count = (1e-8, 1e-8, 7) if tag in ('f32', 'f64') else (1e-3, 0.0, 7)
+    u, m, v = draw(tag, n, 11)
+    want = O.forward_inplace(u.copy(), m.copy(), v.copy(), B1, B2, eps, eps_root, count)
+    du, dm, dv = (dev(a, tag) for a in (u, m, v))
+    assert lib.toa_adam_set_schedule(schedule) in (0, 1, 2)
+    print(f'forward_inplace {tag} n={n} schedule={schedule}', flush=True)
+    rc = lib.toa_adam_forward_inplace(CODE[tag], du.data_ptr(), dm.data_ptr(), dv.data_ptr(), n,
+                                      B1, B2, eps, eps_root, count,
+                                      torch.cuda.current_stream().cuda_stream)
+    lib.toa_adam_set_schedule(0)
+    assert rc == 0, lib.toa_adam_error_string(rc)
+    for got, exp, name in zip((du, dm, dv), want, ('updates', 'mu', 'nu')):
+        assert_bit_equal(host(got, tag), exp, f'{tag} schedule {schedule} {name}')
+
+
+@pytest.mark.parametrize('levels', [(14, 16, 18, 21, 25, 32)])
+def test_staged_schedule_at_every_residency_level(levels):
+    """The level only bounds how many workgroups share a compute unit; results cannot depend on it."""
+    lib = _lib.load()
+    n = BIG['f32']
+    u, m, v = draw('f32', n, 12)
+    want = O.forward_inplace(u.copy(), m.copy(), v.copy(), B1, B2, 1e-8, 0.0, 1000)
+    for w in levels:
+        du, dm, dv = (dev(a, 'f32') for a in (u, m, v))
+        lib.toa_adam_set_waves_per_cu(w)
+        print(f'forward_inplace f32 n={n} staged waves={w}', flush=True)
+        rc = lib.toa_adam_forward_inplace(CODE['f32'], du.data_ptr(), dm.data_ptr(),
+                                          dv.data_ptr(), n, B1, B2, 1e-8, 0.0, 1000,
+                                          torch.cuda.current_stream().cuda_stream)
+        lib.toa_adam_set_waves_per_cu(0)
+        assert rc == 0, lib.toa_adam_error_string(rc)
+        for got, exp, name in zip((du, dm, dv), want, ('updates', 'mu', 'nu')):
+            assert_bit_equal(host(got, 'f32'), exp, f'waves {w} {name}')
+
+
+@pytest.mark.parametrize('alias', ['mu is nu', 'all three'])
+def test_overlapping_arrays_keep_the_plain_schedule(alias):
+    """The reference's CPU loop reads an element of all three arrays and then writes mu, nu,
+    updates in that order (adam_op_impl_cpu.cpp:47-61), so with aliased arrays the last write
+    wins.  The staged schedule would read nu after writing mu; the library must notice the overlap
+    and keep the plain schedule, whose result is the reference's."""
+    lib = _lib.load()
+    n = BIG['f32']
+    rng = np.random.default_rng(5)
+    buf = (np.abs(0.05 * rng.standard_normal(n)) + 1e-3).astype(np.float32)
+    g = rng.standard_normal(n).astype(np.float32)
+    dbuf, dg = dev(buf, 'f32'), dev(g, 'f32')
+    if alias == 'mu is nu':
+        O.forward_inplace(g, buf, buf, B1, B2, 1e-8, 0.0, 3)  # same array twice, as on the GPU
+        pu = dg.data_ptr()
+    else:
+        O.forward_inplace(buf, buf, buf, B1, B2, 1e-8, 0.0, 3)
+        pu = dbuf.data_ptr()
+    lib.toa_adam_set_schedule(2)  # staged wherever it is legal: here it is not
+    print(f'forward_inplace f32 n={n} aliased: {alias}', flush=True)
+    rc = lib.toa_adam_forward_inplace(CODE['f32'], pu, dbuf.data_ptr(), dbuf.data_ptr(), n, B1,
+                                      B2, 1e-8, 0.0, 3, torch.cuda.current_stream().cuda_stream)
+    lib.toa_adam_set_schedule(0)
+    assert rc == 0, lib.toa_adam_error_string(rc)
+    assert_bit_equal(host(dbuf, 'f32'), buf, f'aliased ({alias}) state')
+    if alias == 'mu is nu':
+        assert_bit_equal(host(dg, 'f32'), g, f'aliased ({alias}) updates')
+
+
+@pytest.mark.parametrize('schedule', [0, 1, 2])
+def test_list_with_colliding_arrays(schedule):
+    """Leaves whose three arrays lie exactly 16 MiB apart (GPT-2-medium's 4096 x 1024 float32
+    weights allocated side by side): the list picks the staged schedule by itself."""
+    lib = _lib.load()
+    S, K = 4 << 20, 3  # 16 MiB arrays, three leaves; plus one small ragged leaf elsewhere
+    rng = np.random.default_rng(8)
+    arena = (np.abs(0.05 * rng.standard_normal(3 * S * K)) + 1e-3).astype(np.float32)
+    small = [a.astype(np.float32) for a in draw('f32', 70_001, 9)]
+    d_arena = dev(arena, 'f32')
+    d_small = [dev(a, 'f32') for a in small]
+    base = d_arena.data_ptr()
+    pu = [base + 4 * (3 * k) * S for k in range(K)] + [d_small[0].data_ptr()]
+    pm = [p + 4 * S for p in pu[:K]] + [d_small[1].data_ptr()]
+    pv = [p + 8 * S for p in pu[:K]] + [d_small[2].data_ptr()]
+    ns = [S] * K + [70_001]
+    num = K + 1
+    arr = lambda ps: (ctypes.c_void_p * num)(*ps)
+    lib.toa_adam_set_schedule(schedule)
+    print(f'forward_inplace_multi f32 colliding list schedule={schedule}', flush=True)
+    rc = lib.toa_adam_forward_inplace_multi(CODE['f32'], num, arr(pu), arr(pm), arr(pv),
+                                            (ctypes.c_size_t * num)(*ns), B1, B2, 1e-8, 0.0, None,
+                                            4, torch.cuda.current_stream().cuda_stream)
+    lib.toa_adam_set_schedule(0)
+    assert rc == 0, lib.toa_adam_error_string(rc)
+    got = host(d_arena, 'f32')
+    for k in range(K):
+        u, m, v = (arena[(3 * k + a) * S:(3 * k + a + 1) * S].copy() for a in range(3))
+        O.forward_inplace(u, m, v, B1, B2, 1e-8, 0.0, 4)
+        for a, exp, name in zip(range(3), (u, m, v), ('updates', 'mu', 'nu')):
+            assert_bit_equal(got[(3 * k + a) * S:(3 * k + a + 1) * S], exp, f'leaf {k} {name}')
+    O.forward_inplace(small[0], small[1], small[2], B1, B2, 1e-8, 0.0, 4)
+    for t, exp, name in zip(d_small, small, ('updates', 'mu', 'nu')):
+        assert_bit_equal(host(t, 'f32'), exp, f'small leaf {name}')

@@ -20,7 +20,15 @@
 //     make 32, 25, 21, 18, 16, 14, 12, 11, 10 ... the levels that exist; the
 //     in-place step peaks at 12 waves per CU, the out-of-place ops at 18-32;
 //   * every array is touched once, so loads and stores carry the
-//     non-temporal hint (worth ~10 %).
+//     non-temporal hint (worth ~10 %);
+//   * the in-place step runs a staged schedule (tile_full_staged): one memory
+//     operation of a wave at a time, each result stored as soon as it exists --
+//     load g | load mu | store mu', load nu | store nu', store u'.  A wave then
+//     never presents the memory system with three reads (or three writes) to
+//     three arrays at once.  That is worth 1.5-2 % where the arrays lie a
+//     multiple of 2 MiB apart (what a caching allocator hands out for large
+//     tensors) and removes a 10-17 % loss where they lie a multiple of 16 MiB
+//     apart (three accesses of one wave then meet in one DRAM bank).
 //
 // Arithmetic follows /root/reference/src/adam_op/adam_op_impl_cpu.cpp to the
 // rounding: every product and sum is rounded on its own (build with
@@ -183,6 +191,10 @@ __device__ __forceinline__ void st(V *p, V v) {
         *p = v;
 }
 
+// Waits until every memory operation this wave has issued is complete; the compiler may not move
+// loads or stores across it.
+__device__ __forceinline__ void wait_for_memory() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 __device__ __forceinline__ float toa_sqrt(float x) { return sqrtf(x); }
 __device__ __forceinline__ double toa_sqrt(double x) { return sqrt(x); }
 // a 16-bit value picks the float overload; the root is NOT rounded back
@@ -266,6 +278,18 @@ struct IsSpeculative<Op, decltype((void)Op::kSpeculative)> {
     static constexpr bool value = Op::kSpeculative;
 };
 
+// An op is staged when its three outputs come from three steps that need the inputs one after
+// the other:  a = first(in0, in1),  b = second(in0, in2),  c = third(a, b)  (third_quick for the
+// speculative 16-bit route).  tile_full_staged() stores a and b as soon as they exist.
+template <class Op, class = void>
+struct IsStaged {
+    static constexpr bool value = false;
+};
+template <class Op>
+struct IsStaged<Op, decltype((void)Op::kStaged)> {
+    static constexpr bool value = Op::kStaged;
+};
+
 // Residency level by element type, measured per op: float32, float64, float16, bfloat16.  (The
 // 16-bit types spend more ALU time per byte on re-rounding, bfloat16 the most.)
 template <typename T>
@@ -284,39 +308,61 @@ constexpr int waves_by_type(int wide, int half, int bfloat) {
 // best number of resident single-wave workgroups per compute unit.
 // ---------------------------------------------------------------------------
 
+// The three steps of one Adam update as the reference writes them (adam_op_impl_cpu.cpp:47-61):
+// the two moments, then the step direction from the bias-corrected moments.  Shared by the
+// in-place step and the one-pass differentiable forward.
+template <typename T>
+struct AdamSteps {
+    T b1, b2, c1, c2, eps, eps_root;
+    __device__ __forceinline__ T first(T g, T m) const { return b1 * m + (1 - b1) * g; }
+    __device__ __forceinline__ T second(T g, T v) const { return b2 * v + (1 - b2) * g * g; }
+    __device__ __forceinline__ T third(T m1, T v1) const {
+        const T mh = m1 * c1;
+        const T vh = v1 * c2;
+        return adam_direction(mh, vh, eps_root, eps);
+    }
+    __device__ __forceinline__ bool third_quick(T m1, T v1, T &out) const {
+        const T mh = m1 * c1;
+        const T vh = v1 * c2;
+        bool ok = true;
+        if constexpr (HasQuickDirection<T>::value)
+            out = adam_direction_quick(mh, vh, eps_root, eps, ok);
+        else
+            out = adam_direction(mh, vh, eps_root, eps);
+        return ok;
+    }
+    template <bool QUICK>
+    __device__ __forceinline__ bool run(const T (&in)[3], T (&out)[3]) const {
+        out[0] = first(in[0], in[1]);
+        out[1] = second(in[0], in[2]);
+        if constexpr (QUICK) return third_quick(out[0], out[1], out[2]);
+        out[2] = third(out[0], out[1]);
+        return true;
+    }
+    __device__ __forceinline__ void operator()(const T (&in)[3], T (&out)[3]) const {
+        run<false>(in, out);
+    }
+    __device__ __forceinline__ bool quick(const T (&in)[3], T (&out)[3]) const {
+        return run<true>(in, out);
+    }
+};
+
 // adam_op_impl_cpu.cpp:47-61.  Slots: 0 updates, 1 mu, 2 nu.
 template <typename T>
-struct ForwardInplace {
+struct ForwardInplace : AdamSteps<T> {
     static constexpr int NIN = 3, NOUT = 3, NPTR = 3;
     // read-modify-write: a tight window wins
     static constexpr int kWavesPerCU = waves_by_type<T>(12, 10, 16, 32);
     static constexpr int kWavesPerCUMulti = waves_by_type<T>(16, 21, 32);
+    // The staged schedule (tile_full_staged) exposes a wave's whole arithmetic between its memory
+    // operations; bfloat16's re-rounding makes that long enough to cost more than the schedule
+    // gains (5.9 against 6.3 TB/s), so bfloat16 keeps the plain one.
+    static constexpr bool kStaged = !__is_same(T, bfloat_t);
+    static constexpr int kWavesPerCUStaged = waves_by_type<T>(18, 18, 21, 32);
+    static constexpr int kWavesPerCUMultiStaged = waves_by_type<T>(25, 25, 32);
     // outputs are produced as (mu', nu', updates') and stored in that order
     __device__ static constexpr int out_slot(int j) { return j == 0 ? 1 : (j == 1 ? 2 : 0); }
     static constexpr bool kSpeculative = HasQuickDirection<T>::value;
-    T b1, b2, c1, c2, eps, eps_root;
-    template <bool QUICK>
-    __device__ __forceinline__ bool run(const T (&in)[NIN], T (&out)[NOUT]) const {
-        const T g = in[0], m = in[1], v = in[2];
-        const T m1 = b1 * m + (1 - b1) * g;
-        const T v1 = b2 * v + (1 - b2) * g * g;
-        const T mh = m1 * c1;
-        const T vh = v1 * c2;
-        out[0] = m1;
-        out[1] = v1;
-        bool ok = true;
-        if constexpr (QUICK)
-            out[2] = adam_direction_quick(mh, vh, eps_root, eps, ok);
-        else
-            out[2] = adam_direction(mh, vh, eps_root, eps);
-        return ok;
-    }
-    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
-        run<false>(in, out);
-    }
-    __device__ __forceinline__ bool quick(const T (&in)[NIN], T (&out)[NOUT]) const {
-        return run<true>(in, out);
-    }
 };
 
 // adam_op_impl_cpu.cpp:103-108.  Slots: 0 updates, 1 mu, 2 mu_out.
@@ -430,35 +476,12 @@ struct BackwardUpdates {
 // float32 element, one launch instead of three).  Same expressions as ForwardInplace, written
 // to fresh outputs.  Slots: 0 updates, 1 mu, 2 nu, 3 new_mu, 4 new_nu, 5 new_updates.
 template <typename T>
-struct ForwardAll {
+struct ForwardAll : AdamSteps<T> {
     static constexpr int NIN = 3, NOUT = 3, NPTR = 6;
     static constexpr int kWavesPerCU = waves_by_type<T>(11, 10, 16, 18);  // six streams per wave: few waves fill the queues
     static constexpr int kWavesPerCUMulti = waves_by_type<T>(18, 21, 32);
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     static constexpr bool kSpeculative = HasQuickDirection<T>::value;
-    T b1, b2, c1, c2, eps, eps_root;
-    template <bool QUICK>
-    __device__ __forceinline__ bool run(const T (&in)[NIN], T (&out)[NOUT]) const {
-        const T g = in[0], m = in[1], v = in[2];
-        const T m1 = b1 * m + (1 - b1) * g;
-        const T v1 = b2 * v + (1 - b2) * g * g;
-        const T mh = m1 * c1;
-        const T vh = v1 * c2;
-        out[0] = m1;
-        out[1] = v1;
-        bool ok = true;
-        if constexpr (QUICK)
-            out[2] = adam_direction_quick(mh, vh, eps_root, eps, ok);
-        else
-            out[2] = adam_direction(mh, vh, eps_root, eps);
-        return ok;
-    }
-    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
-        run<false>(in, out);
-    }
-    __device__ __forceinline__ bool quick(const T (&in)[NIN], T (&out)[NOUT]) const {
-        return run<true>(in, out);
-    }
 };
 
 // The whole backward of that step in one pass: backward_updates, the two sums autograd would
@@ -617,6 +640,56 @@ __device__ __forceinline__ void tile_full(const Op &op, const TensorPtrs<T, Op> 
                    out[j][k]);
 }
 
+// The staged schedule of a whole tile for ops with three inputs and three outputs (IsStaged): one
+// memory operation of the wave in flight at a time (two where a store and the next load go out
+// together), every result stored as soon as it exists:
+//     load in0 | load in1 | store out0, load in2 | store out1, store out2
+// Same arithmetic as tile_full, other order of memory operations -- so the arrays of a tensor
+// must not overlap one another (the host checks; tile_full loads everything before it stores).
+template <typename T, class Op, bool NT>
+__device__ __forceinline__ void tile_full_staged(const Op &op, const TensorPtrs<T, Op> &tp,
+                                                 size_t vec_base) {
+    static_assert(Op::NIN == 3 && Op::NOUT == 3, "three in, three out");
+    using V = typename Vec<T>::type;
+    constexpr int VN = Vec<T>::N;
+    const size_t v0 = vec_base + threadIdx.x;
+    const V g = ld<NT>(reinterpret_cast<const V *>(tp.p[0]) + v0);
+    wait_for_memory();
+    const V m = ld<NT>(reinterpret_cast<const V *>(tp.p[1]) + v0);
+    wait_for_memory();
+    V a;
+#pragma unroll
+    for (int e = 0; e < VN; ++e) Vec<T>::set(a, e, op.first(Vec<T>::get(g, e), Vec<T>::get(m, e)));
+    st<NT>(reinterpret_cast<V *>(tp.p[Op::out_slot(0)]) + v0, a);
+    const V v = ld<NT>(reinterpret_cast<const V *>(tp.p[2]) + v0);
+    wait_for_memory();
+    V b;
+#pragma unroll
+    for (int e = 0; e < VN; ++e) Vec<T>::set(b, e, op.second(Vec<T>::get(g, e), Vec<T>::get(v, e)));
+    st<NT>(reinterpret_cast<V *>(tp.p[Op::out_slot(1)]) + v0, b);
+    V c;
+    if constexpr (IsSpeculative<Op>::value) {
+        uint32_t redo = 0;
+#pragma unroll
+        for (int e = 0; e < VN; ++e) {
+            T r;
+            if (!op.third_quick(Vec<T>::get(a, e), Vec<T>::get(b, e), r)) redo |= 1u << e;
+            Vec<T>::set(c, e, r);
+        }
+        if (redo != 0) {  // rare: an element the quick route could not settle
+#pragma unroll
+            for (int e = 0; e < VN; ++e)
+                if (redo & (1u << e))
+                    Vec<T>::set(c, e, op.third(Vec<T>::get(a, e), Vec<T>::get(b, e)));
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < VN; ++e)
+            Vec<T>::set(c, e, op.third(Vec<T>::get(a, e), Vec<T>::get(b, e)));
+    }
+    st<NT>(reinterpret_cast<V *>(tp.p[Op::out_slot(2)]) + v0, c);
+}
+
 // All pointers 16-byte aligned, tile cut short by the end of the tensor:
 // `rem` (< Tile::ELEMS) elements remain from element index `base`.
 template <typename T, class Op, int UNROLL>
@@ -693,16 +766,19 @@ __device__ __forceinline__ bool all_aligned16(const TensorPtrs<T, Op> &tp) {
     return (bits & 15u) == 0;
 }
 
-template <typename T, class Op, int UNROLL, bool NT>
+template <typename T, class Op, int UNROLL, bool NT, bool STAGED = false>
 __device__ __forceinline__ void process_tile(const Op &op, const TensorPtrs<T, Op> &tp, size_t n,
                                              size_t tile, bool aligned) {
     using TL = Tile<T, UNROLL>;
     const size_t base = tile * TL::ELEMS;
     const size_t left = n - base;
     if (aligned) {
-        if (left >= (size_t)TL::ELEMS)
-            tile_full<T, Op, UNROLL, NT>(op, tp, tile * TL::VECS);
-        else
+        if (left >= (size_t)TL::ELEMS) {
+            if constexpr (STAGED)
+                tile_full_staged<T, Op, NT>(op, tp, tile * TL::VECS);
+            else
+                tile_full<T, Op, UNROLL, NT>(op, tp, tile * TL::VECS);
+        } else
             tile_partial<T, Op, UNROLL>(op, tp, base, (uint32_t)left);
     } else {
         const uint32_t cnt = left >= (size_t)TL::ELEMS ? (uint32_t)TL::ELEMS : (uint32_t)left;
@@ -725,10 +801,14 @@ __global__ __launch_bounds__(kBlock) void stream_kernel(const Op op, const Tenso
 // The common case without its branches: every pointer 16-byte aligned and only whole tiles,
 // one workgroup per tile.  The host launches this over the whole tiles of a tensor and hands a
 // ragged last tile to stream_kernel.
-template <typename T, class Op, int UNROLL, bool NT>
+template <typename T, class Op, int UNROLL, bool NT, bool STAGED = false>
 __global__ __launch_bounds__(kBlock) void full_tiles_kernel(const Op op,
                                                             const TensorPtrs<T, Op> tp) {
-    tile_full<T, Op, UNROLL, NT>(op, tp, (size_t)blockIdx.x * Tile<T, UNROLL>::VECS);
+    static_assert(!STAGED || UNROLL == 1, "the staged schedule handles one vector per lane");
+    if constexpr (STAGED)
+        tile_full_staged<T, Op, NT>(op, tp, (size_t)blockIdx.x * Tile<T, UNROLL>::VECS);
+    else
+        tile_full<T, Op, UNROLL, NT>(op, tp, (size_t)blockIdx.x * Tile<T, UNROLL>::VECS);
 }
 
 // ---------------------------------------------------------------------------
@@ -775,7 +855,7 @@ struct MultiTable {
     uint32_t total;  // tiles in this launch
 };
 
-template <typename T, class Op, int UNROLL, bool NT>
+template <typename T, class Op, int UNROLL, bool NT, bool STAGED = false>
 __global__ __launch_bounds__(kBlock) void multi_stream_kernel(const Op op,
                                                               const MultiTable<T, Op> tab) {
     using Table = MultiTable<T, Op>;
@@ -795,7 +875,8 @@ __global__ __launch_bounds__(kBlock) void multi_stream_kernel(const Op op,
 #pragma unroll
         for (int i = 0; i < Op::NPTR; ++i) tp.p[i] = rec.p[i];
         const bool aligned = all_aligned16<T, Op>(tp);
-        process_tile<T, Op, UNROLL, NT>(op, tp, (size_t)rec.n, (size_t)(tile - first), aligned);
+        process_tile<T, Op, UNROLL, NT, STAGED>(op, tp, (size_t)rec.n, (size_t)(tile - first),
+                                                aligned);
     }
 }
 
