@@ -163,3 +163,79 @@ def test_list_with_colliding_arrays(schedule):
     O.forward_inplace(small[0], small[1], small[2], B1, B2, 1e-8, 0.0, 4)
     for t, exp, name in zip(d_small, small, ('updates', 'mu', 'nu')):
         assert_bit_equal(host(t, 'f32'), exp, f'small leaf {name}')
+
+
+@pytest.mark.parametrize('tag', ['f32', 'f64', 'f16', 'bf16'])
+@pytest.mark.parametrize('schedule', [1, 2])
+def test_forward_all_both_schedules(tag, schedule):
+    """The one-pass differentiable forward equals forward_mu, forward_nu, forward_updates."""
+    lib = _lib.load()
+    n = BIG[tag]
+    eps, eps_root, count = (1e-8, 1e-8, 3) if tag in ('f32', 'f64') else (1e-3, 0.0, 3)
+    u, m, v = draw(tag, n, 21)
+    e_mu, e_nu = O.forward_mu(u, m, B1), O.forward_nu(u, v, B2)
+    e_u = O.forward_updates(e_mu, e_nu, B1, B2, eps, eps_root, count)
+    du, dm, dv = (dev(a, tag) for a in (u, m, v))
+    outs = [torch.empty_like(du) for _ in range(3)]
+    lib.toa_adam_set_schedule(schedule)
+    print(f'forward_all {tag} n={n} schedule={schedule}', flush=True)
+    rc = lib.toa_adam_forward_all(CODE[tag], du.data_ptr(), dm.data_ptr(), dv.data_ptr(), n, B1,
+                                  B2, eps, eps_root, count, outs[0].data_ptr(),
+                                  outs[1].data_ptr(), outs[2].data_ptr(),
+                                  torch.cuda.current_stream().cuda_stream)
+    lib.toa_adam_set_schedule(0)
+    assert rc == 0, lib.toa_adam_error_string(rc)
+    for got, exp, name in zip(outs, (e_mu, e_nu, e_u), ('new_mu', 'new_nu', 'new_updates')):
+        assert_bit_equal(host(got, tag), exp, f'{tag} schedule {schedule} {name}')
+    for got, exp, name in zip((du, dm, dv), (u, m, v), ('updates', 'mu', 'nu')):
+        assert_bit_equal(host(got, tag), exp, f'{tag} schedule {schedule} input {name} untouched')
+
+
+@pytest.mark.parametrize('tag', ['f32', 'f64'])
+@pytest.mark.parametrize('schedule', [0, 1, 2])
+@pytest.mark.parametrize('variant', ['adam', 'adam maximize', 'adam + L2', 'adamw', 'adamw maximize'])
+def test_fused_step_both_schedules(tag, schedule, variant):
+    lib = _lib.load()
+    n = BIG[tag]
+    wd = 0.0 if variant.startswith('adam') and '+' not in variant and 'w' not in variant else 0.02
+    decoupled, maximize = 'adamw' in variant, 'maximize' in variant
+    write_updates = variant in ('adam', 'adamw maximize')
+    rng = np.random.default_rng(31)
+    np_t = {'f32': np.float32, 'f64': np.float64}[tag]
+    p = rng.standard_normal(n).astype(np_t)
+    g, m, v = draw(tag, n, 32)
+    dp, dg, dm, dv = (dev(a, tag) for a in (p, g, m, v))
+    O.fused_step(p, g, m, v, B1, B2, 1e-8, 1e-8, 9, 0.01, maximize, write_updates, wd, decoupled)
+    lib.toa_adam_set_schedule(schedule)
+    print(f'fused_step {tag} n={n} schedule={schedule} {variant}', flush=True)
+    rc = lib.toa_adam_fused_step(CODE[tag], dp.data_ptr(), dg.data_ptr(), dm.data_ptr(),
+                                 dv.data_ptr(), n, B1, B2, 1e-8, 1e-8, 9, 0.01, wd, int(decoupled),
+                                 int(maximize), int(write_updates),
+                                 torch.cuda.current_stream().cuda_stream)
+    lib.toa_adam_set_schedule(0)
+    assert rc == 0, lib.toa_adam_error_string(rc)
+    for got, exp, name in zip((dp, dg, dm, dv), (p, g, m, v), ('params', 'updates', 'mu', 'nu')):
+        assert_bit_equal(host(got, tag), exp, f'{tag} schedule {schedule} {variant} {name}')
+
+
+def test_fused_step_list_takes_the_staged_schedule():
+    """A ragged list through toa_adam_fused_step_multi (lists are staged for this op)."""
+    lib = _lib.load()
+    sizes = [BIG['f32'], 5, 0, 70_001, 256 * 8200]
+    rng = np.random.default_rng(41)
+    host_lists = []
+    for k, n in enumerate(sizes):
+        g, m, v = draw('f32', n, 42 + k)
+        host_lists.append([rng.standard_normal(n).astype(np.float32), g, m, v])
+    dev_lists = [[dev(a, 'f32') for a in leaf] for leaf in host_lists]
+    num = len(sizes)
+    col = lambda j: (ctypes.c_void_p * num)(*[leaf[j].data_ptr() for leaf in dev_lists])
+    print('fused_step_multi f32 ragged list', flush=True)
+    rc = lib.toa_adam_fused_step_multi(CODE['f32'], num, col(0), col(1), col(2), col(3),
+                                       (ctypes.c_size_t * num)(*sizes), B1, B2, 1e-8, 0.0, None, 2,
+                                       1e-3, 0.01, 1, 0, 1, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, lib.toa_adam_error_string(rc)
+    for k, (h, d) in enumerate(zip(host_lists, dev_lists)):
+        O.fused_step(h[0], h[1], h[2], h[3], B1, B2, 1e-8, 0.0, 2, 1e-3, False, True, 0.01, True)
+        for got, exp, name in zip(d, h, ('params', 'updates', 'mu', 'nu')):
+            assert_bit_equal(host(got, 'f32'), exp, f'leaf {k} {name}')

@@ -290,6 +290,32 @@ struct IsStaged<Op, decltype((void)Op::kStaged)> {
     static constexpr bool value = Op::kStaged;
 };
 
+// What a staged op sees of its tile: one 128-bit vector per lane of every array.
+template <typename T, class Op, bool NT>
+struct StagedIO {
+    using V = typename Vec<T>::type;
+    T *const *p;  // the tensor's pointer slots
+    size_t v0;    // this lane's vector index
+    __device__ __forceinline__ V load(int slot) const {
+        return ld<NT>(reinterpret_cast<const V *>(p[slot]) + v0);
+    }
+    __device__ __forceinline__ void store(int slot, V x) const {
+        st<NT>(reinterpret_cast<V *>(p[slot]) + v0, x);
+    }
+    // every memory operation issued so far is complete; nothing moves across
+    __device__ __forceinline__ void wait() const { wait_for_memory(); }
+};
+
+// r[e] = f(a[e], b[e]) over the elements of two vectors
+template <typename T, class F>
+__device__ __forceinline__ typename Vec<T>::type vmap(const typename Vec<T>::type &a,
+                                                      const typename Vec<T>::type &b, F f) {
+    typename Vec<T>::type r;
+#pragma unroll
+    for (int e = 0; e < Vec<T>::N; ++e) Vec<T>::set(r, e, f(Vec<T>::get(a, e), Vec<T>::get(b, e)));
+    return r;
+}
+
 // Residency level by element type, measured per op: float32, float64, float16, bfloat16.  (The
 // 16-bit types spend more ALU time per byte on re-rounding, bfloat16 the most.)
 template <typename T>
@@ -331,6 +357,41 @@ struct AdamSteps {
             out = adam_direction(mh, vh, eps_root, eps);
         return ok;
     }
+    // load in0 | load in1 | store out0, load in2 | store out1, store out2
+    template <class Op, class IO>
+    __device__ __forceinline__ void staged_steps(const IO &io) const {
+        using V = typename Vec<T>::type;
+        constexpr int VN = Vec<T>::N;
+        const V g = io.load(0);
+        io.wait();
+        const V m = io.load(1);
+        io.wait();
+        const V a = vmap<T>(g, m, [&](T x, T y) { return first(x, y); });
+        io.store(Op::out_slot(0), a);
+        const V v = io.load(2);
+        io.wait();
+        const V b = vmap<T>(g, v, [&](T x, T y) { return second(x, y); });
+        io.store(Op::out_slot(1), b);
+        V c;
+        if constexpr (HasQuickDirection<T>::value) {
+            uint32_t redo = 0;
+#pragma unroll
+            for (int e = 0; e < VN; ++e) {
+                T r;
+                if (!third_quick(Vec<T>::get(a, e), Vec<T>::get(b, e), r)) redo |= 1u << e;
+                Vec<T>::set(c, e, r);
+            }
+            if (redo != 0) {  // rare: an element the quick route could not settle
+#pragma unroll
+                for (int e = 0; e < VN; ++e)
+                    if (redo & (1u << e))
+                        Vec<T>::set(c, e, third(Vec<T>::get(a, e), Vec<T>::get(b, e)));
+            }
+        } else {
+            c = vmap<T>(a, b, [&](T x, T y) { return third(x, y); });
+        }
+        io.store(Op::out_slot(2), c);
+    }
     template <bool QUICK>
     __device__ __forceinline__ bool run(const T (&in)[3], T (&out)[3]) const {
         out[0] = first(in[0], in[1]);
@@ -359,10 +420,16 @@ struct ForwardInplace : AdamSteps<T> {
     // gains (5.9 against 6.3 TB/s), so bfloat16 keeps the plain one.
     static constexpr bool kStaged = !__is_same(T, bfloat_t);
     static constexpr int kWavesPerCUStaged = waves_by_type<T>(18, 18, 21, 32);
-    static constexpr int kWavesPerCUMultiStaged = waves_by_type<T>(25, 25, 32);
+    // A list gains nothing from the staged schedule (6.51 TB/s either way on the GPT-2-medium
+    // list) unless its arrays collide in DRAM, so lists are staged only then.
+    static constexpr bool kStagedLists = false;
     // outputs are produced as (mu', nu', updates') and stored in that order
     __device__ static constexpr int out_slot(int j) { return j == 0 ? 1 : (j == 1 ? 2 : 0); }
     static constexpr bool kSpeculative = HasQuickDirection<T>::value;
+    template <class IO>
+    __device__ __forceinline__ void staged(const IO &io) const {
+        this->template staged_steps<ForwardInplace>(io);
+    }
 };
 
 // adam_op_impl_cpu.cpp:103-108.  Slots: 0 updates, 1 mu, 2 mu_out.
@@ -480,8 +547,17 @@ struct ForwardAll : AdamSteps<T> {
     static constexpr int NIN = 3, NOUT = 3, NPTR = 6;
     static constexpr int kWavesPerCU = waves_by_type<T>(11, 10, 16, 18);  // six streams per wave: few waves fill the queues
     static constexpr int kWavesPerCUMulti = waves_by_type<T>(18, 21, 32);
+    // measured: float64 6.75 against 6.55 TB/s, float16 6.69 against 6.46; float32 loses
+    // (6.45 against 6.62) and bfloat16 is bound by its arithmetic
+    static constexpr bool kStaged = __is_same(T, double) || __is_same(T, half_t);
+    static constexpr int kWavesPerCUStaged = waves_by_type<T>(18, 18, 21, 32);
+    static constexpr bool kStagedLists = false;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     static constexpr bool kSpeculative = HasQuickDirection<T>::value;
+    template <class IO>
+    __device__ __forceinline__ void staged(const IO &io) const {
+        this->template staged_steps<ForwardAll>(io);
+    }
 };
 
 // The whole backward of that step in one pass: backward_updates, the two sums autograd would
@@ -542,26 +618,73 @@ struct FusedStep {
     static constexpr int NIN = 4, NOUT = WRITE_UPDATES ? 4 : 3, NPTR = 4;
     static constexpr int kWavesPerCU = waves_by_type<T>(12, 10, 12, 12);
     static constexpr int kWavesPerCUMulti = 16;
+    // staged: 6.77 against 6.66 TB/s on one tensor, 6.61 against 6.41 on the GPT-2-medium list
+    static constexpr bool kStaged = true;
+    static constexpr int kWavesPerCUStaged = 21;
+    static constexpr bool kStagedLists = true;
     // outputs: mu', nu', params', then the scaled update
     __device__ static constexpr int out_slot(int j) { return j == 3 ? 0 : j + 1; }
     T b1, b2, c1, c2, eps, eps_root, neg_lr, wd;
     int decay;
     bool maximize;
-    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
-        T g = maximize ? -in[0] : in[0];
-        const T m = in[1], v = in[2], p = in[3];
+    // the gradient the moments see
+    __device__ __forceinline__ T gradient(T g, T p) const {
+        g = maximize ? -g : g;
         if (decay == kDecayIntoGradient) g = toa_fma(wd, p, g);
-        const T m1 = b1 * m + (1 - b1) * g;
-        const T v1 = b2 * v + (1 - b2) * g * g;
+        return g;
+    }
+    __device__ __forceinline__ T first(T g, T m) const { return b1 * m + (1 - b1) * g; }
+    __device__ __forceinline__ T second(T g, T v) const { return b2 * v + (1 - b2) * g * g; }
+    __device__ __forceinline__ T direction(T m1, T v1) const {
         const T mh = m1 * c1;
         const T vh = v1 * c2;
-        T u1 = adam_direction(mh, vh, eps_root, eps);
+        return adam_direction(mh, vh, eps_root, eps);
+    }
+    // the scaled update from the direction
+    __device__ __forceinline__ T scaled(T u1, T p) const {
         if (decay == kDecayIntoUpdate) u1 = toa_fma(wd, p, u1);
-        const T step = u1 * neg_lr;
+        return u1 * neg_lr;
+    }
+    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
+        const T p = in[3];
+        const T g = gradient(in[0], p);
+        const T m1 = first(g, in[1]);
+        const T v1 = second(g, in[2]);
+        const T step = scaled(direction(m1, v1), p);
         out[0] = m1;
         out[1] = v1;
         out[2] = p + step;
         if constexpr (WRITE_UPDATES) out[3] = step;
+    }
+    // load g [and p, when the gradient needs it] | load mu | store mu', load nu |
+    // store nu', load p | store p' [and the scaled update]
+    template <class IO>
+    __device__ __forceinline__ void staged(const IO &io) const {
+        using V = typename Vec<T>::type;
+        const bool early_p = decay == kDecayIntoGradient;
+        V g = io.load(0);
+        V p;
+        if (early_p) p = io.load(3);
+        io.wait();
+        if (early_p || maximize) {
+            if (!early_p) p = g;  // any value: gradient() ignores it without that decay
+            g = vmap<T>(g, p, [&](T x, T y) { return gradient(x, y); });
+        }
+        const V m = io.load(1);
+        io.wait();
+        const V m1 = vmap<T>(g, m, [&](T x, T y) { return first(x, y); });
+        io.store(1, m1);
+        const V v = io.load(2);
+        io.wait();
+        const V v1 = vmap<T>(g, v, [&](T x, T y) { return second(x, y); });
+        io.store(2, v1);
+        if (!early_p) p = io.load(3);
+        const V u1 = vmap<T>(m1, v1, [&](T x, T y) { return direction(x, y); });
+        if (!early_p) io.wait();
+        const V step = vmap<T>(u1, p, [&](T x, T y) { return scaled(x, y); });
+        const V p1 = vmap<T>(p, step, [&](T x, T y) { return x + y; });
+        io.store(3, p1);
+        if constexpr (WRITE_UPDATES) io.store(0, step);
     }
 };
 
@@ -640,54 +763,16 @@ __device__ __forceinline__ void tile_full(const Op &op, const TensorPtrs<T, Op> 
                    out[j][k]);
 }
 
-// The staged schedule of a whole tile for ops with three inputs and three outputs (IsStaged): one
-// memory operation of the wave in flight at a time (two where a store and the next load go out
-// together), every result stored as soon as it exists:
-//     load in0 | load in1 | store out0, load in2 | store out1, store out2
-// Same arithmetic as tile_full, other order of memory operations -- so the arrays of a tensor
-// must not overlap one another (the host checks; tile_full loads everything before it stores).
+// The staged schedule of a whole tile (ops with IsStaged): the op's own program of loads, waits
+// and stores, one memory operation of the wave in flight at a time (two where a store and the
+// next load go out together), every result stored as soon as it exists.  Same arithmetic as
+// tile_full, other order of memory operations -- so the arrays of a tensor must not overlap one
+// another (the host checks; tile_full loads everything before it stores).
 template <typename T, class Op, bool NT>
 __device__ __forceinline__ void tile_full_staged(const Op &op, const TensorPtrs<T, Op> &tp,
                                                  size_t vec_base) {
-    static_assert(Op::NIN == 3 && Op::NOUT == 3, "three in, three out");
-    using V = typename Vec<T>::type;
-    constexpr int VN = Vec<T>::N;
-    const size_t v0 = vec_base + threadIdx.x;
-    const V g = ld<NT>(reinterpret_cast<const V *>(tp.p[0]) + v0);
-    wait_for_memory();
-    const V m = ld<NT>(reinterpret_cast<const V *>(tp.p[1]) + v0);
-    wait_for_memory();
-    V a;
-#pragma unroll
-    for (int e = 0; e < VN; ++e) Vec<T>::set(a, e, op.first(Vec<T>::get(g, e), Vec<T>::get(m, e)));
-    st<NT>(reinterpret_cast<V *>(tp.p[Op::out_slot(0)]) + v0, a);
-    const V v = ld<NT>(reinterpret_cast<const V *>(tp.p[2]) + v0);
-    wait_for_memory();
-    V b;
-#pragma unroll
-    for (int e = 0; e < VN; ++e) Vec<T>::set(b, e, op.second(Vec<T>::get(g, e), Vec<T>::get(v, e)));
-    st<NT>(reinterpret_cast<V *>(tp.p[Op::out_slot(1)]) + v0, b);
-    V c;
-    if constexpr (IsSpeculative<Op>::value) {
-        uint32_t redo = 0;
-#pragma unroll
-        for (int e = 0; e < VN; ++e) {
-            T r;
-            if (!op.third_quick(Vec<T>::get(a, e), Vec<T>::get(b, e), r)) redo |= 1u << e;
-            Vec<T>::set(c, e, r);
-        }
-        if (redo != 0) {  // rare: an element the quick route could not settle
-#pragma unroll
-            for (int e = 0; e < VN; ++e)
-                if (redo & (1u << e))
-                    Vec<T>::set(c, e, op.third(Vec<T>::get(a, e), Vec<T>::get(b, e)));
-        }
-    } else {
-#pragma unroll
-        for (int e = 0; e < VN; ++e)
-            Vec<T>::set(c, e, op.third(Vec<T>::get(a, e), Vec<T>::get(b, e)));
-    }
-    st<NT>(reinterpret_cast<V *>(tp.p[Op::out_slot(2)]) + v0, c);
+    const StagedIO<T, Op, NT> io{tp.p, vec_base + threadIdx.x};
+    op.staged(io);
 }
 
 // All pointers 16-byte aligned, tile cut short by the end of the tensor:

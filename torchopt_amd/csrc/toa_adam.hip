@@ -81,7 +81,7 @@ unsigned lds_reservation(bool multi, size_t num_tiles, bool staged = false) {
     if (o) return lds_for_waves(o);
     if (num_tiles <= kOneRoundTiles) return 0;
     if constexpr (IsStaged<Op>::value) {
-        // a list is staged only when its arrays collide, and then wants the single-tensor level
+        // lists run the staged schedule at the single-tensor level
         if (staged) return lds_for_waves(Op::kWavesPerCUStaged);
     }
     return lds_for_waves(multi ? Op::kWavesPerCUMulti : Op::kWavesPerCU);
@@ -212,9 +212,9 @@ int launch_multi(MakeOp make_op, size_t num_tensors,
         if ((n[k] + tile - 1) / tile > 0x7fffffffu) return TOA_ESIZE;
     }
 
-    // A list takes the staged schedule when a quarter or more of its elements belong to tensors
-    // whose arrays collide in DRAM (it then runs 12 % faster; a list without collisions runs the
-    // same either way) and every tensor's arrays are disjoint, which the schedule needs.
+    // A list takes the staged schedule when the op gains from it on any list (kStagedLists), or
+    // when a quarter or more of its elements belong to tensors whose arrays collide in DRAM (it
+    // then runs 12 % faster) -- and every tensor's arrays are disjoint, which the schedule needs.
     bool staged = false;
     if constexpr (IsStaged<Op>::value) {
         const int schedule = g_schedule.load(std::memory_order_relaxed);
@@ -231,7 +231,7 @@ int launch_multi(MakeOp make_op, size_t num_tensors,
                 total += n[k];
                 if (arrays_collide(cp, n[k])) colliding += n[k];
             }
-            staged = disjoint && (schedule == 2 || colliding * 4 >= total);
+            staged = disjoint && (schedule == 2 || Op::kStagedLists || colliding * 4 >= total);
         }
     }
 
