@@ -517,3 +517,28 @@ def test_repeated_steps_track_the_oracle():
         assert_parity(host(gg), g, f'step {step} updates')
     assert_parity(host(gmu), mu, 'mu after 10 steps')
     assert_parity(host(gnu), nu, 'nu after 10 steps')
+
+
+def test_every_residency_override_launches():
+    """toa_adam_set_waves_per_cu reserves dynamic LDS to bound residency (2..32 workgroups per
+    compute unit; up to 55 040 bytes).  Every level must launch and give the oracle's result."""
+    lib = _lib.load()
+    n = 70_001
+    try:
+        for waves in range(2, 33):
+            a = rand(np.float32, n, 900 + waves)
+            want = O.forward_inplace(a['updates'].copy(), a['mu'].copy(), a['nu'].copy(), 0.9,
+                                     0.999, 1e-8, 0.0, 3)
+            u, m, v = dev(a['updates']), dev(a['mu']), dev(a['nu'])
+            lib.toa_adam_set_waves_per_cu(waves)
+            print(f'forward_inplace f32 n={n} waves override {waves}', flush=True)
+            rc = lib.toa_adam_forward_inplace(CODE['f32'], u.data_ptr(), m.data_ptr(),
+                                              v.data_ptr(), n, 0.9, 0.999, 1e-8, 0.0, 3,
+                                              torch.cuda.current_stream().cuda_stream)
+            assert rc == 0, (waves, lib.toa_adam_error_string(rc))
+            for got, exp, name in zip((u, m, v), want, ('updates', 'mu', 'nu')):
+                assert_parity(host(got), exp, f'waves {waves} {name}')
+        assert lib.toa_adam_set_waves_per_cu(1) == 32  # one per CU is not served: back to defaults
+        assert lib.toa_adam_set_waves_per_cu(0) == 0
+    finally:
+        lib.toa_adam_set_waves_per_cu(0)

@@ -204,6 +204,58 @@ def test_differentiable_branch_with_missing_outside_gradients(which):
             assert_bit_equal(host(b.grad), host(a.grad), f'{which} leaf {k} grad wrt {what}')
 
 
+@pytest.mark.parametrize('which', ['no_update_gradient', 'mu_only', 'nothing_for_one_leaf'])
+def test_leaf_whose_update_receives_no_gradient(which):
+    """A leaf whose new_updates does not feed the loss: the per-leaf chain never runs
+    backward_updates for it, so the infinities its new_updates / new_mu ratio may hold must not
+    reach the gradients of the one-pass node either (0 * inf would be NaN), and a -0 outside
+    gradient must stay -0."""
+    rng = np.random.default_rng(33)
+    shapes = [(40,), (9,), (6, 3)]
+    data = [[np.asarray(rng.standard_normal(s), dtype=np.float32) for _ in range(3)]
+            for s in shapes]
+    # leaf 1: a tiny non-zero new_mu under a huge update -> new_updates / new_mu overflows
+    data[1][0][:] = 0.0
+    data[1][1][:] = 1e-38
+    data[1][2][:] = 0.0
+    cots = [[np.asarray(rng.standard_normal(s), dtype=np.float32) for _ in range(3)]
+            for s in shapes]
+    cots[1][0][:3] = -0.0
+
+    def leaves():
+        return [[dev(g).requires_grad_(True), dev(m).requires_grad_(True),
+                 dev(np.abs(v)).requires_grad_(True)] for g, m, v in data]
+
+    def loss_terms(outs):
+        terms = []
+        for k, (new_mu, new_nu, new_u) in enumerate(outs):
+            if k != 1:
+                terms.append((new_u * dev(cots[k][2])).sum())
+                terms.append((new_nu * dev(cots[k][1])).sum())
+            if k == 1 and which == 'nothing_for_one_leaf':
+                continue
+            terms.append((new_mu * dev(cots[k][0])).sum())
+            if k == 1 and which == 'no_update_gradient':
+                terms.append((new_nu * dev(cots[k][1])).sum())
+        return sum(terms)
+
+    single = leaves()
+    op = AdamOp(B1, B2, 0.0, eps_root=0.0, inplace=False)
+    loss_terms([op(m, v, g, 2) for g, m, v in single]).backward()
+    multi = leaves()
+    mop = MultiAdamOp(B1, B2, 0.0, eps_root=0.0, inplace=False)
+    new_mu, new_nu, new_u = mop([x[1] for x in multi], [x[2] for x in multi],
+                                [x[0] for x in multi], 2)
+    assert not torch.isfinite(new_u[1] / new_mu[1]).all()  # the case is what it claims to be
+    loss_terms(list(zip(new_mu, new_nu, new_u))).backward()
+    for k in range(len(shapes)):
+        for a, b, what in zip(single[k], multi[k], ('updates', 'mu', 'nu')):
+            if a.grad is None:
+                assert b.grad is None, f'{which} leaf {k}: {what} got a gradient from nowhere'
+            else:
+                assert_bit_equal(host(b.grad), host(a.grad), f'{which} leaf {k} grad wrt {what}')
+
+
 def test_meta_step_through_the_transformation():
     """A MAML-style inner step: params' = params - lr * adam(grad); the outer loss
     differentiates through the update, the moments and the step."""

@@ -6,6 +6,7 @@ computing it somewhere else."""
 from __future__ import annotations
 
 import ctypes
+import warnings
 import os
 import re
 
@@ -217,3 +218,30 @@ def test_product_never_imports_the_oracle():
                 text = open(os.path.join(root, f)).read()
                 assert not re.search(r'^\s*(from|import)\s+oracle\b', text, flags=re.M), f
                 assert 'liboracle' not in text and 'adam_oracle' not in text, f
+
+
+def test_asking_for_the_non_accelerated_path_warns():
+    """The reference builds another scaler for use_accelerated_op=False
+    (/root/reference/torchopt/alias/adam.py:118); here the request is answered with a warning."""
+    import torchopt_amd
+    from torchopt_amd import alias
+
+    with pytest.warns(UserWarning, match='use_accelerated_op=False'):
+        alias.adam(use_accelerated_op=False)
+    with pytest.warns(UserWarning, match='use_accelerated_op=False'):
+        alias.adamw(use_accelerated_op=False)
+    with pytest.warns(UserWarning, match='use_accelerated_op=False'):
+        torchopt_amd.FusedAdam([torch.zeros(3, requires_grad=True)], use_accelerated_op=False)
+    with warnings.catch_warnings():
+        warnings.simplefilter('error')
+        alias.adam(use_accelerated_op=True)
+
+
+def test_availability_probe_is_loud_about_the_cpu():
+    """TorchOpt answers True for 'cpu' (/root/reference/tests/test_accelerated_op.py:33-34);
+    this build has no CPU kernels and says so."""
+    with pytest.warns(UserWarning, match='no CPU kernels'):
+        assert not accelerated_op_available('cpu')
+    with pytest.warns(UserWarning, match='no CPU kernels'):
+        assert not accelerated_op_available(['cpu', 'cuda'])
+    assert not accelerated_op_available('not-a-device')

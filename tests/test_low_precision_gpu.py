@@ -201,22 +201,30 @@ def test_multi_tensor_and_autograd(tag):
     assert_bit_equal(host(v.grad, tag), gv, 'd nu')
 
 
-def test_throughput_is_reported_not_assumed(capsys):
-    """Not an assertion on speed: prints the in-place step's rate for 2^27 16-bit elements so the
-    log of a GPU run shows where the 16-bit types stand (12 bytes per element)."""
-    n = 1 << 27
-    for tag, dt in TORCH.items():
-        u = torch.randn(n, device='cuda').to(dt)
-        m = (0.1 * torch.randn(n, device='cuda')).to(dt)
-        v = (0.01 * torch.randn(n, device='cuda')).abs().to(dt)
-        for _ in range(20):
-            adam_op.forward_(u, m, v, 0.9, 0.999, 1e-3, 0.0, 10)
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(50):
-            adam_op.forward_(u, m, v, 0.9, 0.999, 1e-3, 0.0, 10)
-        e1.record()
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1) / 50
-        with capsys.disabled():
-            print(f'\n[{tag}] forward_ 2^27 elements: {ms:.4f} ms, {12 * n / ms / 1e6:.0f} GB/s')
+@pytest.mark.parametrize('tag', ['f16', 'bf16'])
+@pytest.mark.parametrize('eps', [-1e-3, -0.25, -4.0, float('nan')])
+def test_negative_eps_takes_the_exact_chain(tag, eps):
+    """The quick route's error bound assumes root + eps does not cancel.  The raw ops accept a
+    negative (or NaN) eps, so those must go through the exact chain: the aligned call (quick
+    route where allowed) against the same data one element off alignment (always exact) and
+    against the CPU oracle, over every new_mu pattern and a spread of new_nu values."""
+    dt = TORCH[tag]
+    every = torch.arange(65536, dtype=torch.int32, device='cuda').to(torch.int16)
+    nus = torch.tensor([0.0, 1e-6, 2.5e-4, 1e-3, 0.0625, 0.25, 1.0, 4.0, 15.9, 16.0, 16.1, 300.0],
+                       device='cuda').to(dt)
+    rows = nus.numel()
+    n = rows * 65536
+    mu = every.repeat(rows).view(dt)
+    nu = nus.repeat_interleave(65536)
+    off_mu = torch.empty(n + 8, dtype=dt, device='cuda')[1:n + 1]
+    off_nu = torch.empty(n + 8, dtype=dt, device='cuda')[1:n + 1]
+    off_mu.copy_(mu)
+    off_nu.copy_(nu)
+    quick = adam_op.forward_updates(mu, nu, 0.9, 0.999, eps, 0.0, 3)
+    exact = adam_op.forward_updates(off_mu, off_nu, 0.9, 0.999, eps, 0.0, 3)
+    with np.errstate(all='ignore'):
+        want = O.forward_updates(host(mu, tag), host(nu, tag), 0.9, 0.999, eps, 0.0, 3)
+    assert_bit_equal(host(exact, tag), want, f'{tag} eps={eps}: element-wise path')
+    assert_bit_equal(host(quick, tag), want, f'{tag} eps={eps}: aligned path')
+
+

@@ -150,20 +150,56 @@ class MultiAdamOp:
             saved, k = ctx.saved_tensors, ctx.k
             b1, b2, _eps, eps_root, counts = ctx.hyper
             new_updates, new_mu, updates = saved[:k], saved[k:2 * k], saved[2 * k:]
+            g_mu, g_nu, g_u = grads[:k], grads[k:2 * k], grads[2 * k:]
+            dupdates: list = [None] * k
+            dmu: list = [None] * k
+            dnu: list = [None] * k
 
-            def outside(gs):
-                # Gradients reaching new_mu / new_nu from outside the step.  None at all: the
-                # kernel skips the addition, as autograd would.  Some: members without one get
-                # -0.0, the exact identity of IEEE addition (x + -0.0 is x for every x, signed
-                # zeros included), so they too come out as if nothing had been added.
-                if all(g is None for g in gs):
-                    return None
-                return [torch.full_like(m, -0.0) if g is None else g for g, m in zip(gs, new_mu)]
+            def pick(seq, idx):
+                return [seq[i] for i in idx]
 
-            d_u = [torch.zeros_like(m) if g is None else g for g, m in zip(grads[2 * k:], new_mu)]
-            dupdates, dmu, dnu = adam_op.backward_all_multi(
-                d_u, outside(grads[:k]), outside(grads[k:2 * k]), list(new_updates),
-                list(new_mu), list(updates), b1, b2, eps_root, counts)
+            def counts_of(idx):
+                return pick(counts, idx) if isinstance(counts, (list, tuple)) else counts
+
+            # Leaves whose new_updates received a gradient: the one-pass backward.
+            live = [i for i in range(k) if g_u[i] is not None]
+            if live:
+                def outside(gs):
+                    # Gradients reaching new_mu / new_nu from outside the step.  None at all:
+                    # the kernel skips the addition, as autograd would.  Some: members without
+                    # one get -0.0, the exact identity of IEEE addition (x + -0.0 is x for every
+                    # x, signed zeros included), so they too come out as if nothing was added.
+                    gs = pick(gs, live)
+                    if all(g is None for g in gs):
+                        return None
+                    return [torch.full_like(new_mu[i], -0.0) if g is None else g
+                            for g, i in zip(gs, live)]
+
+                du, dm, dn = adam_op.backward_all_multi(
+                    pick(g_u, live), outside(g_mu), outside(g_nu), pick(new_updates, live),
+                    pick(new_mu, live), pick(updates, live), b1, b2, eps_root, counts_of(live))
+                for j, i in enumerate(live):
+                    dupdates[i], dmu[i], dnu[i] = du[j], dm[j], dn[j]
+
+            # Leaves whose new_updates received none: the per-leaf chain never runs
+            # backward_updates for them, so nothing of new_updates / new_mu (which may hold
+            # infinities) enters; only the outside gradients flow on through backward_mu and
+            # backward_nu, and a leaf with neither gets no gradient at all.
+            dead = [i for i in range(k) if g_u[i] is None]
+            via_mu = [i for i in dead if g_mu[i] is not None]
+            via_nu = [i for i in dead if g_nu[i] is not None]
+            if via_mu:
+                du, dm = adam_op.backward_mu_multi(pick(g_mu, via_mu), pick(updates, via_mu),
+                                                   pick(updates, via_mu), b1)
+                for j, i in enumerate(via_mu):
+                    dupdates[i], dmu[i] = du[j], dm[j]
+            if via_nu:
+                du, dn = adam_op.backward_nu_multi(pick(g_nu, via_nu), pick(updates, via_nu),
+                                                   pick(updates, via_nu), b2)
+                for j, i in enumerate(via_nu):
+                    # autograd adds the two contributions to d(updates) where both exist
+                    dupdates[i] = du[j] if dupdates[i] is None else dupdates[i] + du[j]
+                    dnu[i] = dn[j]
             return (None, None, *dupdates, *dmu, *dnu)
 
     def __init__(

@@ -26,7 +26,7 @@ from typing import Any, Callable, NamedTuple
 import torch
 from torch.utils import _pytree as pytree
 
-from torchopt_amd.base import GradientTransformation
+from torchopt_amd.base import GradientTransformation, accelerated_only
 from torchopt_amd.transform.scale_by_adam import _inc_counts, _remember, scale_by_accelerated_adam
 
 
@@ -211,10 +211,10 @@ def adam(
     eps_root: float = 0.0,
     moment_requires_grad: bool = False,
     maximize: bool = False,
-    use_accelerated_op: bool = True,  # accepted for the reference's call sites; always the case
+    use_accelerated_op: bool = True,  # False warns: only the accelerated path exists here
 ) -> GradientTransformation:
     """Functional Adam on the fused operator (L2 weight decay is added to the gradient)."""
-    del use_accelerated_op
+    accelerated_only(use_accelerated_op, 'adam')
     b1, b2 = betas
     _check(lr, b1, b2, eps, weight_decay)
     return chain(
@@ -234,11 +234,11 @@ def adamw(
     mask: Any = None,
     moment_requires_grad: bool = False,
     maximize: bool = False,
-    use_accelerated_op: bool = True,  # accepted for the reference's call sites; always the case
+    use_accelerated_op: bool = True,  # False warns: only the accelerated path exists here
 ) -> GradientTransformation:
     """Functional AdamW on the fused operator (decoupled decay is added to the scaled update;
     `mask` selects the leaves that decay)."""
-    del use_accelerated_op
+    accelerated_only(use_accelerated_op, 'adamw')
     b1, b2 = betas
     _check(lr, b1, b2, eps, weight_decay)
     return chain(

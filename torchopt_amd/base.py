@@ -5,6 +5,7 @@ the reference's own."""
 
 from __future__ import annotations
 
+import warnings
 from typing import Any, Callable, NamedTuple
 
 
@@ -14,3 +15,15 @@ class GradientTransformation(NamedTuple):
 
     init: Callable[..., Any]
     update: Callable[..., Any]
+
+
+def accelerated_only(use_accelerated_op: bool, who: str) -> None:
+    """The reference builds a different (pure-PyTorch) scaler when ``use_accelerated_op`` is false
+    (/root/reference/torchopt/alias/adam.py:118).  This package holds the fused operator only, so
+    a caller asking for the other path is told that it still gets the fused one."""
+    if not use_accelerated_op:
+        warnings.warn(
+            f'{who}: use_accelerated_op=False was requested, but torchopt_amd implements the '
+            'accelerated (fused, GPU-only) Adam operator alone; the accelerated path is used. '
+            'Take the non-accelerated scaler from TorchOpt itself if that is what you need.',
+            UserWarning, stacklevel=3)

@@ -218,8 +218,8 @@ __device__ __forceinline__ T adam_direction(T mh, T vh, T eps_root, T eps) {
 // product and quotient: 4.5 * 2^-23 relative).  If q' is further than 16 float ulps from the
 // midpoint between two bfloat16 values, both round to the same bfloat16 and `ok` is set.
 // Otherwise -- about one element in two thousand -- or when an operand is outside the range
-// where the 1-ulp claims hold (denormal, zero divisor, infinity, NaN, negative), the caller
-// runs the exact chain for that element.  Checked against the exact chain for every
+// where the 1-ulp claims hold (denormal, zero divisor, infinity, NaN, negative; a negative eps,
+// with which root + eps can cancel), the caller runs the exact chain for that element.  Checked against the exact chain for every
 // (mu_hat, nu_hat + eps_root) pair of bit patterns.
 template <typename T>
 struct HasQuickDirection {
@@ -244,6 +244,7 @@ __device__ __forceinline__ bfloat_t adam_direction_quick(bfloat_t mh, bfloat_t v
     const uint32_t low = __builtin_bit_cast(uint32_t, q) & 0xffffu;
     const float aq = __builtin_fabsf(q);
     ok = (x == 0.0f || x >= 1.17549435e-38f) &&          // normal or zero radicand
+         e >= 0.0f &&  // no cancellation in root + eps (a negative or NaN eps takes the exact chain)
          d >= 5.42101086e-20f && d <= 1.84467441e19f &&  // 2^-64 .. 2^64
          ((aq >= 7.88860905e-31f && aq <= 1.26765060e30f) || m == 0.0f) &&  // 2^-100 .. 2^100
          (low - 0x7ff0u > 0x20u);  // not within 16 ulps of the midpoint 0x8000
@@ -260,7 +261,7 @@ __device__ __forceinline__ half_t adam_direction_quick(half_t mh, half_t vh, hal
     const float q = m * __builtin_amdgcn_rcpf(d);
     const uint32_t low = __builtin_bit_cast(uint32_t, q) & 0x1fffu;
     const float aq = __builtin_fabsf(q);
-    ok = x >= 0.0f && d >= 5.42101086e-20f && d <= 1.84467441e19f &&
+    ok = x >= 0.0f && e >= 0.0f && d >= 5.42101086e-20f && d <= 1.84467441e19f &&
          ((aq >= 6.10351562e-05f && aq <= 32768.0f) || m == 0.0f) &&  // 2^-14 .. 2^15
          (low - 0x0ff0u > 0x20u);  // not within 16 ulps of the midpoint 0x1000
     return half_t(q);

@@ -33,9 +33,12 @@ constexpr unsigned kMaxGrid = 1u << 25;  // default cap on workgroups per launch
 constexpr int kLdsGranule = 1280;
 constexpr int kLdsGranulesPerCU = 128;
 constexpr int kMaxWavesPerCU = 32;
+// One workgroup per CU would need 83 200 bytes of dynamic LDS, more than the 64 KiB a launch may
+// reserve without raising the kernel's limit; two per CU (55 040 bytes) is the lowest level served.
+constexpr int kMinWavesPerCU = 2;
 
 // Global override of the per-op resident-wave cap: -1 = not yet initialised,
-// 0 = use each op's own kWavesPerCU, 1..32 = that many for every op.  Set by
+// 0 = use each op's own kWavesPerCU, 2..32 = that many for every op.  Set by
 // toa_adam_set_waves_per_cu() or, initially, by the environment variable
 // TOA_ADAM_WAVES_PER_CU (read once).
 std::atomic<int> g_waves_override{-1};
@@ -46,7 +49,7 @@ int waves_override() {
         w = 0;
         if (const char *env = std::getenv("TOA_ADAM_WAVES_PER_CU")) {
             const int v = std::atoi(env);
-            if (v >= 1 && v <= kMaxWavesPerCU) w = v;
+            if (v >= kMinWavesPerCU && v <= kMaxWavesPerCU) w = v;
         }
         g_waves_override.store(w, std::memory_order_relaxed);
     }
@@ -67,6 +70,7 @@ static_assert(lds_for_waves(14) == 11520 && lds_for_waves(16) == 10240, "14 and 
 static_assert(lds_for_waves(25) == 6400 && lds_for_waves(24) == 7680, "25 and 21 per CU");
 static_assert(lds_for_waves(31) == 6400 && lds_for_waves(32) == 0, "25, then no reservation");
 static_assert(lds_for_waves(1) == 65 * 1280, "one per CU: more than half of the LDS");
+static_assert(lds_for_waves(kMinWavesPerCU) <= 64 * 1024, "every served level fits a launch");
 
 // The multi-tensor kernel spends three dependent scalar loads finding its tensor before any
 // memory traffic starts, so its best level sits one or two steps above the single-tensor one.
@@ -406,7 +410,8 @@ int toa_adam_abi_version(void) { return 2; }
 
 int toa_adam_set_waves_per_cu(int waves) {
     const int prev = waves_override();
-    g_waves_override.store(waves >= 1 && waves <= kMaxWavesPerCU ? waves : 0, std::memory_order_relaxed);
+    g_waves_override.store(waves >= kMinWavesPerCU && waves <= kMaxWavesPerCU ? waves : 0,
+                           std::memory_order_relaxed);
     return prev;
 }
 

@@ -15,6 +15,7 @@ import torch
 from torch import nn
 
 from torchopt_amd import alias
+from torchopt_amd.base import accelerated_only
 
 
 __all__ = ['MetaAdam', 'MetaAdamW']
@@ -72,7 +73,7 @@ class MetaAdam(_MetaOptimizer):
                  weight_decay: float = 0.0, *, eps_root: float = 0.0,
                  moment_requires_grad: bool = True, maximize: bool = False,
                  use_accelerated_op: bool = True) -> None:
-        del use_accelerated_op  # the reference's keyword; the fused operator is the only path
+        accelerated_only(use_accelerated_op, 'MetaAdam')
         super().__init__(module, alias.adam(lr, betas, eps, weight_decay, eps_root=eps_root,
                                             moment_requires_grad=moment_requires_grad,
                                             maximize=maximize))
@@ -85,7 +86,7 @@ class MetaAdamW(_MetaOptimizer):
                  weight_decay: float = 1e-2, *, eps_root: float = 0.0, mask=None,
                  moment_requires_grad: bool = False, maximize: bool = False,
                  use_accelerated_op: bool = True) -> None:
-        del use_accelerated_op
+        accelerated_only(use_accelerated_op, 'MetaAdamW')
         super().__init__(module, alias.adamw(lr, betas, eps, weight_decay, eps_root=eps_root,
                                              mask=mask,
                                              moment_requires_grad=moment_requires_grad,

@@ -30,6 +30,7 @@ from typing import Callable, Iterable, Sequence
 import torch
 
 from torchopt_amd.accelerated_op.adam_op import adam_op
+from torchopt_amd.base import accelerated_only
 from torchopt_amd.transform.scale_by_adam import (INT64_MAX, ScaleByAdamState, _host_value,
                                                  _remember)
 
@@ -57,8 +58,8 @@ class FusedAdam:
         use_accelerated_op: bool = True,
     ) -> None:
         # `use_accelerated_op` is accepted so that the reference's constructor calls carry over
-        # (optim/adam.py:56-65); the fused operator is the only path here either way
-        del use_accelerated_op
+        # (optim/adam.py:56-65); the fused operator is the only path here, and False warns
+        accelerated_only(use_accelerated_op, type(self).__name__)
         if not callable(lr) and not lr >= 0.0:
             raise ValueError(f'Invalid learning rate: {lr}')
         if not eps >= 0.0:
