@@ -81,6 +81,23 @@ TOA_API int toa_adam_set_waves_per_cu(int waves);
  * Returns the previous setting.  No counterpart in the reference. */
 TOA_API int toa_adam_set_schedule(int schedule);
 
+/* Lists longer than one kernel-argument table (96 tensors for ops with three pointer slots, 80
+ * with four, 64 with five, fewer beyond) run as ONE launch over a device-resident table, a
+ * "plan": one 96-byte record per tensor, written by small kernels that carry the records in
+ * their arguments and cached per (device, stream, list) in memory the library allocates (at most
+ * 4 plans per stream, 64 per process), with a coarse index from tiles to records in the launch's
+ * own arguments.  A call whose list is cached costs one launch and no other device work.
+ * Under stream capture, or when no plan memory can be had, such lists take one launch per
+ * table instead (every launch then carries its table in its arguments, so a captured graph
+ * depends on nothing a later call may rewrite).
+ *   toa_adam_set_plan_mode   0 (default) as above; 1 never use plans; 2 use plans for every
+ *                            list, however short.  Returns the previous mode.
+ *   toa_adam_release_plans   frees every cached plan (waits for the devices that hold one to
+ *                            drain).  Returns 0 or the last hipError_t.
+ * No counterpart in the reference. */
+TOA_API int toa_adam_set_plan_mode(int mode);
+TOA_API int toa_adam_release_plans(void);
+
 /* Cap on workgroups per launch (default and maximum 2^25).  Every kernel normally runs one
  * workgroup per 1 KiB tile; beyond the cap workgroups stride over the remaining tiles.  Lowering
  * the cap exercises that path on small inputs (tests) and trades dispatch work for loop
@@ -139,8 +156,8 @@ TOA_API int toa_adam_backward_updates(int dtype, const void *dupdates, const voi
 /* ---- multi-tensor entry points ------------------------------------------
  * One call covers a whole list of tensors (a flattened pytree): the host loop
  * the reference runs per leaf (/root/reference/torchopt/transform/
- * scale_by_adam.py:325-332, 378-385) collapses into one launch per
- * TOA_MT_MAX_TENSORS(...) tensors that share a step count.  The arrays of
+ * scale_by_adam.py:325-332, 378-385) collapses into one launch per group of
+ * tensors that share a step count (see toa_adam_set_plan_mode for long lists).  The arrays of
  * pointers, lengths and counts are HOST arrays of num_tensors entries; they
  * are consumed before the call returns.  counts may be NULL when count_all
  * applies to every tensor.  Zero-length tensors are skipped. */

@@ -966,4 +966,107 @@ __global__ __launch_bounds__(kBlock) void multi_stream_kernel(const Op op,
     }
 }
 
+// ---------------------------------------------------------------------------
+// Lists longer than a kernel-argument table: the records live in device memory (a "plan"), so
+// one launch covers a list of any length.
+//
+// A plan is one 96-byte record per tensor.  The launch carries, in its kernel arguments, a
+// coarse index: for every cell of 2^shift consecutive tiles of the global tile numbering, the
+// number of the record that owns the cell's first tile.  A workgroup reads its cell's entry
+// (kernel arguments: hot in the scalar cache), then that record (hot too: thousands of
+// consecutive tiles share it), and has its tensor unless a tensor boundary lies in the cell
+// before its tile; then it walks the records forward, at most as many steps as tensors start
+// inside one cell.  Records reach the device in kernel arguments of small fill kernels (no copy
+// engine, no pinned staging, nothing for a later launch to find changed).
+// ---------------------------------------------------------------------------
+constexpr int kPlanSlots = 9;  // most pointer slots of any op (backward_all with both gradients)
+
+struct alignas(32) PlanRec {
+    void *p[kPlanSlots];
+    uint64_t n;           // elements
+    uint32_t first;       // first global tile of this tensor
+    uint32_t next_first;  // first global tile of the next tensor (the total for the last one)
+    uint32_t index;       // position in the record array
+    uint32_t reserved;
+};
+static_assert(sizeof(PlanRec) == 96, "three 32-byte scalar loads");
+
+constexpr int kPlanCells = 832;  // 3328 bytes of kernel arguments
+
+struct PlanView {
+    const PlanRec *recs;
+    uint32_t total;  // tiles
+    uint32_t shift;  // log2 of the tiles per cell
+    uint32_t num;    // records
+    uint32_t reserved;
+    uint32_t cell[kPlanCells];  // record that owns tile (i << shift)
+};
+
+// What the host knows of one tensor, as it travels in kernel arguments.
+template <int NPTR>
+struct PlanSeed {
+    void *p[NPTR];
+    uint64_t n;
+    uint32_t first, next_first;
+};
+template <int NPTR>
+struct PlanSeedChunk {
+    static constexpr int MAX = 3584 / (int)sizeof(PlanSeed<NPTR>);
+    PlanSeed<NPTR> seed[MAX];
+};
+
+template <int NPTR>
+__global__ __launch_bounds__(128) void plan_fill_kernel(PlanRec *recs, uint32_t at, uint32_t count,
+                                                        const PlanSeedChunk<NPTR> chunk) {
+    const uint32_t i = threadIdx.x;
+    if (i >= count) return;
+    PlanRec r;
+#pragma unroll
+    for (int j = 0; j < kPlanSlots; ++j) r.p[j] = nullptr;
+#pragma unroll
+    for (int j = 0; j < NPTR; ++j) r.p[j] = chunk.seed[i].p[j];
+    r.n = chunk.seed[i].n;
+    r.first = chunk.seed[i].first;
+    r.next_first = chunk.seed[i].next_first;
+    r.index = at + i;
+    r.reserved = 0;
+    recs[at + i] = r;
+}
+static_assert(PlanSeedChunk<kPlanSlots>::MAX >= 1 && PlanSeedChunk<3>::MAX <= 128,
+              "one fill workgroup covers a chunk");
+
+// A record read at a wave-uniform address from memory no kernel writes while this one runs:
+// through the constant address space, so the scalar unit fetches it (three 32-byte loads).
+__device__ __forceinline__ PlanRec load_record(const PlanRec *at) {
+    using ConstWord = const __attribute__((address_space(4))) uint64_t;
+    ConstWord *w = (ConstWord *)at;
+    PlanRec r;
+#pragma unroll
+    for (int j = 0; j < kPlanSlots; ++j) r.p[j] = reinterpret_cast<void *>(w[j]);
+    r.n = w[kPlanSlots];
+    const uint64_t tiles = w[kPlanSlots + 1], rest = w[kPlanSlots + 2];
+    r.first = (uint32_t)tiles;
+    r.next_first = (uint32_t)(tiles >> 32);
+    r.index = (uint32_t)rest;
+    r.reserved = 0;
+    return r;
+}
+
+template <typename T, class Op, int UNROLL, bool NT, bool STAGED = false>
+__global__ __launch_bounds__(kBlock) void plan_stream_kernel(const Op op, const PlanView plan) {
+    for (uint32_t tile = blockIdx.x; tile < plan.total; tile += gridDim.x) {
+        PlanRec rec = load_record(plan.recs + plan.cell[tile >> plan.shift]);
+        // a tensor boundary lies between the cell's first tile and this one: walk on (never
+        // past the last record)
+        while (tile >= rec.next_first && rec.index + 1 < plan.num)
+            rec = load_record(plan.recs + (rec.index + 1));
+        TensorPtrs<T, Op> tp;
+#pragma unroll
+        for (int i = 0; i < Op::NPTR; ++i) tp.p[i] = static_cast<T *>(rec.p[i]);
+        const bool aligned = all_aligned16<T, Op>(tp);
+        process_tile<T, Op, UNROLL, NT, STAGED>(op, tp, (size_t)rec.n, (size_t)(tile - rec.first),
+                                                aligned);
+    }
+}
+
 }  // namespace toa

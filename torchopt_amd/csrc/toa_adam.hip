@@ -12,6 +12,8 @@
 #include <atomic>
 #include <cmath>
 #include <cstdlib>
+#include <cstring>
+#include <mutex>
 #include <type_traits>
 #include <vector>
 
@@ -194,13 +196,157 @@ int launch_single(const Op &op, T *const (&ptrs)[Op::NPTR], size_t n, void *stre
     return (int)hipGetLastError();
 }
 
-// Launch one op over a list of tensors.  `make_op(count)` builds the op's
-// scalars for one step number; tensors are batched per distinct count and per
-// kernel-argument table capacity.
+// ---------------------------------------------------------------------------
+// Plans: device-resident tables for lists longer than one kernel-argument table.
+// ---------------------------------------------------------------------------
+
+// 0 = plans for lists that need more than one kernel-argument table (the default), 1 = never
+// (several launches instead), 2 = for every list (so that small inputs can exercise the path).
+std::atomic<int> g_plan_mode{0};
+
+constexpr size_t kPlanSlotsPerStream = 4;         // cached plans a stream may hold
+constexpr size_t kPlanSlotsTotal = 64;            // and the process as a whole
+
+size_t plan_bytes(size_t num) { return num * sizeof(PlanRec); }
+
+// Writes the records for `seeds` into `mem` (device memory of at least plan_bytes(seeds.size()))
+// on `stream`: fill kernels carrying the records in their arguments.
+template <int NPTR>
+int plan_write(void *mem, const std::vector<PlanSeed<NPTR>> &seeds, hipStream_t stream) {
+    using Chunk = PlanSeedChunk<NPTR>;
+    PlanRec *recs = static_cast<PlanRec *>(mem);
+    const uint32_t num = (uint32_t)seeds.size();
+    Chunk chunk;
+    for (uint32_t at = 0; at < num; at += Chunk::MAX) {
+        const uint32_t count = num - at < (uint32_t)Chunk::MAX ? num - at : Chunk::MAX;
+        std::memcpy(chunk.seed, seeds.data() + at, count * sizeof(PlanSeed<NPTR>));
+        hipLaunchKernelGGL((plan_fill_kernel<NPTR>), dim3(1), dim3(128), 0, stream, recs, at,
+                           count, chunk);
+        if (const int rc = (int)hipGetLastError()) return rc;
+    }
+    return 0;
+}
+
+// The launch's view of a plan: the coarse index from tile cells to records.
+template <int NPTR>
+PlanView plan_view(void *mem, const std::vector<PlanSeed<NPTR>> &seeds, uint32_t total) {
+    PlanView v;
+    v.recs = static_cast<const PlanRec *>(mem);
+    v.total = total;
+    v.num = (uint32_t)seeds.size();
+    v.reserved = 0;
+    v.shift = 0;
+    while ((((uint64_t)total + (1u << v.shift) - 1) >> v.shift) > (uint64_t)kPlanCells) ++v.shift;
+    uint32_t k = 0;
+    for (uint32_t c = 0; c < (uint32_t)kPlanCells; ++c) {
+        const uint64_t tile = (uint64_t)c << v.shift;
+        while (k + 1 < v.num && seeds[k].next_first <= tile) ++k;
+        v.cell[c] = k;
+    }
+    return v;
+}
+
+// Cached plans.  A plan's memory is written and read by work enqueued on ONE stream, so stream
+// order keeps a rewrite behind the launches that still read the old contents; another stream
+// gets another plan.  Keyed by the exact bytes of the records.
+struct PlanSlot {
+    int device = -1;
+    hipStream_t stream = nullptr;
+    void *mem = nullptr;
+    size_t capacity = 0;
+    std::vector<unsigned char> key;  // empty: contents unknown
+    uint64_t stamp = 0;
+};
+std::mutex g_plan_mutex;
+std::vector<PlanSlot> g_plan_slots;
+uint64_t g_plan_stamp = 0;
+
+// Returns device memory holding the plan for `seeds`, written on `stream` if it was not already
+// there; nullptr when no plan can be had (the caller then launches table by table).
+template <int NPTR>
+void *plan_cached(const std::vector<PlanSeed<NPTR>> &seeds, size_t tile, hipStream_t stream,
+                  int *rc) {
+    *rc = 0;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess ||
+        capturing != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return nullptr;  // a captured launch must not lean on memory a later call may rewrite
+    }
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) return nullptr;
+
+    std::vector<unsigned char> key(16 + seeds.size() * sizeof(PlanSeed<NPTR>));
+    const uint64_t head[2] = {(uint64_t)NPTR, (uint64_t)tile};
+    std::memcpy(key.data(), head, 16);
+    std::memcpy(key.data() + 16, seeds.data(), seeds.size() * sizeof(PlanSeed<NPTR>));
+
+    std::lock_guard<std::mutex> lock(g_plan_mutex);
+    PlanSlot *use = nullptr, *oldest = nullptr;
+    size_t mine = 0;
+    for (PlanSlot &slot : g_plan_slots) {
+        if (slot.device != device || slot.stream != stream) continue;
+        ++mine;
+        if (slot.key == key) use = &slot;
+        if (oldest == nullptr || slot.stamp < oldest->stamp) oldest = &slot;
+    }
+    if (use != nullptr) {
+        use->stamp = ++g_plan_stamp;
+        return use->mem;
+    }
+    const size_t need = plan_bytes(seeds.size());
+    if (mine >= kPlanSlotsPerStream || (oldest != nullptr && g_plan_slots.size() >= kPlanSlotsTotal)) {
+        use = oldest;
+        if (use->capacity < need) {
+            // grow: the old memory may still be read by launches in flight on this stream
+            if (hipStreamSynchronize(stream) != hipSuccess) return nullptr;
+            (void)hipFree(use->mem);
+            use->mem = nullptr;
+            use->capacity = 0;
+        }
+    } else if (g_plan_slots.size() < kPlanSlotsTotal) {
+        g_plan_slots.emplace_back();
+        use = &g_plan_slots.back();
+        use->device = device;
+        use->stream = stream;
+    } else {
+        return nullptr;
+    }
+    if (use->mem == nullptr) {
+        const size_t capacity = need + need / 4;
+        if (hipMalloc(&use->mem, capacity) != hipSuccess) {
+            (void)hipGetLastError();
+            use->mem = nullptr;
+            use->key.clear();
+            return nullptr;
+        }
+        use->capacity = capacity;
+    }
+    use->key.clear();
+    *rc = plan_write<NPTR>(use->mem, seeds, stream);
+    if (*rc) return nullptr;
+    use->key = std::move(key);
+    use->stamp = ++g_plan_stamp;
+    return use->mem;
+}
+
+// Memory for the plan of one call, brought by the caller instead of taken from the cache (the
+// entry point that must not allocate).  The plan is rewritten on every call.
+struct PlanArena {
+    void *mem = nullptr;
+    size_t bytes = 0;
+};
+
+// Launch one op over a list of tensors.  `make_op(count)` builds the op's scalars for one step
+// number; tensors are batched per distinct count.  A batch that fits one kernel-argument table
+// is one launch with the table in its arguments; a longer one is one launch over a
+// device-resident plan (cached per stream and list), or -- where no plan can be had: under
+// stream capture, or with plans switched off -- one launch per table.
 template <typename T, class Op, class MakeOp>
 int launch_multi(MakeOp make_op, size_t num_tensors,
                  const void *const *const (&lists)[Op::NPTR],
-                 const size_t *n, const uint64_t *counts, uint64_t count_all, void *stream) {
+                 const size_t *n, const uint64_t *counts, uint64_t count_all, void *stream,
+                 const PlanArena *arena = nullptr) {
     using Table = MultiTable<T, Op>;
     constexpr size_t tile = Tile<T, kUnroll>::ELEMS;
     if (num_tensors == 0) return 0;
@@ -251,6 +397,8 @@ int launch_multi(MakeOp make_op, size_t num_tensors,
         }
     }
 
+    const int plan_mode = g_plan_mode.load(std::memory_order_relaxed);
+    std::vector<PlanSeed<Op::NPTR>> seeds;
     Table tab;
     uint32_t num = 0;       // tensors in the table being filled
     uint32_t next_tile = 0; // tiles in the table being filled
@@ -263,6 +411,68 @@ int launch_multi(MakeOp make_op, size_t num_tensors,
     };
     for (uint64_t c : distinct) {
         const Op op = make_op(c);
+        auto member = [&](size_t k) { return n[k] != 0 && (counts == nullptr || counts[k] == c); };
+
+        // ---- one launch over a device-resident plan
+        size_t live = 0;
+        uint64_t tiles_all = 0;
+        for (size_t k = 0; k < num_tensors; ++k)
+            if (member(k)) {
+                ++live;
+                tiles_all += (n[k] + tile - 1) / tile;
+            }
+        if (live == 0) continue;
+        const bool wants_plan =
+            arena != nullptr || (plan_mode != 1 && (plan_mode == 2 || live > (size_t)Table::MAX));
+        if (wants_plan && tiles_all < kNoTile && live < kNoTile) {
+            seeds.clear();
+            seeds.reserve(live);
+            uint32_t first = 0;
+            for (size_t k = 0; k < num_tensors; ++k) {
+                if (!member(k)) continue;
+                PlanSeed<Op::NPTR> seed;
+                for (int i = 0; i < Op::NPTR; ++i) seed.p[i] = const_cast<void *>(lists[i][k]);
+                seed.n = n[k];
+                seed.first = first;
+                first += (uint32_t)((n[k] + tile - 1) / tile);
+                seed.next_first = first;
+                seeds.push_back(seed);
+            }
+            void *mem = nullptr;
+            if (arena != nullptr) {
+                if (plan_bytes(live) > arena->bytes) return TOA_ESIZE;
+                if (const int rc = plan_write<Op::NPTR>(arena->mem, seeds, (hipStream_t)stream))
+                    return rc;
+                mem = arena->mem;
+            } else {
+                int rc = 0;
+                mem = plan_cached<Op::NPTR>(seeds, tile, (hipStream_t)stream, &rc);
+                if (rc) return rc;
+            }
+            if (mem != nullptr) {
+                const uint32_t total = (uint32_t)tiles_all;
+                const PlanView view = plan_view<Op::NPTR>(mem, seeds, total);
+                // the lookup is two scalar-cache hits, so the launch wants the residency level
+                // of the single-tensor kernel, not the list kernel's raised one
+                const unsigned lds = lds_reservation<Op>(false, total, staged);
+                if (staged) {
+                    if constexpr (IsStaged<Op>::value)
+                        hipLaunchKernelGGL((plan_stream_kernel<T, Op, kUnroll, kNonTemporal, true>),
+                                           dim3(grid_for(total)), dim3(kBlock), lds,
+                                           (hipStream_t)stream, op, view);
+                } else {
+                    hipLaunchKernelGGL((plan_stream_kernel<T, Op, kUnroll, kNonTemporal>),
+                                       dim3(grid_for(total)), dim3(kBlock), lds,
+                                       (hipStream_t)stream, op, view);
+                }
+                if (const int rc = (int)hipGetLastError()) return rc;
+                continue;
+            }
+        } else if (arena != nullptr) {
+            return TOA_ESIZE;
+        }
+
+        // ---- tables in kernel arguments, one launch each
         reset();
         auto flush = [&]() -> int {
             if (num == 0) return 0;
@@ -283,7 +493,7 @@ int launch_multi(MakeOp make_op, size_t num_tensors,
             return (int)hipGetLastError();
         };
         for (size_t k = 0; k < num_tensors; ++k) {
-            if (n[k] == 0 || (counts != nullptr && counts[k] != c)) continue;
+            if (!member(k)) continue;
             const uint64_t tiles = (n[k] + tile - 1) / tile;
             if (num == (uint32_t)Table::MAX || (uint64_t)next_tile + tiles >= kNoTile) {
                 if (int rc = flush()) return rc;
@@ -419,6 +629,27 @@ int toa_adam_set_schedule(int schedule) {
     const int prev = g_schedule.load(std::memory_order_relaxed);
     g_schedule.store(schedule == 1 || schedule == 2 ? schedule : 0, std::memory_order_relaxed);
     return prev;
+}
+
+int toa_adam_set_plan_mode(int mode) {
+    const int prev = g_plan_mode.load(std::memory_order_relaxed);
+    g_plan_mode.store(mode == 1 || mode == 2 ? mode : 0, std::memory_order_relaxed);
+    return prev;
+}
+
+int toa_adam_release_plans(void) {
+    std::lock_guard<std::mutex> lock(g_plan_mutex);
+    int rc = 0;
+    for (PlanSlot &slot : g_plan_slots) {
+        if (slot.mem == nullptr) continue;
+        int current = 0;
+        (void)hipGetDevice(&current);
+        if (current != slot.device) (void)hipSetDevice(slot.device);
+        if (const int e = (int)hipFree(slot.mem)) rc = e;  // waits for the device to drain
+        if (current != slot.device) (void)hipSetDevice(current);
+    }
+    g_plan_slots.clear();
+    return rc;
 }
 
 unsigned toa_adam_set_max_grid(unsigned workgroups) {
