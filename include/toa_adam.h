@@ -50,7 +50,8 @@ enum { TOA_F32 = 0, TOA_F64 = 1, TOA_F16 = 2, TOA_BF16 = 3 };
 enum {
     TOA_EDTYPE = -1, /* dtype not served by this entry point      */
     TOA_ENULL = -2,  /* a required pointer is NULL while n > 0    */
-    TOA_ESIZE = -3   /* a tensor is too large for the launch grid */
+    TOA_ESIZE = -3,  /* a tensor is too large for the launch grid */
+    TOA_ELIMIT = -4  /* beyond a stated limit of the allocation-free entry point */
 };
 
 /* Library ABI version (bumped on any signature change). */
@@ -166,6 +167,25 @@ TOA_API int toa_adam_forward_inplace_multi(int dtype, size_t num_tensors, void *
                                    void *const *mu, void *const *nu, const size_t *n, double b1,
                                    double b2, double eps, double eps_root,
                                    const uint64_t *counts, uint64_t count_all, void *stream);
+
+/* toa_adam_forward_inplace_multi for callers that cannot allocate device memory -- code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in
+ * the reference.  Same arguments, same results bit for bit, always one launch per distinct step
+ * count however long the list; the per-tensor records live in a device array built into the
+ * library (384 KiB on every GPU the library runs on, held until the process ends) instead of
+ * cached allocations, and are rewritten by every call.  It calls no hipMalloc, hipFree or other
+ * allocating routine and records no memset or copy.
+ *   limit    at most 4096 non-empty tensors per call (and device numbers below 64): beyond that
+ *            it returns TOA_ELIMIT and launches nothing.
+ *   sharing  every call on a GPU uses that GPU's one array: calls that overlap in time on one
+ *            GPU (different streams, or replays of graphs that captured it) race; calls ordered
+ *            by one stream, or otherwise serialised, are safe. */
+TOA_API int toa_adam_forward_inplace_multi_noalloc(int dtype, size_t num_tensors,
+                                                   void *const *updates, void *const *mu,
+                                                   void *const *nu, const size_t *n, double b1,
+                                                   double b2, double eps, double eps_root,
+                                                   const uint64_t *counts, uint64_t count_all,
+                                                   void *stream);
 
 TOA_API int toa_adam_forward_mu_multi(int dtype, size_t num_tensors, const void *const *updates,
                               const void *const *mu, const size_t *n, double b1,

@@ -37,6 +37,7 @@ def test_header_declares_the_expected_surface():
     want |= {'toa_adam_abi_version', 'toa_adam_error_string', 'toa_adam_set_waves_per_cu',
              'toa_adam_fused_step', 'toa_adam_fused_step_multi', 'toa_adam_set_max_grid',
              'toa_adam_set_schedule', 'toa_adam_set_plan_mode', 'toa_adam_release_plans',
+             'toa_adam_forward_inplace_multi_noalloc',
              'toa_adam_forward_all', 'toa_adam_forward_all_multi', 'toa_adam_backward_all',
              'toa_adam_backward_all_multi'}
     assert names == want

@@ -45,6 +45,8 @@ SIGNATURES = {
     'toa_adam_backward_updates': [_i, _vp, _vp, _vp, _sz, _d, _d, _d, _u64, _vp, _vp, _vp],
     'toa_adam_forward_inplace_multi': [_i, _sz, _vpp, _vpp, _vpp, _szp, _d, _d, _d, _d, _u64p,
                                        _u64, _vp],
+    'toa_adam_forward_inplace_multi_noalloc': [_i, _sz, _vpp, _vpp, _vpp, _szp, _d, _d, _d, _d,
+                                               _u64p, _u64, _vp],
     'toa_adam_forward_mu_multi': [_i, _sz, _vpp, _vpp, _szp, _d, _vpp, _vp],
     'toa_adam_forward_nu_multi': [_i, _sz, _vpp, _vpp, _szp, _d, _vpp, _vp],
     'toa_adam_forward_updates_multi': [_i, _sz, _vpp, _vpp, _szp, _d, _d, _d, _d, _u64p, _u64,

@@ -19,6 +19,9 @@
 
 #include "adam_kernels.hpp"
 
+// Bytes of the file-scope plan array behind toa_adam_forward_inplace_multi_noalloc: 4096 records.
+constexpr size_t toa_noalloc_scratch_bytes = 4096 * 96;
+
 namespace {
 
 using namespace toa;
@@ -440,7 +443,7 @@ int launch_multi(MakeOp make_op, size_t num_tensors,
             }
             void *mem = nullptr;
             if (arena != nullptr) {
-                if (plan_bytes(live) > arena->bytes) return TOA_ESIZE;
+                if (plan_bytes(live) > arena->bytes) return TOA_ELIMIT;
                 if (const int rc = plan_write<Op::NPTR>(arena->mem, seeds, (hipStream_t)stream))
                     return rc;
                 mem = arena->mem;
@@ -508,6 +511,44 @@ int launch_multi(MakeOp make_op, size_t num_tensors,
         }
         if (int rc = flush()) return rc;
     }
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Plan memory that needs no allocation: a file-scope device array, one copy per GPU, held until
+// the process ends.  Its name is a host-side stand-in, not a device address: hipGetSymbolAddress
+// gives the address of the current device's copy, once per device.
+// ---------------------------------------------------------------------------
+constexpr size_t kNoAllocMaxTensors = 4096;
+constexpr size_t kNoAllocScratchBytes = kNoAllocMaxTensors * sizeof(PlanRec);  // 384 KiB
+static_assert(kNoAllocScratchBytes == toa_noalloc_scratch_bytes, "the array holds every record");
+constexpr int kNoAllocMaxDevices = 64;
+
+}  // namespace
+
+// No device code names the array (kernels receive its address as an argument); the compiler keeps
+// it, with a symbol the runtime can find, because host code names it below.  (Marking it `used`
+// would pin it to a local symbol, which hipGetSymbolAddress cannot resolve.)
+static __device__ __align__(256) unsigned char scratch[toa_noalloc_scratch_bytes];
+
+namespace {
+
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kNoAllocMaxDevices] = {};
+
+// The current device's copy of `scratch`; looked up on the first call on that device.
+int scratch_for_current_device(void **out) {
+    int device = 0;
+    if (const int rc = (int)hipGetDevice(&device)) return rc;
+    if (device < 0 || device >= kNoAllocMaxDevices) return TOA_ELIMIT;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[device] == nullptr) {
+        void *ptr = nullptr;
+        if (const int rc = (int)hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch))) return rc;
+        if (ptr == nullptr) return (int)hipErrorInvalidSymbol;
+        g_scratch_ptr[device] = ptr;
+    }
+    *out = g_scratch_ptr[device];
     return 0;
 }
 
@@ -665,6 +706,9 @@ const char *toa_adam_error_string(int code) {
         case TOA_EDTYPE: return "toa_adam: unsupported dtype for this entry point";
         case TOA_ENULL: return "toa_adam: null pointer for a non-empty tensor";
         case TOA_ESIZE: return "toa_adam: tensor too large for one launch";
+        case TOA_ELIMIT:
+            return "toa_adam: more than 4096 non-empty tensors (or a device number beyond 63) in "
+                   "a call to the allocation-free entry point";
         default: return code > 0 ? hipGetErrorString((hipError_t)code) : "toa_adam: unknown error";
     }
 }
@@ -755,6 +799,31 @@ int toa_adam_forward_inplace_multi(int dtype, size_t num_tensors, void *const *u
         };
         return launch_multi<T, ForwardInplace<T>>(make, num_tensors, lists, n, counts, count_all,
                                                   stream);
+    });
+}
+
+int toa_adam_forward_inplace_multi_noalloc(int dtype, size_t num_tensors, void *const *updates,
+                                           void *const *mu, void *const *nu, const size_t *n,
+                                           double b1, double b2, double eps, double eps_root,
+                                           const uint64_t *counts, uint64_t count_all,
+                                           void *stream) {
+    size_t live = 0;
+    if (n != nullptr)
+        for (size_t k = 0; k < num_tensors; ++k) live += n[k] != 0;
+    if (live > kNoAllocMaxTensors) return TOA_ELIMIT;
+    PlanArena arena;
+    if (live != 0) {
+        if (const int rc = scratch_for_current_device(&arena.mem)) return rc;
+        arena.bytes = kNoAllocScratchBytes;
+    }
+    TOA_DISPATCH_ALL(dtype, [&] {
+        const void *const *const lists[3] = {CPP(updates), CPP(mu), CPP(nu)};
+        auto make = [&](uint64_t c) {
+            const HostScalars s = host_scalars(b1, b2, eps_root, c);
+            return ForwardInplace<T>{(T)b1, (T)b2, (T)s.c1, (T)s.c2, (T)eps, (T)eps_root};
+        };
+        return launch_multi<T, ForwardInplace<T>>(make, num_tensors, lists, n, counts, count_all,
+                                                  stream, live != 0 ? &arena : nullptr);
     });
 }
 
