@@ -290,6 +290,69 @@ TOA_API int toa_adam_fused_step_multi(int dtype, size_t num_tensors, void *const
                                       int decoupled, int maximize, int write_updates,
                                       void *stream);
 
+/* ---- step number on the device ----------------------------------------------
+ * The reference keeps `count` as a 0-dim int64 tensor on the parameters' device
+ * (/root/reference/torchopt/transform/scale_by_adam.py:401-414) and converts it to size_t on every
+ * call (adam_op.cpp:32-48 through pybind11), which reads it back to the host.  The entry points
+ * above take the step number as a host integer for that reason -- and a captured HIP graph then
+ * replays one particular step.  The *_devcount entry points read it from device memory when the
+ * kernel starts, so ONE captured graph serves a whole training loop: the graph advances the
+ * count (toa_adam_count_advance, or any kernel of the caller's) and every replay computes the
+ * next step.
+ *
+ * The bias corrections 1/(1-b1^count), 1/(1-b2^count), 1-b1^count, 1/(1-b2^count+eps_root) must
+ * stay the host's (double precision with libm's pow, rounded once to the element type: that is
+ * what makes results bit-identical to the reference), so the host tabulates them:
+ *   toa_adam_bias_rows         fills host memory with `rows` rows of 4 values of the element type
+ *                              for step numbers first_count, first_count + 1, ...; the caller
+ *                              uploads them (4 * rows * element size bytes).
+ *   toa_adam_bias_rows_needed  how many rows from first_count on make the table exact for EVERY
+ *                              later step: the corrections stop changing once b^count is below
+ *                              half an ulp of 1 (37 411 steps for b2 = 0.999).  0 if that takes
+ *                              more than `limit` rows.
+ *   toa_adam_count_advance     *count += (*count != INT64_MAX), the reference's inc_count
+ *                              (transform/utils.py:111-126), as a one-thread kernel on `stream`.
+ * A step number below first_count uses row 0, one beyond the table the last row.  `bias_rows`
+ * and `count` are device pointers; `count` is read once per wavefront, when the kernel starts.
+ * Entry points exist for the in-place step and the fused optimizer step, single and list (the
+ * ops a training loop captures); everything else about them is as for their host-count forms.
+ * No counterpart in the reference. */
+TOA_API int toa_adam_bias_rows(int dtype, double b1, double b2, double eps_root,
+                               uint64_t first_count, size_t rows, void *host_out);
+TOA_API size_t toa_adam_bias_rows_needed(double b1, double b2, uint64_t first_count,
+                                         size_t limit);
+TOA_API int toa_adam_count_advance(int64_t *count, void *stream);
+
+TOA_API int toa_adam_forward_inplace_devcount(int dtype, void *updates, void *mu, void *nu,
+                                              size_t n, double b1, double b2, double eps,
+                                              double eps_root, const void *bias_rows,
+                                              uint64_t first_count, size_t rows,
+                                              const int64_t *count, void *stream);
+
+TOA_API int toa_adam_forward_inplace_multi_devcount(int dtype, size_t num_tensors,
+                                                    void *const *updates, void *const *mu,
+                                                    void *const *nu, const size_t *n, double b1,
+                                                    double b2, double eps, double eps_root,
+                                                    const void *bias_rows, uint64_t first_count,
+                                                    size_t rows, const int64_t *count,
+                                                    void *stream);
+
+TOA_API int toa_adam_fused_step_devcount(int dtype, void *params, void *updates, void *mu,
+                                         void *nu, size_t n, double b1, double b2, double eps,
+                                         double eps_root, const void *bias_rows,
+                                         uint64_t first_count, size_t rows, const int64_t *count,
+                                         double lr, double weight_decay, int decoupled,
+                                         int maximize, int write_updates, void *stream);
+
+TOA_API int toa_adam_fused_step_multi_devcount(int dtype, size_t num_tensors, void *const *params,
+                                               void *const *updates, void *const *mu,
+                                               void *const *nu, const size_t *n, double b1,
+                                               double b2, double eps, double eps_root,
+                                               const void *bias_rows, uint64_t first_count,
+                                               size_t rows, const int64_t *count, double lr,
+                                               double weight_decay, int decoupled, int maximize,
+                                               int write_updates, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,7 +23,7 @@ HEADER = os.path.join(REPO, 'include', 'toa_adam.h')
 def declared_functions():
     text = open(HEADER).read()
     text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
-    decls = re.findall(r'TOA_API\s+(?:const\s+char\s*\*|int|unsigned)\s*(\w+)\s*\(([^;]*?)\)\s*;', text,
+    decls = re.findall(r'TOA_API\s+(?:const\s+char\s*\*|int|unsigned|size_t)\s*(\w+)\s*\(([^;]*?)\)\s*;', text,
                        flags=re.S)
     return {name: [a.strip() for a in args.split(',')] if args.strip() != 'void' else []
             for name, args in decls}
@@ -37,7 +37,10 @@ def test_header_declares_the_expected_surface():
     want |= {'toa_adam_abi_version', 'toa_adam_error_string', 'toa_adam_set_waves_per_cu',
              'toa_adam_fused_step', 'toa_adam_fused_step_multi', 'toa_adam_set_max_grid',
              'toa_adam_set_schedule', 'toa_adam_set_plan_mode', 'toa_adam_release_plans',
-             'toa_adam_forward_inplace_multi_noalloc',
+             'toa_adam_forward_inplace_multi_noalloc', 'toa_adam_bias_rows',
+             'toa_adam_bias_rows_needed', 'toa_adam_count_advance',
+             'toa_adam_forward_inplace_devcount', 'toa_adam_forward_inplace_multi_devcount',
+             'toa_adam_fused_step_devcount', 'toa_adam_fused_step_multi_devcount',
              'toa_adam_forward_all', 'toa_adam_forward_all_multi', 'toa_adam_backward_all',
              'toa_adam_backward_all_multi'}
     assert names == want

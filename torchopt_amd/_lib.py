@@ -18,7 +18,7 @@ TOA_F32 = 0
 TOA_F64 = 1
 TOA_F16 = 2
 TOA_BF16 = 3
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _vp = ctypes.c_void_p
 _vpp = ctypes.POINTER(ctypes.c_void_p)
@@ -66,6 +66,18 @@ SIGNATURES = {
                             _vp],
     'toa_adam_fused_step_multi': [_i, _sz, _vpp, _vpp, _vpp, _vpp, _szp, _d, _d, _d, _d, _u64p,
                                   _u64, _d, _d, _i, _i, _i, _vp],
+    # step number on the device
+    'toa_adam_bias_rows': [_i, _d, _d, _d, _u64, _sz, _vp],
+    'toa_adam_bias_rows_needed': [_d, _d, _u64, _sz],
+    'toa_adam_count_advance': [_vp, _vp],
+    'toa_adam_forward_inplace_devcount': [_i, _vp, _vp, _vp, _sz, _d, _d, _d, _d, _vp, _u64, _sz,
+                                          _vp, _vp],
+    'toa_adam_forward_inplace_multi_devcount': [_i, _sz, _vpp, _vpp, _vpp, _szp, _d, _d, _d, _d,
+                                                _vp, _u64, _sz, _vp, _vp],
+    'toa_adam_fused_step_devcount': [_i, _vp, _vp, _vp, _vp, _sz, _d, _d, _d, _d, _vp, _u64, _sz,
+                                     _vp, _d, _d, _i, _i, _i, _vp],
+    'toa_adam_fused_step_multi_devcount': [_i, _sz, _vpp, _vpp, _vpp, _vpp, _szp, _d, _d, _d, _d,
+                                           _vp, _u64, _sz, _vp, _d, _d, _i, _i, _i, _vp],
 }
 
 _lib = None
@@ -99,7 +111,8 @@ def load() -> ctypes.CDLL:
             raise ImportError(f'{LIB_PATH}: ABI version {got}, expected {ABI_VERSION}; rebuild it')
         for name, argtypes in SIGNATURES.items():
             fn = getattr(lib, name)
-            fn.restype = ctypes.c_uint if name == 'toa_adam_set_max_grid' else _i
+            fn.restype = {'toa_adam_set_max_grid': ctypes.c_uint,
+                          'toa_adam_bias_rows_needed': ctypes.c_size_t}.get(name, _i)
             fn.argtypes = argtypes
         _lib = lib
     return _lib

@@ -291,6 +291,67 @@ struct IsStaged<Op, decltype((void)Op::kStaged)> {
     static constexpr bool value = Op::kStaged;
 };
 
+// ---------------------------------------------------------------------------
+// Step number on the device.  The reference keeps `count` as a 0-dim device tensor
+// (/root/reference/torchopt/transform/scale_by_adam.py:401-414) and reads it back on every call;
+// the ordinary entry points here take it as a host integer, which a captured graph would freeze.
+// An op wrapped in AtStep reads the step number from device memory when its kernel starts and
+// takes its bias corrections from a table of rows {c1, c2, p1, q2} that the host filled for
+// steps first, first + 1, ... (in double with libm's pow, rounded to the element type: the same
+// values the host-count entry points put into kernel arguments).  Steps before `first` use the
+// first row, steps beyond the table the last one.
+// ---------------------------------------------------------------------------
+template <typename T>
+struct StepRef {
+    const T *rows;         // 4 values per row
+    const int64_t *count;  // the step number of this step
+    int64_t first;         // step number of row 0
+    int64_t last_row;
+};
+
+// wave-uniform loads through the constant address space: the scalar unit's
+__device__ __forceinline__ float load_uniform(const float *p) {
+    return *(const __attribute__((address_space(4))) float *)p;
+}
+__device__ __forceinline__ double load_uniform(const double *p) {
+    return *(const __attribute__((address_space(4))) double *)p;
+}
+__device__ __forceinline__ int64_t load_uniform(const int64_t *p) {
+    return *(const __attribute__((address_space(4))) int64_t *)p;
+}
+template <class F>
+__device__ __forceinline__ R16<F> load_uniform(const R16<F> *p) {
+    return R16<F>::from_bits(*(const __attribute__((address_space(4))) uint16_t *)p);
+}
+
+template <class Op, typename T>
+struct AtStep : Op {
+    StepRef<T> step;
+    __device__ __forceinline__ void fetch() {
+        int64_t r = load_uniform(step.count) - step.first;
+        r = r < 0 ? 0 : (r > step.last_row ? step.last_row : r);
+        const T *row = step.rows + 4 * r;
+        this->set_bias(load_uniform(row), load_uniform(row + 1), load_uniform(row + 2),
+                       load_uniform(row + 3));
+    }
+};
+template <class Op>
+struct FetchesStep {
+    static constexpr bool value = false;
+};
+template <class Op, typename T>
+struct FetchesStep<AtStep<Op, T>> {
+    static constexpr bool value = true;
+};
+// The op a kernel computes with: the launch's op, with the bias corrections of the current step
+// filled in where the step number lives on the device.
+template <class Op>
+__device__ __forceinline__ Op live_op(const Op &op) {
+    Op live = op;
+    if constexpr (FetchesStep<Op>::value) live.fetch();
+    return live;
+}
+
 // What a staged op sees of its tile: one 128-bit vector per lane of every array.
 template <typename T, class Op, bool NT>
 struct StagedIO {
@@ -341,6 +402,10 @@ constexpr int waves_by_type(int wide, int half, int bfloat) {
 template <typename T>
 struct AdamSteps {
     T b1, b2, c1, c2, eps, eps_root;
+    __device__ __forceinline__ void set_bias(T c1_, T c2_, T, T) {
+        c1 = c1_;
+        c2 = c2_;
+    }
     __device__ __forceinline__ T first(T g, T m) const { return b1 * m + (1 - b1) * g; }
     __device__ __forceinline__ T second(T g, T v) const { return b2 * v + (1 - b2) * g * g; }
     __device__ __forceinline__ T third(T m1, T v1) const {
@@ -628,6 +693,10 @@ struct FusedStep {
     T b1, b2, c1, c2, eps, eps_root, neg_lr, wd;
     int decay;
     bool maximize;
+    __device__ __forceinline__ void set_bias(T c1_, T c2_, T, T) {
+        c1 = c1_;
+        c2 = c2_;
+    }
     // the gradient the moments see
     __device__ __forceinline__ T gradient(T g, T p) const {
         g = maximize ? -g : g;
@@ -880,8 +949,9 @@ template <typename T, class Op, int UNROLL, bool NT>
 __global__ __launch_bounds__(kBlock) void stream_kernel(const Op op, const TensorPtrs<T, Op> tp,
                                                         const size_t n, const size_t num_tiles) {
     const bool aligned = all_aligned16<T, Op>(tp);
+    const Op live = live_op(op);
     for (size_t tile = blockIdx.x; tile < num_tiles; tile += gridDim.x)
-        process_tile<T, Op, UNROLL, NT>(op, tp, n, tile, aligned);
+        process_tile<T, Op, UNROLL, NT>(live, tp, n, tile, aligned);
 }
 
 // The common case without its branches: every pointer 16-byte aligned and only whole tiles,
@@ -891,10 +961,11 @@ template <typename T, class Op, int UNROLL, bool NT, bool STAGED = false>
 __global__ __launch_bounds__(kBlock) void full_tiles_kernel(const Op op,
                                                             const TensorPtrs<T, Op> tp) {
     static_assert(!STAGED || UNROLL == 1, "the staged schedule handles one vector per lane");
+    const Op live = live_op(op);
     if constexpr (STAGED)
-        tile_full_staged<T, Op, NT>(op, tp, (size_t)blockIdx.x * Tile<T, UNROLL>::VECS);
+        tile_full_staged<T, Op, NT>(live, tp, (size_t)blockIdx.x * Tile<T, UNROLL>::VECS);
     else
-        tile_full<T, Op, UNROLL, NT>(op, tp, (size_t)blockIdx.x * Tile<T, UNROLL>::VECS);
+        tile_full<T, Op, UNROLL, NT>(live, tp, (size_t)blockIdx.x * Tile<T, UNROLL>::VECS);
 }
 
 // ---------------------------------------------------------------------------
@@ -945,6 +1016,7 @@ template <typename T, class Op, int UNROLL, bool NT, bool STAGED = false>
 __global__ __launch_bounds__(kBlock) void multi_stream_kernel(const Op op,
                                                               const MultiTable<T, Op> tab) {
     using Table = MultiTable<T, Op>;
+    const Op live = live_op(op);
     for (uint32_t tile = blockIdx.x; tile < tab.total; tile += gridDim.x) {
         uint32_t g = 0;
 #pragma unroll
@@ -961,7 +1033,7 @@ __global__ __launch_bounds__(kBlock) void multi_stream_kernel(const Op op,
 #pragma unroll
         for (int i = 0; i < Op::NPTR; ++i) tp.p[i] = rec.p[i];
         const bool aligned = all_aligned16<T, Op>(tp);
-        process_tile<T, Op, UNROLL, NT, STAGED>(op, tp, (size_t)rec.n, (size_t)(tile - first),
+        process_tile<T, Op, UNROLL, NT, STAGED>(live, tp, (size_t)rec.n, (size_t)(tile - first),
                                                 aligned);
     }
 }
@@ -1054,6 +1126,7 @@ __device__ __forceinline__ PlanRec load_record(const PlanRec *at) {
 
 template <typename T, class Op, int UNROLL, bool NT, bool STAGED = false>
 __global__ __launch_bounds__(kBlock) void plan_stream_kernel(const Op op, const PlanView plan) {
+    const Op live = live_op(op);
     for (uint32_t tile = blockIdx.x; tile < plan.total; tile += gridDim.x) {
         PlanRec rec = load_record(plan.recs + plan.cell[tile >> plan.shift]);
         // a tensor boundary lies between the cell's first tile and this one: walk on (never
@@ -1064,8 +1137,17 @@ __global__ __launch_bounds__(kBlock) void plan_stream_kernel(const Op op, const 
 #pragma unroll
         for (int i = 0; i < Op::NPTR; ++i) tp.p[i] = static_cast<T *>(rec.p[i]);
         const bool aligned = all_aligned16<T, Op>(tp);
-        process_tile<T, Op, UNROLL, NT, STAGED>(op, tp, (size_t)rec.n, (size_t)(tile - rec.first),
+        process_tile<T, Op, UNROLL, NT, STAGED>(live, tp, (size_t)rec.n, (size_t)(tile - rec.first),
                                                 aligned);
+    }
+}
+
+// count <- count + (count != INT64_MAX): the reference's inc_count
+// (/root/reference/torchopt/transform/utils.py:111-126) for a step number that lives on the device.
+__global__ __launch_bounds__(64) void count_advance_kernel(int64_t *count) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        const int64_t c = *count;
+        *count = c + (c != INT64_MAX ? 1 : 0);
     }
 }
 

@@ -674,6 +674,125 @@ py::tuple fusedStepMulti(const py::object &params_o, const py::object &updates_o
     return py::make_tuple(params_o, updates_o, mu_o, nu_o);
 }
 
+// ---- step number on the device ------------------------------------------------------------
+
+// `rows` x 4 tensor on the CPU of element type `dtype`: the bias corrections of step numbers
+// first_count, first_count + 1, ... as the launchers round them.
+Tensor biasRows(const py::object &dtype_o, double b1, double b2, double eps_root,
+                uint64_t first_count, size_t rows) {
+    const at::ScalarType st = torch::python::detail::py_object_to_dtype(dtype_o);
+    Tensor out = at::empty({(int64_t)rows, 4}, at::TensorOptions().dtype(st).device(at::kCPU));
+    check(toa_adam_bias_rows(dtypeCode(out, "adamBiasRows"), b1, b2, eps_root, first_count, rows,
+                             out.data_ptr()),
+          "adamBiasRows");
+    return out;
+}
+
+size_t biasRowsNeeded(double b1, double b2, uint64_t first_count, size_t limit) {
+    return toa_adam_bias_rows_needed(b1, b2, first_count, limit);
+}
+
+// What the device-count entry points need beside the tensors: the table and the step number, on
+// the tensors' device.
+struct DeviceStep {
+    const void *rows;
+    size_t num_rows;
+    const int64_t *count;
+};
+DeviceStep gateStep(const char *name, const Tensor &lead, const Tensor &bias_rows,
+                    const Tensor &count) {
+    TORCH_CHECK(bias_rows.device() == lead.device() && count.device() == lead.device(), name,
+                ": bias_rows and count must live on ", lead.device());
+    TORCH_CHECK(bias_rows.scalar_type() == lead.scalar_type(), name,
+                ": bias_rows must have the tensors' scalar type ", lead.scalar_type());
+    TORCH_CHECK(bias_rows.dim() == 2 && bias_rows.size(1) == 4 && bias_rows.size(0) >= 1 &&
+                    bias_rows.is_contiguous(),
+                name, ": bias_rows must be a contiguous (rows, 4) tensor");
+    TORCH_CHECK(count.scalar_type() == at::kLong && count.numel() == 1, name,
+                ": count must be a one-element int64 tensor");
+    return {bias_rows.data_ptr(), (size_t)bias_rows.size(0), count.data_ptr<int64_t>()};
+}
+
+Tensor countAdvance(const Tensor &count) {
+    if (!count.is_cuda()) throw std::runtime_error("Not implemented");
+    TORCH_CHECK(count.scalar_type() == at::kLong && count.numel() == 1,
+                "adamCountAdvance: count must be a one-element int64 tensor");
+    const OnDeviceOf dev(count);
+    check(toa_adam_count_advance(count.data_ptr<int64_t>(), dev.stream()), "adamCountAdvance");
+    return count;
+}
+
+std::array<Tensor, 3> forwardInplaceDevCount(const Tensor &updates, const Tensor &mu,
+                                             const Tensor &nu, double b1, double b2, double eps,
+                                             double eps_root, const Tensor &bias_rows,
+                                             uint64_t first_count, const Tensor &count) {
+    const char *name = "adamForwardInplaceDevCount";
+    size_t n;
+    const int code = gate(name, updates, {&mu, &nu}, &n);
+    const DeviceStep step = gateStep(name, updates, bias_rows, count);
+    if (n) {
+        requireDense(name, "updates", updates);
+        requireDense(name, "mu", mu);
+        requireDense(name, "nu", nu);
+        TORCH_CHECK(sameLayout(updates, mu) && sameLayout(updates, nu), name,
+                    ": updates, mu and nu must share one memory layout");
+        const OnDeviceOf dev(updates);
+        check(toa_adam_forward_inplace_devcount(code, updates.data_ptr(), mu.data_ptr(),
+                                                nu.data_ptr(), n, b1, b2, eps, eps_root, step.rows,
+                                                first_count, step.num_rows, step.count,
+                                                dev.stream()),
+              name);
+    }
+    return {updates, mu, nu};
+}
+
+py::tuple forwardMultiInplaceDevCount(const py::object &updates_o, const py::object &mu_o,
+                                      const py::object &nu_o, double b1, double b2, double eps,
+                                      double eps_root, const Tensor &bias_rows,
+                                      uint64_t first_count, const Tensor &count) {
+    const char *name = "adamForwardInplaceMultiDevCount";
+    const auto updates = toTensorList(updates_o, "updates");
+    const auto mu = toTensorList(mu_o, "mu");
+    const auto nu = toTensorList(nu_o, "nu");
+    Lists l = gateLists(name, {&updates, &mu, &nu});
+    if (l.num) {
+        const DeviceStep step = gateStep(name, deviceDonor(updates), bias_rows, count);
+        const OnDeviceOf dev(deviceDonor(updates));
+        check(toa_adam_forward_inplace_multi_devcount(
+                  l.code, l.num, l.ptr[0].data(), l.ptr[1].data(), l.ptr[2].data(), l.n.data(), b1,
+                  b2, eps, eps_root, step.rows, first_count, step.num_rows, step.count,
+                  dev.stream()),
+              name);
+    }
+    return py::make_tuple(updates_o, mu_o, nu_o);
+}
+
+py::tuple fusedStepMultiDevCount(const py::object &params_o, const py::object &updates_o,
+                                 const py::object &mu_o, const py::object &nu_o, double b1,
+                                 double b2, double eps, double eps_root, const Tensor &bias_rows,
+                                 uint64_t first_count, const Tensor &count, double lr,
+                                 bool maximize, bool write_updates, double weight_decay,
+                                 bool decoupled) {
+    const char *name = "adamFusedStepMultiDevCount";
+    const auto params = toTensorList(params_o, "params");
+    auto updates = toTensorList(updates_o, "updates");
+    const auto mu = toTensorList(mu_o, "mu");
+    const auto nu = toTensorList(nu_o, "nu");
+    if (!write_updates) updates = asLayoutOfEach(updates, params, name);
+    Lists l = gateLists(name, {&params, &mu, &nu, &updates});
+    if (l.num) {
+        const DeviceStep step = gateStep(name, deviceDonor(params), bias_rows, count);
+        const OnDeviceOf dev(deviceDonor(params));
+        check(toa_adam_fused_step_multi_devcount(
+                  l.code, l.num, l.ptr[0].data(), l.ptr[3].data(), l.ptr[1].data(),
+                  l.ptr[2].data(), l.n.data(), b1, b2, eps, eps_root, step.rows, first_count,
+                  step.num_rows, step.count, lr, weight_decay, (int)decoupled, (int)maximize,
+                  (int)write_updates, dev.stream()),
+              name);
+    }
+    return py::make_tuple(params_o, updates_o, mu_o, nu_o);
+}
+
 }  // namespace
 
 PYBIND11_MODULE(_C, mod) {
@@ -735,5 +854,26 @@ PYBIND11_MODULE(_C, mod) {
     m.def("fused_step_multi_", &fusedStepMulti, "fused_step_ over lists", "params"_a, "updates"_a,
           "mu"_a, "nu"_a, "b1"_a, "b2"_a, "eps"_a, "eps_root"_a, "counts"_a, "lr"_a,
           py::kw_only(), "maximize"_a = false, "write_updates"_a = false,
+          "weight_decay"_a = 0.0, "decoupled"_a = false);
+
+    // the step number on the device: one captured graph serves a whole training loop
+    m.def("bias_rows", &biasRows,
+          "(rows, 4) CPU tensor of bias corrections for steps first_count, first_count + 1, ...",
+          "dtype"_a, "b1"_a, "b2"_a, "eps_root"_a, "first_count"_a, "rows"_a);
+    m.def("bias_rows_needed", &biasRowsNeeded,
+          "rows from first_count on that make a table exact for every later step (0: > limit)",
+          "b1"_a, "b2"_a, "first_count"_a, "limit"_a);
+    m.def("count_advance_", &countAdvance, "count += (count != INT64_MAX), on the device",
+          "count"_a);
+    m.def("forward_devcount_", &forwardInplaceDevCount,
+          "forward_ with the step number read on the device", "updates"_a, "mu"_a, "nu"_a, "b1"_a,
+          "b2"_a, "eps"_a, "eps_root"_a, "bias_rows"_a, "first_count"_a, "count"_a);
+    m.def("forward_multi_devcount_", &forwardMultiInplaceDevCount,
+          "forward_multi_ with the step number read on the device", "updates"_a, "mu"_a, "nu"_a,
+          "b1"_a, "b2"_a, "eps"_a, "eps_root"_a, "bias_rows"_a, "first_count"_a, "count"_a);
+    m.def("fused_step_multi_devcount_", &fusedStepMultiDevCount,
+          "fused_step_multi_ with the step number read on the device", "params"_a, "updates"_a,
+          "mu"_a, "nu"_a, "b1"_a, "b2"_a, "eps"_a, "eps_root"_a, "bias_rows"_a, "first_count"_a,
+          "count"_a, "lr"_a, py::kw_only(), "maximize"_a = false, "write_updates"_a = false,
           "weight_decay"_a = 0.0, "decoupled"_a = false);
 }

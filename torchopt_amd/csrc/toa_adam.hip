@@ -154,6 +154,17 @@ HostScalars host_scalars(double b1, double b2, double eps_root, uint64_t count) 
     return {1 / (1 - pb1), 1 / (1 - pb2), 1 - pb1, 1 / (1 - pb2 + eps_root)};
 }
 
+// The device-side step reference of the *_devcount entry points, checked.
+template <typename T>
+int make_step_ref(const void *bias_rows, uint64_t first_count, size_t rows, const int64_t *count,
+                  StepRef<T> *out) {
+    if (bias_rows == nullptr || count == nullptr) return TOA_ENULL;
+    if (rows == 0 || rows > ((size_t)1 << 40) || first_count > (uint64_t)INT64_MAX) return TOA_ESIZE;
+    *out = StepRef<T>{static_cast<const T *>(bias_rows), count, (int64_t)first_count,
+                      (int64_t)rows - 1};
+    return 0;
+}
+
 template <typename T, class Op>
 int launch_single(const Op &op, T *const (&ptrs)[Op::NPTR], size_t n, void *stream) {
     if (n == 0) return 0;
@@ -351,6 +362,9 @@ int launch_multi(MakeOp make_op, size_t num_tensors,
                  const size_t *n, const uint64_t *counts, uint64_t count_all, void *stream,
                  const PlanArena *arena = nullptr) {
     using Table = MultiTable<T, Op>;
+    // HIP allows 4 KiB of kernel arguments, 256 bytes of them implicit
+    static_assert(sizeof(Op) + sizeof(Table) + 256 <= 4096, "table launch fits its arguments");
+    static_assert(sizeof(Op) + sizeof(PlanView) + 256 <= 4096, "plan launch fits its arguments");
     constexpr size_t tile = Tile<T, kUnroll>::ELEMS;
     if (num_tensors == 0) return 0;
     if (n == nullptr) return TOA_ENULL;
@@ -657,7 +671,7 @@ int backward_all_multi(size_t num, const void *const *dnew_updates,
 
 extern "C" {
 
-int toa_adam_abi_version(void) { return 2; }
+int toa_adam_abi_version(void) { return 3; }
 
 int toa_adam_set_waves_per_cu(int waves) {
     const int prev = waves_override();
@@ -1014,6 +1028,139 @@ int toa_adam_fused_step_multi(int dtype, size_t num_tensors, void *const *params
         };
         return launch_multi<T, FusedStep<T, false>>(make, num_tensors, lists, n, counts,
                                                     count_all, stream);
+    });
+}
+
+// ---- step number on the device ------------------------------------------------------
+
+int toa_adam_bias_rows(int dtype, double b1, double b2, double eps_root, uint64_t first_count,
+                       size_t rows, void *host_out) {
+    if (host_out == nullptr && rows != 0) return TOA_ENULL;
+    TOA_DISPATCH_ALL(dtype, [&] {
+        T *out = static_cast<T *>(host_out);
+        for (size_t r = 0; r < rows; ++r) {
+            const HostScalars s = host_scalars(b1, b2, eps_root, first_count + r);
+            out[4 * r + 0] = (T)s.c1;
+            out[4 * r + 1] = (T)s.c2;
+            out[4 * r + 2] = (T)s.p1;
+            out[4 * r + 3] = (T)s.q2;
+        }
+        return 0;
+    });
+}
+
+size_t toa_adam_bias_rows_needed(double b1, double b2, uint64_t first_count, size_t limit) {
+    // Smallest step number from which 1 - b^count is 1 in double for both decay rates: the rows
+    // of every later step equal that step's.  b^count falls with count, so bisect.
+    auto settled = [&](uint64_t c) {
+        return 1 - std::pow(b1, (double)c) == 1.0 && 1 - std::pow(b2, (double)c) == 1.0;
+    };
+    if (limit == 0) return 0;
+    const uint64_t hi_count = first_count + (limit - 1);
+    if (!settled(hi_count)) return 0;
+    uint64_t lo = first_count, hi = hi_count;  // settled(hi) holds
+    while (lo < hi) {
+        const uint64_t mid = lo + (hi - lo) / 2;
+        if (settled(mid))
+            hi = mid;
+        else
+            lo = mid + 1;
+    }
+    return (size_t)(lo - first_count + 1);
+}
+
+int toa_adam_count_advance(int64_t *count, void *stream) {
+    if (count == nullptr) return TOA_ENULL;
+    hipLaunchKernelGGL(count_advance_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, count);
+    return (int)hipGetLastError();
+}
+
+int toa_adam_forward_inplace_devcount(int dtype, void *updates, void *mu, void *nu, size_t n,
+                                      double b1, double b2, double eps, double eps_root,
+                                      const void *bias_rows, uint64_t first_count, size_t rows,
+                                      const int64_t *count, void *stream) {
+    TOA_DISPATCH_ALL(dtype, [&] {
+        StepRef<T> step;
+        if (const int rc = make_step_ref<T>(bias_rows, first_count, rows, count, &step)) return rc;
+        using Op = AtStep<ForwardInplace<T>, T>;
+        const Op op{{{(T)b1, (T)b2, T(1), T(1), (T)eps, (T)eps_root}}, step};
+        T *const p[3] = {(T *)updates, (T *)mu, (T *)nu};
+        return launch_single<T>(op, p, n, stream);
+    });
+}
+
+int toa_adam_forward_inplace_multi_devcount(int dtype, size_t num_tensors, void *const *updates,
+                                            void *const *mu, void *const *nu, const size_t *n,
+                                            double b1, double b2, double eps, double eps_root,
+                                            const void *bias_rows, uint64_t first_count,
+                                            size_t rows, const int64_t *count, void *stream) {
+    TOA_DISPATCH_ALL(dtype, [&] {
+        StepRef<T> step;
+        if (const int rc = make_step_ref<T>(bias_rows, first_count, rows, count, &step)) return rc;
+        using Op = AtStep<ForwardInplace<T>, T>;
+        const void *const *const lists[3] = {CPP(updates), CPP(mu), CPP(nu)};
+        auto make = [&](uint64_t) {
+            return Op{{{(T)b1, (T)b2, T(1), T(1), (T)eps, (T)eps_root}}, step};
+        };
+        return launch_multi<T, Op>(make, num_tensors, lists, n, nullptr, 0, stream);
+    });
+}
+
+int toa_adam_fused_step_devcount(int dtype, void *params, void *updates, void *mu, void *nu,
+                                 size_t n, double b1, double b2, double eps, double eps_root,
+                                 const void *bias_rows, uint64_t first_count, size_t rows,
+                                 const int64_t *count, double lr, double weight_decay,
+                                 int decoupled, int maximize, int write_updates, void *stream) {
+    const int decay = weight_decay == 0.0 ? kNoDecay
+                                          : (decoupled ? kDecayIntoUpdate : kDecayIntoGradient);
+    TOA_DISPATCH(dtype, [&] {
+        StepRef<T> step;
+        if (const int rc = make_step_ref<T>(bias_rows, first_count, rows, count, &step)) return rc;
+        T *const p[4] = {(T *)updates, (T *)mu, (T *)nu, (T *)params};
+        if (write_updates) {
+            const AtStep<FusedStep<T, true>, T> op{
+                {(T)b1, (T)b2, T(1), T(1), (T)eps, (T)eps_root, (T)(-lr), (T)weight_decay, decay,
+                 maximize != 0},
+                step};
+            return launch_single<T>(op, p, n, stream);
+        }
+        const AtStep<FusedStep<T, false>, T> op{
+            {(T)b1, (T)b2, T(1), T(1), (T)eps, (T)eps_root, (T)(-lr), (T)weight_decay, decay,
+             maximize != 0},
+            step};
+        return launch_single<T>(op, p, n, stream);
+    });
+}
+
+int toa_adam_fused_step_multi_devcount(int dtype, size_t num_tensors, void *const *params,
+                                       void *const *updates, void *const *mu, void *const *nu,
+                                       const size_t *n, double b1, double b2, double eps,
+                                       double eps_root, const void *bias_rows,
+                                       uint64_t first_count, size_t rows, const int64_t *count,
+                                       double lr, double weight_decay, int decoupled,
+                                       int maximize, int write_updates, void *stream) {
+    const int decay = weight_decay == 0.0 ? kNoDecay
+                                          : (decoupled ? kDecayIntoUpdate : kDecayIntoGradient);
+    TOA_DISPATCH(dtype, [&] {
+        StepRef<T> step;
+        if (const int rc = make_step_ref<T>(bias_rows, first_count, rows, count, &step)) return rc;
+        const void *const *const lists[4] = {CPP(updates), CPP(mu), CPP(nu), CPP(params)};
+        if (write_updates) {
+            using Op = AtStep<FusedStep<T, true>, T>;
+            auto make = [&](uint64_t) {
+                return Op{{(T)b1, (T)b2, T(1), T(1), (T)eps, (T)eps_root, (T)(-lr),
+                           (T)weight_decay, decay, maximize != 0},
+                          step};
+            };
+            return launch_multi<T, Op>(make, num_tensors, lists, n, nullptr, 0, stream);
+        }
+        using Op = AtStep<FusedStep<T, false>, T>;
+        auto make = [&](uint64_t) {
+            return Op{{(T)b1, (T)b2, T(1), T(1), (T)eps, (T)eps_root, (T)(-lr), (T)weight_decay,
+                       decay, maximize != 0},
+                      step};
+        };
+        return launch_multi<T, Op>(make, num_tensors, lists, n, nullptr, 0, stream);
     });
 }
 

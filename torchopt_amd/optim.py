@@ -21,6 +21,15 @@ place); the differences are mechanical:
 
 State per parameter group is a `ScaleByAdamState(mu, nu, count)` of tuples, as the
 transformation's own state, so it can be handed to `scale_by_accelerated_adam(...).update`.
+
+`capturable=True` (the name `torch.optim.Adam` uses) keeps the step number where the reference
+keeps it, in a device tensor (/root/reference/torchopt/transform/scale_by_adam.py:401-414), and
+nowhere else: `step()` advances it with a one-thread kernel and the fused step reads it when it
+starts, picking its bias corrections from a table the host filled once (in double with libm's
+`pow`, as the reference's launchers compute them, so results stay bit-identical).  One HIP graph
+captured around `step()` then serves the whole training loop: every replay is the next step.
+Without it a captured `step()` would replay the step number it was captured with, so `step()`
+refuses to run under capture.
 """
 
 from __future__ import annotations
@@ -56,6 +65,7 @@ class FusedAdam:
         eps_root: float = 0.0,
         maximize: bool = False,
         use_accelerated_op: bool = True,
+        capturable: bool = False,
     ) -> None:
         # `use_accelerated_op` is accepted so that the reference's constructor calls carry over
         # (optim/adam.py:56-65); the fused operator is the only path here, and False warns
@@ -73,6 +83,18 @@ class FusedAdam:
             raise ValueError(f'Invalid weight_decay value: {weight_decay}')
         self.lr, self.b1, self.b2, self.eps, self.weight_decay = lr, b1, b2, eps, weight_decay
         self.eps_root, self.maximize = eps_root, maximize
+        self.capturable = bool(capturable)
+        if self.capturable:
+            if callable(lr):
+                raise ValueError('capturable=True needs a constant learning rate: a schedule is '
+                                 'evaluated on the host, which a captured graph would freeze')
+            rows = adam_op.bias_rows_needed(b1, b2, 1, _MAX_BIAS_ROWS)
+            if rows == 0:
+                raise ValueError(
+                    f'capturable=True: the bias corrections of betas={betas} take more than '
+                    f'{_MAX_BIAS_ROWS} steps to settle, too many to tabulate')
+            self._bias_rows_needed = rows
+        self._bias_tables: dict[tuple, torch.Tensor] = {}  # (device, dtype) -> (rows, 4) table
         self.param_groups: list[tuple[torch.Tensor, ...]] = []
         self.state_groups: list[ScaleByAdamState | None] = []
         self._kinds: list[list[tuple]] = []       # (device, dtype) per parameter
@@ -119,11 +141,32 @@ class FusedAdam:
         self._steps = [None if s is None else [_host_value(c) for c in s.count]
                        for s in self.state_groups]
         self._stale = [False] * len(self.state_groups)
+        if self.capturable:
+            # the leaves of one device step together from one shared count tensor
+            for i, s in enumerate(self.state_groups):
+                if s is None:
+                    continue
+                shared: dict[torch.device, torch.Tensor] = {}
+                for c, v in zip(s.count, self._steps[i]):
+                    if c.device not in shared:
+                        shared[c.device] = torch.full((), v, dtype=torch.int64, device=c.device)
+                    elif int(shared[c.device]) != v:
+                        raise ValueError('capturable=True needs the parameters of a group on one '
+                                         'device to share one step count')
+                self.state_groups[i] = s._replace(count=tuple(shared[c.device] for c in s.count))
 
     def _init_state(self, i: int) -> ScaleByAdamState:
         group = self.param_groups[i]
-        count = tuple(_remember(torch.zeros(1, dtype=torch.int64, device=p.device).squeeze_(), 0)
-                      for p in group)
+        if self.capturable:
+            # one count tensor per device, shared by that device's leaves: they step together
+            shared = {}
+            for p in group:
+                if p.device not in shared:
+                    shared[p.device] = torch.zeros(1, dtype=torch.int64, device=p.device).squeeze_()
+            count = tuple(shared[p.device] for p in group)
+        else:
+            count = tuple(_remember(torch.zeros(1, dtype=torch.int64, device=p.device).squeeze_(),
+                                    0) for p in group)
         self._steps[i] = [0] * len(group)
         self._stale[i] = False
         return ScaleByAdamState(mu=tuple(torch.zeros_like(p) for p in group),
@@ -133,7 +176,7 @@ class FusedAdam:
         """Bring the 0-dim device count tensors of group `i` up to the host's step numbers.
         `step()` advances only the host numbers; the tensors are rebuilt (one upload per
         device) when somebody asks for the state."""
-        if not self._stale[i]:
+        if not self._stale[i] or self.capturable:
             return
         state, steps = self.state_groups[i], self._steps[i]
         by_device: dict[torch.device, list[int]] = {}
@@ -147,12 +190,79 @@ class FusedAdam:
         self.state_groups[i] = state._replace(count=tuple(counts))
         self._stale[i] = False
 
+    def _bias_table(self, device: torch.device, dtype: torch.dtype) -> torch.Tensor:
+        key = (device, dtype)
+        if key not in self._bias_tables:
+            host = adam_op.bias_rows(dtype, self.b1, self.b2, self.eps_root, 1,
+                                     self._bias_rows_needed)
+            self._bias_tables[key] = host.to(device)
+        return self._bias_tables[key]
+
+    def _step_on_device(self) -> None:
+        """`step()` with the step numbers on the device: nothing here depends on their values,
+        so a HIP graph captured around it replays as the following steps."""
+        capturing = torch.cuda.is_current_stream_capturing()
+        for i, group in enumerate(self.param_groups):
+            if self.state_groups[i] is None:
+                if capturing:
+                    raise RuntimeError('FusedAdam: take one step (or call init_state()) before '
+                                       'capturing, so that the state exists outside the graph')
+                self.state_groups[i] = self._init_state(i)
+            state = self.state_groups[i]
+            grads = [p.grad for p in group]
+            if all(g is None for g in grads):
+                continue
+            if any(g is None for g in grads):
+                raise RuntimeError('FusedAdam(capturable=True): every parameter of a group must '
+                                   'have a gradient at every step (they share one step count)')
+            buckets: dict[tuple, list[int]] = {}
+            for k in range(len(group)):
+                buckets.setdefault((self._kinds[i][k], self._decays[i][k]), []).append(k)
+            tables = {kind: self._bias_table(*kind) for kind, _ in buckets}  # before any launch
+            advanced = set()
+            for c in state.count:
+                if id(c) not in advanced:
+                    advanced.add(id(c))
+                    adam_op.count_advance_(c)
+            for (kind, decays), ks in buckets.items():
+                whole = len(ks) == len(group)
+                adam_op.fused_step_multi_devcount_(
+                    list(group) if whole else [group[k] for k in ks],
+                    grads if whole else [grads[k] for k in ks],
+                    list(state.mu) if whole else [state.mu[k] for k in ks],
+                    list(state.nu) if whole else [state.nu[k] for k in ks],
+                    self.b1, self.b2, self.eps, self.eps_root, tables[kind], 1,
+                    state.count[ks[0]], self.lr, maximize=self.maximize, write_updates=False,
+                    weight_decay=self.weight_decay if decays else 0.0,
+                    decoupled=self._decoupled)
+            self._steps[i] = None  # the device holds the step numbers now
+
+    def init_state(self) -> None:
+        """Create the moments and step counts now (they are otherwise created by the first
+        `step()`), e.g. before capturing `step()` in a graph."""
+        for i in range(len(self.param_groups)):
+            if self.state_groups[i] is None:
+                self.state_groups[i] = self._init_state(i)
+                if self.capturable:
+                    for p in self.param_groups[i]:
+                        self._bias_table(p.device, p.dtype)
+
     @torch.no_grad()
     def step(self, closure: Callable[[], torch.Tensor] | None = None):
         loss = None
         if closure is not None:
             with torch.enable_grad():
                 loss = closure()
+        if self.capturable:
+            self._step_on_device()
+            return loss
+        if torch.cuda.is_available() and torch.cuda.is_current_stream_capturing():
+            raise RuntimeError(
+                'FusedAdam.step() under stream capture would bake the current step number (and '
+                'its bias corrections) into the graph, and every replay would repeat that step. '
+                'Construct the optimizer with capturable=True to keep the step number on the '
+                'device, or call torchopt_amd._C.adam_op.fused_step_multi_ yourself with the '
+                'count you mean to freeze.')
         scheduled = callable(self.lr)
         for i, group in enumerate(self.param_groups):
             if self.state_groups[i] is None:
@@ -196,12 +306,19 @@ class FusedAdamW(FusedAdam):
 
     def __init__(self, params, lr: float = 1e-3, betas=(0.9, 0.999), eps: float = 1e-8,
                  weight_decay: float = 1e-2, *, eps_root: float = 0.0, mask=None,
-                 maximize: bool = False, use_accelerated_op: bool = True) -> None:
+                 maximize: bool = False, use_accelerated_op: bool = True,
+                 capturable: bool = False) -> None:
         # `mask`: a sequence of booleans, one per parameter, or a callable that makes one from
         # the parameters; False exempts a parameter from the decay (optim/adamw.py:60-63)
         self._mask = mask
         super().__init__(params, lr, betas, eps, weight_decay, eps_root=eps_root,
-                         maximize=maximize, use_accelerated_op=use_accelerated_op)
+                         maximize=maximize, use_accelerated_op=use_accelerated_op,
+                         capturable=capturable)
+
+
+# Most rows a bias-correction table may have (16 bytes per float32 row): enough for b2 up to
+# 0.99999, whose corrections settle after 3.7 million steps.
+_MAX_BIAS_ROWS = 1 << 22
 
 
 # the reference's class names (torchopt.Adam / torchopt.AdamW)

@@ -210,6 +210,15 @@ def _scale_by_accelerated_adam(
                                 count=rebuild(count, params, spec))
 
     def update_fn(updates, state, *, params=None, inplace=True):  # noqa: ARG001
+        if torch.cuda.is_available() and torch.cuda.is_current_stream_capturing():
+            # The step numbers advance on the host here (a mirror of the count tensors), and the
+            # launches carry their bias corrections as arguments: a captured update would replay
+            # one step number for ever.  (The reference fails here too: converting its device
+            # count to size_t reads the device, which capture forbids.)
+            raise RuntimeError(
+                'scale_by_accelerated_adam.update() cannot be captured in a HIP graph: the step '
+                'count is read on the host.  Use torchopt_amd.FusedAdam(..., capturable=True), '
+                'or call the torchopt_amd._C.adam_op functions with the count you mean to freeze.')
         g_leaves, g_spec = flatten(updates)
         mu_leaves, mu_spec = flatten(state.mu)
         nu_leaves, nu_spec = flatten(state.nu)
