@@ -29,6 +29,9 @@ except ImportError as exc:  # no fallback module: the op is the compiled extensi
         f'imported ({exc}); build it with `python torchopt_amd/build.py`. There is no '
         'pure-Python or CPU fallback.') from exc
 
+# the same seven functions, visible to torch.compile while it traces (see library.py)
+from torchopt_amd.accelerated_op.library import dispatch  # noqa: E402
+
 
 class AdamOp:
     """Fused Adam scaling of one leaf: moments update plus bias-corrected step direction."""
@@ -40,12 +43,12 @@ class AdamOp:
         def forward(ctx: Any, updates: torch.Tensor, mu: torch.Tensor, b1: float) -> torch.Tensor:
             ctx.save_for_backward(updates, mu)
             ctx.b1 = b1
-            return adam_op.forward_mu(updates, mu, b1)
+            return dispatch.forward_mu(updates, mu, b1)
 
         @staticmethod
         def backward(ctx: Any, dmu: torch.Tensor):
             updates, mu = ctx.saved_tensors
-            dupdates, dmu_in = adam_op.backward_mu(dmu, updates, mu, ctx.b1)
+            dupdates, dmu_in = dispatch.backward_mu(dmu, updates, mu, ctx.b1)
             return dupdates, dmu_in, None
 
     class NuOp(torch.autograd.Function):
@@ -55,12 +58,12 @@ class AdamOp:
         def forward(ctx: Any, updates: torch.Tensor, nu: torch.Tensor, b2: float) -> torch.Tensor:
             ctx.save_for_backward(updates, nu)
             ctx.b2 = b2
-            return adam_op.forward_nu(updates, nu, b2)
+            return dispatch.forward_nu(updates, nu, b2)
 
         @staticmethod
         def backward(ctx: Any, dnu: torch.Tensor):
             updates, nu = ctx.saved_tensors
-            dupdates, dnu_in = adam_op.backward_nu(dnu, updates, nu, ctx.b2)
+            dupdates, dnu_in = dispatch.backward_nu(dnu, updates, nu, ctx.b2)
             return dupdates, dnu_in, None
 
     class UpdatesOp(torch.autograd.Function):
@@ -70,7 +73,7 @@ class AdamOp:
         @staticmethod
         def forward(ctx: Any, new_mu: torch.Tensor, new_nu: torch.Tensor, hyper: tuple):
             b1, b2, eps, eps_root, count = hyper
-            new_updates = adam_op.forward_updates(new_mu, new_nu, b1, b2, eps, eps_root, count)
+            new_updates = dispatch.forward_updates(new_mu, new_nu, b1, b2, eps, eps_root, count)
             ctx.save_for_backward(new_updates, new_mu, new_nu)
             ctx.hyper = hyper
             return new_updates
@@ -79,7 +82,7 @@ class AdamOp:
         def backward(ctx: Any, dupdates: torch.Tensor):
             new_updates, new_mu, new_nu = ctx.saved_tensors
             b1, b2, _eps, eps_root, count = ctx.hyper
-            dnew_mu, dnew_nu = adam_op.backward_updates(
+            dnew_mu, dnew_nu = dispatch.backward_updates(
                 dupdates, new_updates, new_mu, new_nu, b1, b2, eps_root, count)
             return dnew_mu, dnew_nu, None
 
@@ -103,7 +106,7 @@ class AdamOp:
             return mu, nu, None
         if self.inplace:
             # forward_ hands back [updates, mu, nu]; callers want (mu, nu, updates)
-            new_updates, new_mu, new_nu = adam_op.forward_(
+            new_updates, new_mu, new_nu = dispatch.forward_(
                 updates, mu, nu, self.b1, self.b2, self.eps, self.eps_root, count)
             return new_mu, new_nu, new_updates
         new_mu = self.MuOp.apply(updates, mu, self.b1)
