@@ -33,6 +33,11 @@ import os
 import sys
 import time
 
+# Thread placement of the CPU baseline leg (read by the OpenMP runtime when it starts, so set
+# before anything loads it); values already in the environment win and are what the line reports.
+os.environ.setdefault('OMP_PROC_BIND', 'close')
+os.environ.setdefault('OMP_PLACES', 'cores')
+
 REPO = os.path.dirname(os.path.abspath(__file__))
 if REPO not in sys.path:
     sys.path.insert(0, REPO)
@@ -46,10 +51,15 @@ BYTES_PER_ELEM = {  # op -> number of arrays streamed (multiply by the element s
 }
 
 # HBM bytes per step as counted by rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE in separate runs,
-# each scaled by what the same counter reads for a plain 1 GiB copy: x1.99996 and x1.0); the
-# commands and raw readings are in profiles/*pmc_traffic*.md.  Not measured live: a counter run
-# serialises the kernels, so it cannot share a process with the timed region.
-MEASURED_TRAFFIC_BYTES = {2: 6442431962, 4: 8516628944}
+# each scaled by what the same counter reads for a plain 1 GiB copy); the commands and raw
+# readings are in the profile named beside each figure.  RECORDED there, not measured live: a
+# counter run serialises the kernels, so it cannot share a process with the timed region.  The
+# figures belong to the kernels as they were when the profile was taken; re-record them whenever
+# adam_kernels.hpp or the launch shape changes.
+RECORDED_TRAFFIC = {
+    2: (6442431962, 'profiles/forward_inplace_f32_config2_pmc_traffic.md'),
+    4: (8516628944, 'profiles/forward_inplace_multi_f32_config4_kernel_trace_and_traffic.md'),
+}
 
 B1, B2, EPS = 0.9, 0.999, 1e-8
 
@@ -117,15 +127,44 @@ ESIZE = {'f32': 4, 'f64': 8, 'f16': 2, 'bf16': 2}
 # ----------------------------------------------------------------------------- GPU side
 
 
-def make_state(torch, n, dtype, seed):
-    """updates ~ N(0,1), mu ~ 0.1 N(0,1), nu ~ |0.01 N(0,1)|, generated on the GPU."""
-    g = torch.Generator(device='cuda')
-    g.manual_seed(seed)
-    wide = torch.float32 if dtype in (torch.float16, torch.bfloat16) else dtype
-    u = torch.randn(n, device='cuda', dtype=wide, generator=g).to(dtype)
-    mu = torch.randn(n, device='cuda', dtype=wide, generator=g).mul_(0.1).to(dtype)
-    nu = torch.randn(n, device='cuda', dtype=wide, generator=g).mul_(0.01).abs_().to(dtype)
-    return u, mu, nu
+_HOST = {}  # (config, tensor index) -> the seeded host arrays, shared by the GPU and CPU legs
+
+
+def host_state(cfg_id, index, n, tag, extra=0):
+    """The seeded host arrays of one tensor, as torch CPU tensors: updates ~ N(0,1),
+    mu = 0.1 N(0,1), nu = |0.01 N(0,1)| and `extra` more N(0,1) arrays, drawn in that order from
+    torch's CPU generator with seed 1000 * config + tensor index.  float64 for 'f64', float32
+    otherwise; the 16-bit types are rounded from the float32 draws."""
+    import torch
+
+    key = (cfg_id, index, n, tag, extra)
+    if key not in _HOST:
+        g = torch.Generator(device='cpu')
+        g.manual_seed(1000 * cfg_id + index)
+        wide = torch.float64 if tag == 'f64' else torch.float32
+        arrays = [torch.randn(n, generator=g, dtype=wide),
+                  torch.randn(n, generator=g, dtype=wide).mul_(0.1),
+                  torch.randn(n, generator=g, dtype=wide).mul_(0.01).abs_()]
+        arrays += [torch.randn(n, generator=g, dtype=wide) for _ in range(extra)]
+        narrow = {'f16': torch.float16, 'bf16': torch.bfloat16}.get(tag)
+        if narrow is not None:
+            arrays = [a.to(narrow) for a in arrays]
+        _HOST[key] = arrays
+    return _HOST[key]
+
+
+def preheat(torch, lib, stream, launches=150):
+    """GPU clocks ramp for the first ~15 ms of sustained load in a cold process (the state was
+    just generated on the host and uploaded, so the GPU has been idle): stream through scratch
+    arrays -- never the benchmark's own state -- for ~40 ms before the warm-up steps."""
+    n = 1 << 26
+    scratch = [torch.rand(n, device='cuda') for _ in range(3)]
+    p = [t.data_ptr() for t in scratch]
+    for _ in range(launches):
+        lib.toa_adam_forward_inplace(0, p[0], p[1], p[2], n, B1, B2, EPS, 0.0, 7,
+                                     stream.cuda_stream)
+    torch.cuda.synchronize()
+    return launches
 
 
 def python_level_differentiable_step(torch, shapes, eps_root, count, wall_ms):
@@ -160,27 +199,36 @@ def python_level_differentiable_step(torch, shapes, eps_root, count, wall_ms):
             'python_per_leaf_tensor_expressions_ms': round(wall_ms(per_leaf_expressions) - base, 5)}
 
 
-def time_backward_ops(torch, lib, code, dtype, n, esize, eps_root, count, stream, reps=20):
+def time_backward_ops(torch, lib, cfg_id, code, dtype, tag, n, esize, eps_root, count, stream,
+                      reps=20):
     """backward_mu, backward_nu, backward_updates and the one-pass backward_all on flat arrays of
-    n elements: ms per launch and achieved GB/s (algorithmic bytes: 3, 4, 5 and 9 arrays)."""
-    g = torch.Generator(device='cuda')
-    g.manual_seed(77)
-    arrays = [torch.randn(n, device='cuda', dtype=dtype, generator=g) for _ in range(9)]
-    arrays[2].mul_(0.1)
-    p = [a.data_ptr() for a in arrays]
+    n elements: ms per launch and achieved GB/s (algorithmic bytes: 3, 4, 5 and 9 arrays).  The
+    inputs are what a differentiable step produces from the configuration's seeded state
+    (updates, new_mu, new_updates) and three seeded N(0,1) arrays as incoming gradients."""
+    g, mu, nu, d_mu, d_nu, d_u = (a.cuda() for a in host_state(cfg_id, 0, n, tag, extra=3))
+    new_mu, new_nu, new_u = (torch.empty_like(g) for _ in range(3))
     s = stream.cuda_stream
-    # slots: 0 updates / dupdates, 1 new_updates, 2 new_mu, 3 dmu, 4 dnu, 5..8 outputs
+    rc = lib.toa_adam_forward_all(code, g.data_ptr(), mu.data_ptr(), nu.data_ptr(), n, B1, B2, EPS,
+                                  eps_root, count, new_mu.data_ptr(), new_nu.data_ptr(),
+                                  new_u.data_ptr(), s)
+    if rc:
+        raise RuntimeError(f'forward_all: {lib.toa_adam_error_string(rc).decode()}')
+    del mu, nu, new_nu
+    out = [torch.empty_like(g) for _ in range(3)]
+    o = [t.data_ptr() for t in out]
     ops = {
-        'backward_mu': (3, lambda: lib.toa_adam_backward_mu(code, p[3], n, B1, p[5], p[6], s)),
-        'backward_nu': (4, lambda: lib.toa_adam_backward_nu(code, p[4], p[0], n, B2, p[5], p[6],
-                                                            s)),
+        'backward_mu': (3, lambda: lib.toa_adam_backward_mu(code, d_mu.data_ptr(), n, B1, o[0],
+                                                            o[1], s)),
+        'backward_nu': (4, lambda: lib.toa_adam_backward_nu(code, d_nu.data_ptr(), g.data_ptr(), n,
+                                                            B2, o[0], o[1], s)),
         'backward_updates': (5, lambda: lib.toa_adam_backward_updates(
-            code, p[0], p[1], p[2], n, B1, B2, eps_root, count, p[5], p[6], s)),
+            code, d_u.data_ptr(), new_u.data_ptr(), new_mu.data_ptr(), n, B1, B2, eps_root, count,
+            o[0], o[1], s)),
         'backward_all': (9, lambda: lib.toa_adam_backward_all(
-            code, p[0], p[1], p[2], p[8], p[3], p[4], n, B1, B2, eps_root, count, p[5], p[6],
-            p[7], s)),
+            code, d_u.data_ptr(), new_u.data_ptr(), new_mu.data_ptr(), g.data_ptr(),
+            d_mu.data_ptr(), d_nu.data_ptr(), n, B1, B2, eps_root, count, o[0], o[1], o[2], s)),
     }
-    out = {}
+    res = {}
     for name, (streams, fn) in ops.items():
         for _ in range(5):
             rc = fn()
@@ -193,8 +241,8 @@ def time_backward_ops(torch, lib, code, dtype, n, esize, eps_root, count, stream
         e1.record(stream)
         torch.cuda.synchronize()
         ms = e0.elapsed_time(e1) / reps
-        out[name] = {'ms': round(ms, 5), 'GB/s': round(streams * esize * n / ms / 1e6, 1)}
-    return out
+        res[name] = {'ms': round(ms, 5), 'GB/s': round(streams * esize * n / ms / 1e6, 1)}
+    return res
 
 
 def run_gpu(cfg_id, steps, warmup):
@@ -222,18 +270,14 @@ def run_gpu(cfg_id, steps, warmup):
 
         sizes = [numel(s) for s in cfg['shapes']]
         total, num = sum(sizes), len(sizes)
-        g = torch.Generator(device='cuda')
-        g.manual_seed(1000 * cfg_id)
-
-        def fresh():
-            return [torch.randn(n, device='cuda', dtype=dtype, generator=g) for n in sizes]
+        host = [host_state(cfg_id, k, n, cfg['dtype'], extra=3) for k, n in enumerate(sizes)]
 
         def arr(ts):
             return (ctypes.c_void_p * num)(*[t.data_ptr() for t in ts])
 
-        ups, mus, nus = fresh(), [t.mul_(0.1) for t in fresh()], [t.mul_(0.01).abs_() for t in fresh()]
-        d_u, d_m, d_v = fresh(), fresh(), fresh()
-        outs = [fresh() for _ in range(9)]  # new_mu, new_nu, new_u, 2 x 3 backward outputs
+        ups, mus, nus, d_m, d_v, d_u = ([h[j].cuda() for h in host] for j in range(6))
+        # new_mu, new_nu, new_u, 2 x 3 backward outputs
+        outs = [[torch.empty(n, device='cuda', dtype=dtype) for n in sizes] for _ in range(9)]
         keep = (ups, mus, nus, d_u, d_m, d_v, outs)  # noqa: F841  (owns the device memory)
         a_up, a_mu, a_nu, a_du, a_dm, a_dv = (arr(x) for x in (ups, mus, nus, d_u, d_m, d_v))
         o = [arr(x) for x in outs]
@@ -304,16 +348,12 @@ def run_gpu(cfg_id, steps, warmup):
         # tree, then mu for every leaf, then nu for every leaf (init_fn maps zeros_like over
         # the tree once per moment, /root/reference/torchopt/transform/scale_by_adam.py:401-414),
         # so the three arrays of one leaf lie far apart.
-        gens = []
-        for k in range(len(sizes)):
-            g = torch.Generator(device='cuda')
-            g.manual_seed(1000 * cfg_id + k)
-            gens.append(g)
-        us = [torch.randn(n, device='cuda', dtype=dtype, generator=g) for n, g in zip(sizes, gens)]
-        ms = [torch.randn(n, device='cuda', dtype=dtype, generator=g).mul_(0.1)
-              for n, g in zip(sizes, gens)]
-        vs = [torch.randn(n, device='cuda', dtype=dtype, generator=g).mul_(0.01).abs_()
-              for n, g in zip(sizes, gens)]
+        extra_arrays = 1 if cfg.get('fused_step') else 0
+        host = [host_state(cfg_id, k, n, cfg['dtype'], extra=extra_arrays)
+                for k, n in enumerate(sizes)]
+        us = [h[0].cuda() for h in host]
+        ms = [h[1].cuda() for h in host]
+        vs = [h[2].cuda() for h in host]
         tensors = list(zip(us, ms, vs))
         num = len(sizes)
         pu = (ctypes.c_void_p * num)(*[t[0].data_ptr() for t in tensors])
@@ -328,8 +368,7 @@ def run_gpu(cfg_id, steps, warmup):
                 raise RuntimeError(lib.toa_adam_error_string(rc).decode())
         extra = {'tensors': num}
         if cfg.get('fused_step'):
-            ps = [torch.randn(n, device='cuda', dtype=dtype, generator=g)
-                  for n, g in zip(sizes, gens)]
+            ps = [h[3].cuda() for h in host]
             pp = (ctypes.c_void_p * num)(*[t.data_ptr() for t in ps])
             lr = 1e-3
 
@@ -357,7 +396,7 @@ def run_gpu(cfg_id, steps, warmup):
                          three_pass_chain_bytes_per_element=11 * esize)
     else:
         total = cfg['n']
-        u, mu, nu = make_state(torch, total, dtype, 1000 * cfg_id)
+        u, mu, nu = (a.cuda() for a in host_state(cfg_id, 0, total, cfg['dtype']))
         pu, pm, pv = u.data_ptr(), mu.data_ptr(), nu.data_ptr()
 
         extra = {}
@@ -388,8 +427,9 @@ def run_gpu(cfg_id, steps, warmup):
                 if rc:
                     raise RuntimeError(lib.toa_adam_error_string(rc).decode())
         if cfg.get('backward'):
-            extra['backward_ops'] = time_backward_ops(torch, lib, code, dtype, total, esize,
-                                                      eps_root, count, stream)
+            extra['backward_ops'] = time_backward_ops(torch, lib, cfg_id, code, dtype,
+                                                      cfg['dtype'], total, esize, eps_root, count,
+                                                      stream)
         if alg_small(total * esize):
             # The timed loop below re-runs on state that stays in the 256 MB Infinity Cache; a
             # real optimizer step finds its state in HBM.  Time single launches after sweeping
@@ -407,6 +447,7 @@ def run_gpu(cfg_id, steps, warmup):
             del sweep
             extra['cold_cache_ms_per_launch'] = round(sorted(cold)[len(cold) // 2], 5)
 
+    extra['preheat_launches_on_scratch_arrays'] = preheat(torch, lib, stream)
     for _ in range(warmup):
         step()
     ev0 = torch.cuda.Event(enable_timing=True)
@@ -439,7 +480,7 @@ def run_gpu(cfg_id, steps, warmup):
     kern_ms = ev0.elapsed_time(ev1) / steps  # stream time per launch (launches are back to back)
     alg_bytes = bytes_per_elem * total
     achieved = alg_bytes / (kern_ms * 1e-3) / 1e9
-    traffic = MEASURED_TRAFFIC_BYTES.get(cfg_id)
+    traffic, traffic_source = RECORDED_TRAFFIC.get(cfg_id, (None, None))
     return {
         'elements': total,
         'ms_per_step': wall_ms,
@@ -447,6 +488,8 @@ def run_gpu(cfg_id, steps, warmup):
         'roofline': {
             'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
             'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': traffic,
+            'traffic_source': (f'recorded in {traffic_source} (rocprofv3 --pmc), not measured in '
+                               'this run' if traffic_source else None),
             'kernel_ms': round(kern_ms, 5), 'algorithmic_bytes_per_launch': alg_bytes,
             'bytes_per_element': bytes_per_elem, **spread,
         },
@@ -530,102 +573,300 @@ def run_ceiling(array_bytes=1 << 30, reps=20):
 # ----------------------------------------------------------------------------- CPU baseline
 
 
+def host_cores():
+    """The CPUs this process may run on, cut to the box's CPU share (OMP_NUM_THREADS, 16 where it
+    is unset) -- not every core the machine shows.  The reference's op asks the OpenMP runtime
+    for the number of processors, which is the size of the affinity mask the runtime saw when it
+    loaded, so `main()` calls this before anything imports torch."""
+    global _HOST_CORES
+    if _HOST_CORES is None:  # once: an OpenMP runtime with OMP_PROC_BIND set pins this thread later
+        share = int(os.environ.get('OMP_NUM_THREADS', '16') or 16)
+        try:
+            avail = sorted(os.sched_getaffinity(0))
+            if len(avail) > share:
+                os.sched_setaffinity(0, set(avail[:share]))
+                avail = avail[:share]
+            _HOST_CORES = max(1, len(avail))
+        except (AttributeError, OSError):
+            _HOST_CORES = max(1, min(share, os.cpu_count() or 1))
+    return _HOST_CORES
+
+
+_HOST_CORES = None
+
+
+CPU_SAMPLE_ELEMS = 1 << 26  # most elements the CPU leg works on (3 x 256 MiB of float32 state)
+
+
+def cpu_model():
+    try:
+        with open('/proc/cpuinfo') as f:
+            for line in f:
+                if line.startswith('model name'):
+                    return line.split(':', 1)[1].strip()
+    except OSError:
+        pass
+    return 'unknown'
+
+
+class CpuOps:
+    """The seven CPU ops on torch CPU tensors: the reference's own compiled CPU op where
+    oracle/_ref holds it (kind 'reference'), this repository's C restatement of it otherwise
+    (kind 'port').  Only this leg of the benchmark touches `oracle/`."""
+
+    def __init__(self):
+        from oracle import adam_oracle
+
+        self.port = adam_oracle
+        self.ref = None
+        try:
+            self.ref = adam_oracle.load_reference()
+        except Exception as exc:  # noqa: BLE001
+            print(f'[bench] compiled reference not usable ({exc}); timing the C port',
+                  file=sys.stderr)
+        self.kind = 'reference' if self.ref is not None else 'port'
+
+    def _np(self, t):
+        import torch
+
+        if t.dtype == torch.bfloat16:  # bfloat16 travels as uint16 bit patterns on the NumPy side
+            import numpy as np
+
+            return t.view(torch.int16).numpy().view(np.uint16)
+        return t.numpy()
+
+    def _t(self, a, like):
+        import numpy as np
+        import torch
+
+        if like.dtype == torch.bfloat16:
+            return torch.from_numpy(a.view(np.int16)).view(torch.bfloat16)
+        return torch.from_numpy(a)
+
+    def forward_(self, u, m, v, eps, eps_root, count):
+        if self.ref is not None:
+            self.ref.adam_op.forward_(u, m, v, B1, B2, eps, eps_root, count)
+        else:
+            self.port.forward_inplace(self._np(u), self._np(m), self._np(v), B1, B2, eps, eps_root,
+                                      count)
+
+    def forward_mu(self, u, m):
+        if self.ref is not None:
+            return self.ref.adam_op.forward_mu(u, m, B1)
+        return self._t(self.port.forward_mu(self._np(u), self._np(m), B1), u)
+
+    def forward_nu(self, u, v):
+        if self.ref is not None:
+            return self.ref.adam_op.forward_nu(u, v, B2)
+        return self._t(self.port.forward_nu(self._np(u), self._np(v), B2), u)
+
+    def forward_updates(self, m, v, eps, eps_root, count):
+        if self.ref is not None:
+            return self.ref.adam_op.forward_updates(m, v, B1, B2, eps, eps_root, count)
+        return self._t(self.port.forward_updates(self._np(m), self._np(v), B1, B2, eps, eps_root,
+                                                 count), m)
+
+    def backward_mu(self, d, u, m):
+        if self.ref is not None:
+            return self.ref.adam_op.backward_mu(d, u, m, B1)
+        return [self._t(a, d) for a in self.port.backward_mu(self._np(d), B1)]
+
+    def backward_nu(self, d, u, v):
+        if self.ref is not None:
+            return self.ref.adam_op.backward_nu(d, u, v, B2)
+        return [self._t(a, d) for a in self.port.backward_nu(self._np(d), self._np(u), B2)]
+
+    def backward_updates(self, d, u, m, v, eps_root, count):
+        if self.ref is not None:
+            return self.ref.adam_op.backward_updates(d, u, m, v, B1, B2, eps_root, count)
+        return [self._t(a, d) for a in self.port.backward_updates(
+            self._np(d), self._np(u), self._np(m), B1, B2, eps_root, count)]
+
+
+def ulp_report(pairs):
+    """(GPU tensor, CPU tensor) pairs -> elements checked, elements that differ, largest distance
+    in units in the last place (NaNs of any payload count as equal)."""
+    import numpy as np
+    import torch
+
+    checked = differing = worst = 0
+    for got, want in pairs:
+        got = got.detach().cpu()
+        bits = {2: torch.int16, 4: torch.int32, 8: torch.int64}[got.element_size()]
+        nan = torch.isnan(got.float() if got.element_size() == 2 else got) & torch.isnan(
+            want.float() if want.element_size() == 2 else want)
+        a = got.contiguous().view(bits).numpy().astype(np.int64)
+        b = want.contiguous().view(bits).numpy().astype(np.int64)
+        lo = int(np.iinfo({2: np.int16, 4: np.int32, 8: np.int64}[got.element_size()]).min)
+        a, b = np.where(a < 0, lo - a, a), np.where(b < 0, lo - b, b)  # monotone integer line
+        d = np.abs(a - b)
+        d[nan.numpy()] = 0
+        checked += d.size
+        differing += int(np.count_nonzero(d))
+        worst = max(worst, int(d.max(initial=0)))
+    return {'elements_checked': checked, 'differing': differing, 'max_ulp': worst}
+
+
 def run_cpu_baseline(cfg_id, budget_s=12.0):
-    """Time the reference CPU op (oracle/_ref, where built) or the C port on a bounded sample.
+    """The CPU ops the configuration names, timed on the host's cores on a bounded sample of the
+    same seeded inputs the GPU leg uses (untiled: every element its own draw), and the parity of
+    the GPU's results with the CPU's on that sample.
 
     Only this leg touches `oracle/`; it is the reported baseline, never the measured product.
     """
-    import numpy as np
+    import ctypes
 
-    from oracle import adam_oracle
-
-    cfg = CONFIGS[cfg_id]
-    tag = cfg['dtype']
-    np_dtype = {'f32': np.float32, 'f64': np.float64, 'f16': np.float16, 'bf16': np.float32}[tag]
-    eps = cfg.get('eps', EPS)
-    full = cfg['n'] if 'n' in cfg else sum(numel(s) for s in cfg['shapes'])
-    n = min(full, 1 << 26)
-
-    # the box's CPU share, not every core the machine shows
-    share = int(os.environ.get('OMP_NUM_THREADS', '16') or 16)
-    try:
-        avail = sorted(os.sched_getaffinity(0))
-        cores = max(1, min(share, len(avail)))
-        os.sched_setaffinity(0, set(avail[:cores]))
-    except (AttributeError, OSError):
-        cores = max(1, min(share, os.cpu_count() or 1))
-
-    rng = np.random.default_rng(1000 * cfg_id)
-    block = 1 << 20
-    reps = (n + block - 1) // block
-    u = np.tile(rng.standard_normal(block).astype(np_dtype), reps)[:n].copy()
-    mu = np.tile((0.1 * rng.standard_normal(block)).astype(np_dtype), reps)[:n].copy()
-    nu = np.tile(np.abs(0.01 * rng.standard_normal(block)).astype(np_dtype), reps)[:n].copy()
-    if tag == 'bf16':  # bfloat16 travels as uint16 bit patterns on the NumPy side
-        u, mu, nu = (adam_oracle.bf16_bits(a) for a in (u, mu, nu))
-
-    def as_torch(a):
-        t = torch.from_numpy(a.view(np.int16) if tag == 'bf16' else a)
-        return t.view(torch.bfloat16) if tag == 'bf16' else t
-
-    ref = None
-    try:
-        ref = adam_oracle.load_reference()
-    except Exception as exc:  # noqa: BLE001
-        print(f'[bench] compiled reference not usable ({exc}); timing the C port',
-              file=sys.stderr)
     import torch
 
     from torchopt_amd import _lib
 
-    if ref is not None:
-        tu, tm, tv = as_torch(u), as_torch(mu), as_torch(nu)  # share memory with u, mu, nu
-
-        def one():
-            ref.adam_op.forward_(tu, tm, tv, B1, B2, eps, cfg['eps_root'], cfg['count'])
-        kind = 'reference'
-    else:
-        def one():
-            adam_oracle.forward_inplace(u, mu, nu, B1, B2, eps, cfg['eps_root'], cfg['count'])
-        kind = 'port'
-
-    # Parity on this sample: the GPU's first application from the seeded state against the
-    # CPU's (which doubles as the CPU warm-up: threads, page faults).
-    dev = [as_torch(a).cuda() for a in (u, mu, nu)]
+    cfg = CONFIGS[cfg_id]
+    tag = cfg['dtype']
+    eps = cfg.get('eps', EPS)
+    eps_root, count = cfg['eps_root'], cfg['count']
+    esize = ESIZE[tag]
+    lib = _lib.load()
     code = {'f32': _lib.TOA_F32, 'f64': _lib.TOA_F64, 'f16': _lib.TOA_F16,
             'bf16': _lib.TOA_BF16}[tag]
-    rc = _lib.load().toa_adam_forward_inplace(
-        code, dev[0].data_ptr(), dev[1].data_ptr(), dev[2].data_ptr(), n, B1, B2, eps,
-        cfg['eps_root'], cfg['count'], torch.cuda.current_stream().cuda_stream)
-    if rc:
-        raise RuntimeError(f'toa_adam_forward_inplace returned {rc}')
-    one()
-    itype = {2: np.int16, 4: np.int32, 8: np.int64}[ESIZE[tag]]
-    worst, differing = 0, 0
-    for got, want in zip(dev, (u, mu, nu)):
-        got = got.view(torch.int16) if tag == 'bf16' else got
-        a = got.cpu().numpy().view(itype).astype(np.int64)
-        b = want.view(itype).astype(np.int64)
-        lo = np.iinfo(itype).min
-        a, b = np.where(a < 0, lo - a, a), np.where(b < 0, lo - b, b)  # monotone integer line
-        d = np.abs(a - b)
-        worst, differing = max(worst, int(d.max())), differing + int(np.count_nonzero(d))
-    del dev
-    parity = {'elements_checked': 3 * n, 'differing': differing, 'max_ulp': worst}
+    sptr = torch.cuda.current_stream().cuda_stream
+
+    cores = host_cores()
+    torch.set_num_threads(cores)
+    cpu = CpuOps()
+
+    def check(rc):
+        if rc:
+            raise RuntimeError(lib.toa_adam_error_string(rc).decode())
+
+    # ---- the leaves of the sample: seeded host arrays, cloned (the GPU leg owns the originals)
+    if 'shapes' in cfg:
+        sizes = [numel(x) for x in cfg['shapes']]
+        extra = 3 if cfg.get('differentiable') else (1 if cfg.get('fused_step') else 0)
+        leaves, taken = [], 0
+        for k, n in enumerate(sizes):
+            if taken + n > CPU_SAMPLE_ELEMS and leaves:
+                break
+            leaves.append([a.clone() for a in host_state(cfg_id, k, n, tag, extra=extra)])
+            taken += n
+        full = sum(sizes)
+        what = f'the first {len(leaves)} of {len(sizes)} tensors ({taken} of {full} elements)'
+    else:
+        full = cfg['n']
+        n = min(full, CPU_SAMPLE_ELEMS)
+        extra = 3 if cfg.get('backward') else 0
+        leaves = [[a[:n].clone() for a in host_state(cfg_id, 0, full, tag, extra=extra)]]
+        taken = n
+        what = (f'the first {n} of {full} elements' if n < full else f'all {full} elements')
+    dev = [[a.cuda() for a in leaf] for leaf in leaves]
+    num = len(leaves)
+
+    def col(j):
+        return (ctypes.c_void_p * num)(*[leaf[j].data_ptr() for leaf in dev])
+
+    ns = (ctypes.c_size_t * num)(*[leaf[0].numel() for leaf in leaves])
+
+    # ---- one pass of the configuration's ops on the CPU; the first pass doubles as warm-up
+    # (threads, page faults) and as the reference for the parity check
+    if cfg.get('differentiable'):
+        ops = 'forward_mu, forward_nu, forward_updates, backward_updates, backward_nu, backward_mu, leaf by leaf'
+        bytes_per_elem = 21 * esize  # 3 + 3 + 3 arrays forward, 5 + 4 + 3 backward
+
+        def one():
+            outs = []
+            for g, m, v, d_m, d_v, d_u in leaves:
+                new_m, new_v = cpu.forward_mu(g, m), cpu.forward_nu(g, v)
+                new_u = cpu.forward_updates(new_m, new_v, eps, eps_root, count)
+                bm, bv = cpu.backward_updates(d_u, new_u, new_m, new_v, eps_root, count)
+                outs.append((new_m, new_v, new_u, bm, bv, *cpu.backward_nu(d_v, g, v),
+                             *cpu.backward_mu(d_m, g, m)))
+            return outs
+
+        want = one()
+        o = [[torch.empty_like(leaf[0]) for leaf in dev] for _ in range(9)]
+        oc = [(ctypes.c_void_p * num)(*[t.data_ptr() for t in x]) for x in o]
+        check(lib.toa_adam_forward_mu_multi(code, num, col(0), col(1), ns, B1, oc[0], sptr))
+        check(lib.toa_adam_forward_nu_multi(code, num, col(0), col(2), ns, B2, oc[1], sptr))
+        check(lib.toa_adam_forward_updates_multi(code, num, oc[0], oc[1], ns, B1, B2, eps, eps_root,
+                                                 None, count, oc[2], sptr))
+        check(lib.toa_adam_backward_updates_multi(code, num, col(5), oc[2], oc[0], ns, B1, B2,
+                                                  eps_root, None, count, oc[3], oc[4], sptr))
+        check(lib.toa_adam_backward_nu_multi(code, num, col(4), col(0), ns, B2, oc[5], oc[6], sptr))
+        check(lib.toa_adam_backward_mu_multi(code, num, col(3), ns, B1, oc[7], oc[8], sptr))
+        pairs = [(o[j][k], want[k][j]) for k in range(num) for j in range(9)]
+    elif cfg.get('backward'):
+        ops = 'forward_ in place, then backward_mu, backward_nu, backward_updates'
+        bytes_per_elem = (6 + 3 + 4 + 5) * esize
+        g0, m0, v0, d_m, d_v, d_u = leaves[0]
+        gw, mw, vw = g0.clone(), m0.clone(), v0.clone()  # forward_ overwrites these, pass after pass
+
+        def one():
+            cpu.forward_(gw, mw, vw, eps, eps_root, count)  # gw: the update, mw / vw: new moments
+            return (gw, mw, vw, *cpu.backward_mu(d_m, g0, m0), *cpu.backward_nu(d_v, g0, v0),
+                    *cpu.backward_updates(d_u, gw, mw, vw, eps_root, count))
+
+        want = [t.clone() for t in one()]
+        dg, dm, dv = (t.clone() for t in dev[0][:3])
+        o = [torch.empty_like(dg) for _ in range(6)]
+        p = [t.data_ptr() for t in o]
+        check(lib.toa_adam_forward_inplace(code, dg.data_ptr(), dm.data_ptr(), dv.data_ptr(), taken,
+                                           B1, B2, eps, eps_root, count, sptr))
+        check(lib.toa_adam_backward_mu(code, dev[0][3].data_ptr(), taken, B1, p[0], p[1], sptr))
+        check(lib.toa_adam_backward_nu(code, dev[0][4].data_ptr(), dev[0][0].data_ptr(), taken, B2,
+                                       p[2], p[3], sptr))
+        check(lib.toa_adam_backward_updates(code, dev[0][5].data_ptr(), dg.data_ptr(),
+                                            dm.data_ptr(), taken, B1, B2, eps_root, count, p[4],
+                                            p[5], sptr))
+        pairs = list(zip((dg, dm, dv, *o), want))
+    elif cfg.get('fused_step'):
+        ops = 'forward_ in place, updates.mul_(-lr), params.add_(updates), leaf by leaf'
+        bytes_per_elem = 11 * esize
+        lr = 1e-3
+
+        def one():
+            for g, m, v, p in leaves:
+                cpu.forward_(g, m, v, eps, eps_root, count)
+                g.mul_(-lr)
+                p.add_(g)
+
+        one()
+        check(lib.toa_adam_fused_step_multi(code, num, col(3), col(0), col(1), col(2), ns, B1, B2,
+                                            eps, eps_root, None, count, lr, 0.0, 0, 0, 1, sptr))
+        pairs = [(dev[k][j], leaves[k][j]) for k in range(num) for j in range(4)]
+    else:
+        ops = 'forward_ in place' + (', leaf by leaf' if num > 1 else '')
+        bytes_per_elem = 6 * esize
+
+        def one():
+            for g, m, v in leaves:
+                cpu.forward_(g, m, v, eps, eps_root, count)
+
+        one()
+        check(lib.toa_adam_forward_inplace_multi(code, num, col(0), col(1), col(2), ns, B1, B2,
+                                                 eps, eps_root, None, count, sptr))
+        pairs = [(dev[k][j], leaves[k][j]) for k in range(num) for j in range(3)]
+    torch.cuda.synchronize()
+    parity = ulp_report(pairs)
+    del dev, pairs
 
     times = []
     t_end = time.perf_counter() + budget_s
-    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 25):
+    while len(times) < 5 or (time.perf_counter() < t_end and len(times) < 25):
         t0 = time.perf_counter()
         one()
         times.append(time.perf_counter() - t0)
     med = sorted(times)[len(times) // 2]
-    esize = ESIZE[tag]
     return {
-        'value': n / med, 'unit': 'elements/s', 'cores': cores, 'kind': kind,
-        'sample': f'{n} of {full} elements ({cfg["dtype"]}), forward_ in place, '
-                  f'median of {len(times)} passes after 1 warm-up',
-        'gb_per_s': round(BYTES_PER_ELEM['forward_'] * esize * n / med / 1e9, 2),
+        'value': taken / med, 'unit': 'elements/s', 'cores': cores, 'kind': cpu.kind,
+        'sample': f'{what} ({tag}); {ops}; median of {len(times)} passes after 1 warm-up pass; '
+                  'untiled seeded inputs, the ones the GPU leg uses',
+        'gb_per_s': round(bytes_per_elem * taken / med / 1e9, 2),
+        'bytes_per_element': bytes_per_elem,
+        'cpu_model': cpu_model(),
+        'threads_policy': 'min(n / 1000, cores) per op, as the reference sets it',
+        'omp': {k: os.environ.get(k, 'unset') for k in ('OMP_NUM_THREADS', 'OMP_PROC_BIND',
+                                                      'OMP_PLACES')},
+        'note': 'host CPUs differ between GPU boxes (5e9 to 1e10 elements/s seen for config 2): '
+                'compare only within one line',
         'parity_gpu_vs_cpu': parity,
     }
 
@@ -659,6 +900,8 @@ def main(argv=None):
         print(json.dumps(run_ceiling()), flush=True)
         return 0
 
+    host_cores()  # before torch (and with it the OpenMP runtime) loads
+
     gpu = run_gpu(args.config, args.steps, args.warmup)
     cfg = CONFIGS[args.config]
     if args.pmc_calibration:
@@ -684,7 +927,7 @@ def main(argv=None):
         'scaling': 'weak',
         'vs_baseline': None,
         'dtype': cfg['dtype'],
-        'data': 'synthetic',
+        'data': 'synthetic (seeded CPU generator, seed = 1000 * config + tensor index, uploaded once)',
         'config': {'workload': cfg['name'], 'elements': gpu['elements'], 'b1': B1, 'b2': B2,
                    'eps': cfg.get('eps', EPS), 'eps_root': cfg['eps_root'], 'count': cfg['count'],
                    'device': gpu['device'], **gpu['extra']},
@@ -692,6 +935,7 @@ def main(argv=None):
     }
     if not args.no_cpu_baseline:
         line['cpu_baseline'] = run_cpu_baseline(args.config)
+    _HOST.clear()
     print(json.dumps(line), flush=True)
     return 0
 
