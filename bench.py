@@ -153,16 +153,16 @@ def host_state(cfg_id, index, n, tag, extra=0):
     return _HOST[key]
 
 
-def preheat(torch, lib, stream, launches=150):
+def preheat(torch, launches=120):
     """GPU clocks ramp for the first ~15 ms of sustained load in a cold process (the state was
     just generated on the host and uploaded, so the GPU has been idle): stream through scratch
-    arrays -- never the benchmark's own state -- for ~40 ms before the warm-up steps."""
-    n = 1 << 26
-    scratch = [torch.rand(n, device='cuda') for _ in range(3)]
-    p = [t.data_ptr() for t in scratch]
+    arrays -- never the benchmark's own state, and with PyTorch's own kernels, so that a kernel
+    trace of the run holds the operator's kernels for the benchmark's steps only -- for ~40 ms
+    before the warm-up steps."""
+    a = torch.rand(1 << 27, device='cuda')
+    b = torch.rand(1 << 27, device='cuda')
     for _ in range(launches):
-        lib.toa_adam_forward_inplace(0, p[0], p[1], p[2], n, B1, B2, EPS, 0.0, 7,
-                                     stream.cuda_stream)
+        a.add_(b)
     torch.cuda.synchronize()
     return launches
 
@@ -447,7 +447,7 @@ def run_gpu(cfg_id, steps, warmup):
             del sweep
             extra['cold_cache_ms_per_launch'] = round(sorted(cold)[len(cold) // 2], 5)
 
-    extra['preheat_launches_on_scratch_arrays'] = preheat(torch, lib, stream)
+    extra['preheat_launches_on_scratch_arrays'] = preheat(torch)
     for _ in range(warmup):
         step()
     ev0 = torch.cuda.Event(enable_timing=True)
@@ -522,6 +522,24 @@ def lds_for_waves(waves):
     return 0 if waves >= 32 else (128 // (waves + 1) + 1) * 1280
 
 
+# Launch shapes of bench_probe_inplace3 (three arrays read and written back) and the residency
+# levels each is swept over: workgroups per compute unit through the LDS reservation, except for
+# the persistent grid, whose level is its grid size per compute unit.
+INPLACE3_SHAPES = (
+    ('one wave per workgroup, one 1 KiB tile per wave (the plain schedule)', 0,
+     (32, 25, 21, 18, 16, 14, 12, 11, 10, 9, 8)),
+    ('same, one memory operation of a wave at a time (the staged schedule)', 1,
+     (32, 25, 21, 18, 16, 14, 12)),
+    ('same, a wait after every load and store', 2, (32, 25, 21, 18, 16)),
+    ('256-thread workgroups, one tile per wave', 3, (8, 6, 5, 4, 3, 2)),
+    ('512-thread workgroups, one tile per wave', 4, (4, 3, 2)),
+    ('two tiles per wave, all loads before the first store', 5, (16, 12, 10, 8, 7, 6, 5, 4)),
+    ('four tiles per wave, all loads before the first store', 6, (8, 6, 5, 4, 3, 2)),
+    ('persistent grid striding over the tiles, next tile loaded before the current one is '
+     'stored', 7, (16, 12, 10, 8, 6, 4)),
+)
+
+
 def run_ceiling(array_bytes=1 << 30, reps=20):
     import ctypes
 
@@ -534,9 +552,26 @@ def run_ceiling(array_bytes=1 << 30, reps=20):
     probe.bench_probe_stream.argtypes = [ctypes.c_int, ctypes.c_int,
                                          ctypes.POINTER(ctypes.c_void_p), ctypes.c_size_t,
                                          ctypes.c_uint, ctypes.c_void_p]
+    probe.bench_probe_inplace3.restype = ctypes.c_int
+    probe.bench_probe_inplace3.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
+                                           ctypes.c_void_p, ctypes.c_size_t, ctypes.c_size_t,
+                                           ctypes.c_uint, ctypes.c_int, ctypes.c_void_p]
     stream = torch.cuda.current_stream()
-    arrays = [torch.rand(array_bytes // 4, device='cuda') for _ in range(7)]
+    # normally distributed like the operator's state: throughput depends on the bits moved
+    arrays = [torch.randn(array_bytes // 4, device='cuda') for _ in range(7)]
     torch.cuda.synchronize()
+
+    def timed(launch):
+        for _ in range(4):
+            launch()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record(stream)
+        for _ in range(reps):
+            launch()
+        ev1.record(stream)
+        torch.cuda.synchronize()
+        return ev0.elapsed_time(ev1) / reps
+
     out = {}
     shapes = [(r, w, False) for r, w in ((1, 0), (3, 0), (0, 1), (0, 3), (1, 1), (2, 1), (3, 3),
                                          (4, 3))]
@@ -552,22 +587,64 @@ def run_ceiling(array_bytes=1 << 30, reps=20):
                                               lds_for_waves(waves), stream.cuda_stream)
                 if rc:
                     raise RuntimeError(f'bench_probe_stream({reads}, {writes}) returned {rc}')
-            for _ in range(4):
-                launch()
-            ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            ev0.record(stream)
-            for _ in range(reps):
-                launch()
-            ev1.record(stream)
-            torch.cuda.synchronize()
-            gbs = (reads + writes) * array_bytes / (ev0.elapsed_time(ev1) / reps * 1e-3) / 1e9
+            gbs = (reads + writes) * array_bytes / (timed(launch) * 1e-3) / 1e9
             if gbs > best[0]:
                 best = (gbs, waves)
         out[f'{reads}R{writes}W' + (' in place' if in_place else '')] = {'GB/s': round(best[0], 1), 'frac_of_peak': round(
             best[0] / HBM_PEAK_GBS, 4), 'waves_per_cu': best[1]}
+
+    # The in-place step's pattern under a family of launch shapes, on two placements of the same
+    # three arrays: separate allocations as the allocator hands them out (what the operator
+    # gets), and one arena in which they interleave in 64 KiB pieces (the most favourable
+    # placement found: every wave's three tiles then sit in different DRAM banks).
+    del arrays[3:]
+    arena = torch.randn(3 * (array_bytes // 4), device='cuda')
+    a0, a1, a2 = (t.data_ptr() for t in arrays)
+    layouts = (('three separate arrays', (a0, a1, a2), 0),
+               ('one arena, arrays interleaved in 64 KiB pieces', (arena.data_ptr(), None, None),
+                64 << 10))
+    family = {}
+    for layout, ptrs3, piece in layouts:
+        rows, top = {}, (0.0, None)
+        for name, code, levels in INPLACE3_SHAPES:
+            best = (0.0, None)
+            for level in levels:
+                lds = 0 if code == 7 else lds_for_waves(level)
+
+                def launch():
+                    rc = probe.bench_probe_inplace3(code, ptrs3[0], ptrs3[1], ptrs3[2], array_bytes,
+                                                    piece, lds, level, stream.cuda_stream)
+                    if rc:
+                        raise RuntimeError(f'bench_probe_inplace3(shape {code}) returned {rc}')
+                gbs = 6 * array_bytes / (timed(launch) * 1e-3) / 1e9
+                if gbs > best[0]:
+                    best = (gbs, level)
+            rows[name] = {'GB/s': round(best[0], 1), 'frac_of_peak': round(best[0] / HBM_PEAK_GBS, 4),
+                          'workgroups_per_cu': best[1]}
+            if best[0] > top[0]:
+                top = (best[0], name)
+        family[layout] = {'shapes': rows, 'best_shape': top[1], 'best_GB/s': round(top[0], 1),
+                          'best_frac_of_peak': round(top[0] / HBM_PEAK_GBS, 4)}
+    # The same pass (staged shape, three separate arrays) over other data: the rate depends on the
+    # bits that cross the memory interface, so a ceiling holds for the data it was taken on.
+    by_data = {}
+    for label, fill in (('zeros', lambda t: t.zero_()),
+                        ('uniform in [1, 2): one sign, one exponent', lambda t: t.uniform_(1.0, 2.0)),
+                        ('normal (0, 1), as the operator\'s gradients', lambda t: t.normal_())):
+        for t in arrays:
+            fill(t)
+
+        def launch():
+            rc = probe.bench_probe_inplace3(1, a0, a1, a2, array_bytes, 0, lds_for_waves(18), 0,
+                                            stream.cuda_stream)
+            if rc:
+                raise RuntimeError(f'bench_probe_inplace3 returned {rc}')
+        by_data[label] = round(6 * array_bytes / (timed(launch) * 1e-3) / 1e9, 1)
     return {'metric': 'hbm_streaming_ceiling', 'unit': 'GB/s', 'peak': HBM_PEAK_GBS,
             'array_bytes': array_bytes, 'launches_timed': reps,
-            'device': torch.cuda.get_device_name(0), 'ceilings': out}
+            'device': torch.cuda.get_device_name(0), 'ceilings': out,
+            'three_arrays_read_and_written_back': family,
+            'staged_shape_by_data_GB/s': by_data}
 
 
 # ----------------------------------------------------------------------------- CPU baseline
