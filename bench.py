@@ -114,11 +114,11 @@ CONFIGS = {
             dtype='f32', shapes=gpt2_medium_shapes(), eps_root=0.0, count=1, fused_step=True),
     6: dict(name='config6: fused forward_ in place, 268 435 456 float16 elements (arithmetic of '
                  'the reference CPU op on at::Half: every operation rounded to 16 bits), '
-                 'eps=1e-3, count=1000, a fresh gradient array every step',
+                 'eps=1e-3, count=1000, gradients from eight arrays in rotation',
             dtype='f16', n=1 << 28, eps=1e-3, eps_root=0.0, count=1000, fresh_gradients=True),
     7: dict(name='config7: fused forward_ in place, 268 435 456 bfloat16 elements (arithmetic of '
-                 'the reference CPU op on at::BFloat16), eps=1e-3, count=1000, a fresh gradient array '
-                 'every step',
+                 'the reference CPU op on at::BFloat16), eps=1e-3, count=1000, gradients from eight '
+                 'arrays in rotation',
             dtype='bf16', n=1 << 28, eps=1e-3, eps_root=0.0, count=1000, fresh_gradients=True),
 }
 ESIZE = {'f32': 4, 'f64': 8, 'f16': 2, 'bf16': 2}
@@ -404,12 +404,12 @@ def run_gpu(cfg_id, steps, warmup):
             # A training loop hands the step a new gradient every time; re-applying the step to
             # its own output instead drives every element towards one fixed point, which no real
             # run does and which the 16-bit kernels' data-dependent quick route would be timed
-            # on.  So each step gets its own freshly drawn gradient array (as many as the step
-            # count, at most 64 of them in rotation).
+            # on.  So the steps draw their gradients from eight arrays in rotation (a training loop
+            # reuses its gradient buffers too: pages and TLB entries are warm, the values new).
             g = torch.Generator(device='cuda')
             g.manual_seed(1000 * cfg_id + 1)
             fresh = [torch.randn(total, device='cuda', generator=g).to(dtype)
-                     for _ in range(min(steps + warmup, 64))]
+                     for _ in range(min(steps + warmup, 8))]
             ptrs, turn = [t.data_ptr() for t in fresh], [0]
             extra['gradient_arrays'] = len(fresh)
 

@@ -77,6 +77,23 @@ struct HalfFormat {  // IEEE binary16
         return sign | (uint16_t)h;
 #endif
     }
+    // two values at once (element 0 in the low half); same rounding as encode / decode
+    static __host__ __device__ inline uint32_t encode2(float lo, float hi) {
+#if defined(__HIP_DEVICE_COMPILE__)
+        typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+        typedef float float2_t __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2_t{lo, hi}, half2_t));
+#else
+        return (uint32_t)encode(lo) | ((uint32_t)encode(hi) << 16);
+#endif
+    }
+    static __host__ __device__ inline void decode2(uint32_t p, float &lo, float &hi) {
+        lo = decode((uint16_t)(p & 0xffffu));
+        hi = decode((uint16_t)(p >> 16));
+    }
+    static __host__ __device__ inline void round2(float a, float b, float &lo, float &hi) {
+        decode2(encode2(a, b), lo, hi);
+    }
     static __host__ __device__ inline float decode(uint16_t h) {
 #if defined(__HIP_DEVICE_COMPILE__)
         return static_cast<float>(__builtin_bit_cast(_Float16, h));
@@ -102,6 +119,30 @@ struct BFloatFormat {  // upper half of a binary32, round to nearest even
     }
     static __host__ __device__ inline float decode(uint16_t b) {
         return __builtin_bit_cast(float, (uint32_t)b << 16);
+    }
+    // two values at once (element 0 in the low half): one v_cvt_pk_bf16_f32 rounds both
+    static __host__ __device__ inline uint32_t encode2(float lo, float hi) {
+#if defined(__HIP_DEVICE_COMPILE__)
+        typedef __bf16 bfloat2_t __attribute__((ext_vector_type(2)));
+        typedef float float2_t __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2_t{lo, hi}, bfloat2_t));
+#else
+        return (uint32_t)encode(lo) | ((uint32_t)encode(hi) << 16);
+#endif
+    }
+    static __host__ __device__ inline void decode2(uint32_t p, float &lo, float &hi) {
+        lo = __builtin_bit_cast(float, p << 16);
+        hi = __builtin_bit_cast(float, p & 0xffff0000u);
+    }
+    // f rounded to bfloat16 and left in a float: a bfloat16 is the upper half of a float, so
+    // converting the pair (0, f) yields that float's bit pattern outright -- one instruction,
+    // where convert-then-widen takes two.
+    static __host__ __device__ inline float rounded(float f) {
+        return __builtin_bit_cast(float, encode2(0.0f, f));
+    }
+    static __host__ __device__ inline void round2(float a, float b, float &lo, float &hi) {
+        lo = rounded(a);
+        hi = rounded(b);
     }
 };
 
@@ -153,6 +194,72 @@ __host__ __device__ inline bool operator==(R16<F> a, int b) { return (float)a ==
 using half_t = R16<HalfFormat>;
 using bfloat_t = R16<BFloatFormat>;
 
+// ---------------------------------------------------------------------------
+// Two 16-bit values computed side by side (device code only).  Same arithmetic as R16 -- every
+// operation between 16-bit values rounded back to 16 bits, operations with a float operand left
+// unrounded -- but the two values stay in registers as floats that are exactly representable in
+// the 16-bit format: a bfloat16 rounding is then ONE instruction (see BFloatFormat::rounded)
+// instead of convert-and-widen, a float16 rounding one packed conversion for both values, and
+// the two results leave as one packed word.  Roundings are what the 16-bit kernels spend most of
+// their time on.
+// ---------------------------------------------------------------------------
+struct Float2 {  // two unrounded floats
+    float lo, hi;
+};
+
+template <class F>
+struct Pair16 {
+    float lo, hi;  // each exactly representable in F
+    Pair16() = default;
+    __device__ static Pair16 from_bits(uint32_t p) {
+        Pair16 r;
+        F::decode2(p, r.lo, r.hi);
+        return r;
+    }
+    __device__ static Pair16 rounded(float a, float b) {
+        Pair16 r;
+        F::round2(a, b, r.lo, r.hi);
+        return r;
+    }
+    __device__ uint32_t bits() const { return F::encode2(lo, hi); }  // exact: nothing to round
+    __device__ explicit Pair16(R16<F> s) {
+        lo = hi = (float)s;
+    }
+    __device__ Pair16(int i) { *this = rounded((float)i, (float)i); }
+    __device__ Pair16(Float2 f) { *this = rounded(f.lo, f.hi); }  // the one rounding of a result
+    __device__ R16<F> half(int h) const { return R16<F>(h ? hi : lo); }
+};
+#define TOA_PAIR_BINOP(OP)                                                                       \
+    template <class F>                                                                           \
+    __device__ inline Pair16<F> operator OP(Pair16<F> a, Pair16<F> b) {                          \
+        return Pair16<F>::rounded(a.lo OP b.lo, a.hi OP b.hi);                                   \
+    }                                                                                            \
+    template <class F>                                                                           \
+    __device__ inline Pair16<F> operator OP(int a, Pair16<F> b) {                                \
+        return Pair16<F>(a) OP b;                                                                \
+    }                                                                                            \
+    template <class F>                                                                           \
+    __device__ inline Float2 operator OP(Pair16<F> a, Float2 b) {                                \
+        return {a.lo OP b.lo, a.hi OP b.hi};                                                     \
+    }                                                                                            \
+    template <class F>                                                                           \
+    __device__ inline Float2 operator OP(Float2 a, Pair16<F> b) {                                \
+        return {a.lo OP b.lo, a.hi OP b.hi};                                                     \
+    }
+TOA_PAIR_BINOP(+)
+TOA_PAIR_BINOP(-)
+TOA_PAIR_BINOP(*)
+TOA_PAIR_BINOP(/)
+#undef TOA_PAIR_BINOP
+template <typename T>
+struct PairOf {  // the pair type a 16-bit element type computes in; void for the wide types
+    using type = void;
+};
+template <class F>
+struct PairOf<R16<F>> {
+    using type = Pair16<F>;
+};
+
 // 128-bit access types and element accessors.
 template <typename T>
 struct Vec;
@@ -200,6 +307,12 @@ __device__ __forceinline__ double toa_sqrt(double x) { return sqrt(x); }
 // a 16-bit value picks the float overload; the root is NOT rounded back
 template <class F>
 __device__ __forceinline__ float toa_sqrt(R16<F> x) { return sqrtf((float)x); }
+
+// as for one 16-bit value: the root is taken in float and NOT rounded back
+template <class F>
+__device__ __forceinline__ Float2 toa_sqrt(Pair16<F> x) {
+    return {sqrtf(x.lo), sqrtf(x.hi)};
+}
 
 // The step direction mu_hat / (sqrt(nu_hat + eps_root) + eps) as the reference writes it
 // (adam_op_impl_cpu.cpp:58-60, 177-179).
@@ -265,6 +378,55 @@ __device__ __forceinline__ half_t adam_direction_quick(half_t mh, half_t vh, hal
          ((aq >= 6.10351562e-05f && aq <= 32768.0f) || m == 0.0f) &&  // 2^-14 .. 2^15
          (low - 0x0ff0u > 0x20u);  // not within 16 ulps of the midpoint 0x1000
     return half_t(q);
+}
+
+// The quick route for two values at once; returns the halves that must repeat through the exact
+// chain (bit 0: low, bit 1: high).  Same claims as above, with the conditions that do not depend
+// on the element checked once: with 2^-64 <= eps <= 2^63 and a radicand that is zero or a positive
+// normal number (or eps = 0 and a positive normal radicand), root + eps lies in [2^-64, 2^65] --
+// the reciprocal's good range -- whatever the element, so only the radicand's class, the quotient's range and its distance from a rounding
+// midpoint remain per element.  Written without short-circuit operators: the compiler then emits
+// straight-line compares instead of a branch per element.
+template <class F>
+struct QuickLimits;
+template <>
+struct QuickLimits<BFloatFormat> {  // 8 significant bits; any normal float result will do
+    static constexpr uint32_t kLowMask = 0xffffu, kMid = 0x8000u;
+    static constexpr uint32_t kMinBits = 0x0d800000u, kMaxBits = 0x71800000u;  // 2^-100 .. 2^100
+};
+template <>
+struct QuickLimits<HalfFormat> {  // 11 significant bits; the result must be a normal float16
+    static constexpr uint32_t kLowMask = 0x1fffu, kMid = 0x1000u;
+    static constexpr uint32_t kMinBits = 0x38800000u, kMaxBits = 0x47000000u;  // 2^-14 .. 2^15
+};
+
+template <class F>
+__device__ __forceinline__ Pair16<F> adam_direction_quick(Pair16<F> mh, Pair16<F> vh,
+                                                          Pair16<F> eps_root, Pair16<F> eps,
+                                                          uint32_t &bad) {
+    using L = QuickLimits<F>;
+    const Pair16<F> x = vh + eps_root;
+    const float e = eps.lo;  // both halves hold the same hyper-parameter
+    // eps = 0 is served too: the radicand must then be positive (a zero one would divide by zero)
+    const bool eps_fits = ((e >= 5.42101086e-20f) & (e <= 9.22337204e18f)) | (e == 0.0f);
+    const int radicand_classes = e == 0.0f ? 0x100 : 0x160;
+    auto one = [&](float xx, float m, float &q) -> bool {
+        const float d = __builtin_amdgcn_sqrtf(xx) + e;
+        q = m * __builtin_amdgcn_rcpf(d);
+        const uint32_t qb = __builtin_bit_cast(uint32_t, q);
+        const uint32_t aq = qb & 0x7fffffffu;
+        // zero or a positive normal radicand (class bits: +normal 0x100, +0 0x040, -0 0x020)
+        const bool radicand = __builtin_amdgcn_classf(xx, radicand_classes);
+        const bool range = (aq - L::kMinBits <= L::kMaxBits - L::kMinBits) | (aq == 0u);
+        // not within 16 float ulps of the midpoint between two 16-bit values
+        const bool clear = ((qb & L::kLowMask) - (L::kMid - 0x10u)) > 0x20u;
+        return radicand & range & clear;
+    };
+    float q_lo, q_hi;
+    const bool ok_lo = one(x.lo, mh.lo, q_lo) & eps_fits;
+    const bool ok_hi = one(x.hi, mh.hi, q_hi) & eps_fits;
+    bad = (ok_lo ? 0u : 1u) | (ok_hi ? 0u : 2u);
+    return Pair16<F>::rounded(q_lo, q_hi);
 }
 
 // An op is speculative when it offers `quick(in, out) -> bool` beside the exact operator():
@@ -406,12 +568,36 @@ struct AdamSteps {
         c1 = c1_;
         c2 = c2_;
     }
-    __device__ __forceinline__ T first(T g, T m) const { return b1 * m + (1 - b1) * g; }
-    __device__ __forceinline__ T second(T g, T v) const { return b2 * v + (1 - b2) * g * g; }
-    __device__ __forceinline__ T third(T m1, T v1) const {
-        const T mh = m1 * c1;
-        const T vh = v1 * c2;
-        return adam_direction(mh, vh, eps_root, eps);
+    // U is T, or for the 16-bit types the pair type that computes two elements side by side
+    template <class U>
+    __device__ __forceinline__ U first(U g, U m) const {
+        return U(b1) * m + (1 - U(b1)) * g;
+    }
+    template <class U>
+    __device__ __forceinline__ U second(U g, U v) const {
+        return U(b2) * v + (1 - U(b2)) * g * g;
+    }
+    template <class U>
+    __device__ __forceinline__ U third(U m1, U v1) const {
+        const U mh = m1 * U(c1);
+        const U vh = v1 * U(c2);
+        return adam_direction(mh, vh, U(eps_root), U(eps));
+    }
+    // two elements through all three steps, the third by the quick route; returns the halves
+    // that must repeat through the exact chain (bit 0, bit 1)
+    template <class P>
+    __device__ __forceinline__ uint32_t quick_pair(const P (&in)[3], P (&out)[3]) const {
+        out[0] = first<P>(in[0], in[1]);
+        out[1] = second<P>(in[0], in[2]);
+        return third_quick_pair<P>(out[0], out[1], out[2]);
+    }
+    template <class P>
+    __device__ __forceinline__ uint32_t third_quick_pair(P m1, P v1, P &out) const {
+        const P mh = m1 * P(c1);
+        const P vh = v1 * P(c2);
+        uint32_t bad;
+        out = adam_direction_quick(mh, vh, P(eps_root), P(eps), bad);
+        return bad;
     }
     __device__ __forceinline__ bool third_quick(T m1, T v1, T &out) const {
         const T mh = m1 * c1;
@@ -428,42 +614,87 @@ struct AdamSteps {
     __device__ __forceinline__ void staged_steps(const IO &io) const {
         using V = typename Vec<T>::type;
         constexpr int VN = Vec<T>::N;
-        const V g = io.load(0);
-        io.wait();
-        const V m = io.load(1);
-        io.wait();
-        const V a = vmap<T>(g, m, [&](T x, T y) { return first(x, y); });
-        io.store(Op::out_slot(0), a);
-        const V v = io.load(2);
-        io.wait();
-        const V b = vmap<T>(g, v, [&](T x, T y) { return second(x, y); });
-        io.store(Op::out_slot(1), b);
-        V c;
-        if constexpr (HasQuickDirection<T>::value) {
+        if constexpr (__is_same(T, bfloat_t)) {
+            // bfloat16: two elements per step (see Pair16), the quick route for both.  (float16
+            // gains nothing from pairs here -- its roundings have no one-instruction form -- and
+            // takes the element-wise branch below.)
+            using P = typename PairOf<T>::type;
+            typedef uint32_t Words __attribute__((ext_vector_type(4)));
+            const Words g = __builtin_bit_cast(Words, io.load(0));
+            io.wait();
+            const Words m = __builtin_bit_cast(Words, io.load(1));
+            io.wait();
+            P gp[4], ap[4], bp[4];
+            Words a, b, c;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                gp[e] = P::from_bits(g[e]);
+                ap[e] = first<P>(gp[e], P::from_bits(m[e]));
+                a[e] = ap[e].bits();
+            }
+            io.store(Op::out_slot(0), __builtin_bit_cast(V, a));
+            const Words v = __builtin_bit_cast(Words, io.load(2));
+            io.wait();
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                bp[e] = second<P>(gp[e], P::from_bits(v[e]));
+                b[e] = bp[e].bits();
+            }
+            io.store(Op::out_slot(1), __builtin_bit_cast(V, b));
             uint32_t redo = 0;
 #pragma unroll
-            for (int e = 0; e < VN; ++e) {
-                T r;
-                if (!third_quick(Vec<T>::get(a, e), Vec<T>::get(b, e), r)) redo |= 1u << e;
-                Vec<T>::set(c, e, r);
+            for (int e = 0; e < 4; ++e) {
+                P r;
+                redo |= third_quick_pair<P>(ap[e], bp[e], r) << (2 * e);
+                c[e] = r.bits();
             }
+            V res = __builtin_bit_cast(V, c);
             if (redo != 0) {  // rare: an element the quick route could not settle
+                const V av = __builtin_bit_cast(V, a), bv = __builtin_bit_cast(V, b);
 #pragma unroll
                 for (int e = 0; e < VN; ++e)
                     if (redo & (1u << e))
-                        Vec<T>::set(c, e, third(Vec<T>::get(a, e), Vec<T>::get(b, e)));
+                        Vec<T>::set(res, e, third<T>(Vec<T>::get(av, e), Vec<T>::get(bv, e)));
             }
+            io.store(Op::out_slot(2), res);
         } else {
-            c = vmap<T>(a, b, [&](T x, T y) { return third(x, y); });
+            const V g = io.load(0);
+            io.wait();
+            const V m = io.load(1);
+            io.wait();
+            const V a = vmap<T>(g, m, [&](T x, T y) { return first<T>(x, y); });
+            io.store(Op::out_slot(0), a);
+            const V v = io.load(2);
+            io.wait();
+            const V b = vmap<T>(g, v, [&](T x, T y) { return second<T>(x, y); });
+            io.store(Op::out_slot(1), b);
+            V c;
+            if constexpr (HasQuickDirection<T>::value) {
+                uint32_t redo = 0;
+#pragma unroll
+                for (int e = 0; e < VN; ++e) {
+                    T r;
+                    if (!third_quick(Vec<T>::get(a, e), Vec<T>::get(b, e), r)) redo |= 1u << e;
+                    Vec<T>::set(c, e, r);
+                }
+                if (redo != 0) {  // rare: an element the quick route could not settle
+#pragma unroll
+                    for (int e = 0; e < VN; ++e)
+                        if (redo & (1u << e))
+                            Vec<T>::set(c, e, third<T>(Vec<T>::get(a, e), Vec<T>::get(b, e)));
+                }
+            } else {
+                c = vmap<T>(a, b, [&](T x, T y) { return third<T>(x, y); });
+            }
+            io.store(Op::out_slot(2), c);
         }
-        io.store(Op::out_slot(2), c);
     }
     template <bool QUICK>
     __device__ __forceinline__ bool run(const T (&in)[3], T (&out)[3]) const {
-        out[0] = first(in[0], in[1]);
-        out[1] = second(in[0], in[2]);
+        out[0] = first<T>(in[0], in[1]);
+        out[1] = second<T>(in[0], in[2]);
         if constexpr (QUICK) return third_quick(out[0], out[1], out[2]);
-        out[2] = third(out[0], out[1]);
+        out[2] = third<T>(out[0], out[1]);
         return true;
     }
     __device__ __forceinline__ void operator()(const T (&in)[3], T (&out)[3]) const {
@@ -479,19 +710,19 @@ template <typename T>
 struct ForwardInplace : AdamSteps<T> {
     static constexpr int NIN = 3, NOUT = 3, NPTR = 3;
     // read-modify-write: a tight window wins
-    static constexpr int kWavesPerCU = waves_by_type<T>(12, 10, 16, 32);
-    static constexpr int kWavesPerCUMulti = waves_by_type<T>(16, 21, 32);
-    // The staged schedule (tile_full_staged) exposes a wave's whole arithmetic between its memory
-    // operations; bfloat16's re-rounding makes that long enough to cost more than the schedule
-    // gains (5.9 against 6.3 TB/s), so bfloat16 keeps the plain one.
-    static constexpr bool kStaged = !__is_same(T, bfloat_t);
-    static constexpr int kWavesPerCUStaged = waves_by_type<T>(18, 18, 21, 32);
-    // A list gains nothing from the staged schedule (6.51 TB/s either way on the GPT-2-medium
-    // list) unless its arrays collide in DRAM, so lists are staged only then.
-    static constexpr bool kStagedLists = false;
+    static constexpr int kWavesPerCU = waves_by_type<T>(12, 10, 16, 14);
+    static constexpr int kWavesPerCUMulti = waves_by_type<T>(16, 25, 25);
+    static constexpr bool kStaged = true;
+    static constexpr int kWavesPerCUStaged = waves_by_type<T>(18, 18, 21, 21);
+    // A float32 / float64 list gains nothing from the staged schedule (6.5-6.6 TB/s either way
+    // on the GPT-2-medium list) unless its arrays collide in DRAM, so such lists are staged only
+    // then; the 16-bit lists gain 5-10 % from it at full residency.
+    static constexpr bool kStagedLists = sizeof(T) == 2;
+    static constexpr int kWavesPerCUStagedLists = waves_by_type<T>(18, 18, 32, 32);
     // outputs are produced as (mu', nu', updates') and stored in that order
     __device__ static constexpr int out_slot(int j) { return j == 0 ? 1 : (j == 1 ? 2 : 0); }
     static constexpr bool kSpeculative = HasQuickDirection<T>::value;
+    static constexpr bool kPairs = true;
     template <class IO>
     __device__ __forceinline__ void staged(const IO &io) const {
         this->template staged_steps<ForwardInplace>(io);
@@ -534,7 +765,16 @@ struct ForwardUpdates {
     static constexpr int kWavesPerCUMulti = 32;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     static constexpr bool kSpeculative = HasQuickDirection<T>::value;
+    static constexpr bool kPairs = true;
     T c1, c2, eps, eps_root;
+    template <class P>
+    __device__ __forceinline__ uint32_t quick_pair(const P (&in)[NIN], P (&out)[NOUT]) const {
+        const P mh = in[0] * P(c1);
+        const P vh = in[1] * P(c2);
+        uint32_t bad;
+        out[0] = adam_direction_quick(mh, vh, P(eps_root), P(eps), bad);
+        return bad;
+    }
     template <bool QUICK>
     __device__ __forceinline__ bool run(const T (&in)[NIN], T (&out)[NOUT]) const {
         const T mh = in[0] * c1;
@@ -611,7 +851,7 @@ struct BackwardUpdates {
 template <typename T>
 struct ForwardAll : AdamSteps<T> {
     static constexpr int NIN = 3, NOUT = 3, NPTR = 6;
-    static constexpr int kWavesPerCU = waves_by_type<T>(11, 10, 16, 18);  // six streams per wave: few waves fill the queues
+    static constexpr int kWavesPerCU = waves_by_type<T>(11, 10, 16, 14);  // six streams per wave: few waves fill the queues
     static constexpr int kWavesPerCUMulti = waves_by_type<T>(18, 21, 32);
     // measured: float64 6.75 against 6.55 TB/s, float16 6.69 against 6.46; float32 loses
     // (6.45 against 6.62) and bfloat16 is bound by its arithmetic
@@ -620,6 +860,7 @@ struct ForwardAll : AdamSteps<T> {
     static constexpr bool kStagedLists = false;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     static constexpr bool kSpeculative = HasQuickDirection<T>::value;
+    static constexpr bool kPairs = true;
     template <class IO>
     __device__ __forceinline__ void staged(const IO &io) const {
         this->template staged_steps<ForwardAll>(io);
@@ -758,6 +999,16 @@ struct FusedStep {
     }
 };
 
+// The 16-bit instantiations of the ops built on AdamSteps compute whole tiles pair-wise.
+template <typename T, class Op, class = void>
+struct UsesPairs {
+    static constexpr bool value = false;
+};
+template <class F, class Op>
+struct UsesPairs<R16<F>, Op, decltype((void)Op::kPairs)> {
+    static constexpr bool value = Op::kPairs;
+};
+
 // ---------------------------------------------------------------------------
 // Tile processing.  A tile is kBlock * UNROLL vectors (that * Vec<T>::N
 // elements) of one tensor; the library instantiates UNROLL = 1.
@@ -788,6 +1039,44 @@ __device__ __forceinline__ void tile_full(const Op &op, const TensorPtrs<T, Op> 
 #pragma unroll
         for (int i = 0; i < Op::NIN; ++i)
             in[i][k] = ld<NT>(reinterpret_cast<const V *>(tp.p[i]) + v0 + (size_t)k * kBlock);
+
+    if constexpr (UsesPairs<T, Op>::value && UNROLL == 1) {
+        // a 16-bit op with a pair form: two elements per step, the quick route for both
+        using P = typename PairOf<T>::type;
+        typedef uint32_t Words __attribute__((ext_vector_type(4)));
+        Words w[Op::NIN], o[Op::NOUT];
+#pragma unroll
+        for (int i = 0; i < Op::NIN; ++i) w[i] = __builtin_bit_cast(Words, in[i][0]);
+        uint32_t redo = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            P a[Op::NIN], r[Op::NOUT];
+#pragma unroll
+            for (int i = 0; i < Op::NIN; ++i) a[i] = P::from_bits(w[i][e]);
+            redo |= op.quick_pair(a, r) << (2 * e);
+#pragma unroll
+            for (int j = 0; j < Op::NOUT; ++j) o[j][e] = r[j].bits();
+        }
+        V res[Op::NOUT];
+#pragma unroll
+        for (int j = 0; j < Op::NOUT; ++j) res[j] = __builtin_bit_cast(V, o[j]);
+        if (redo != 0) {  // rare: an element the quick route could not settle
+#pragma unroll
+            for (int e = 0; e < VN; ++e)
+                if (redo & (1u << e)) {
+                    T a[Op::NIN], r[Op::NOUT];
+#pragma unroll
+                    for (int i = 0; i < Op::NIN; ++i) a[i] = Vec<T>::get(in[i][0], e);
+                    op(a, r);
+#pragma unroll
+                    for (int j = 0; j < Op::NOUT; ++j) Vec<T>::set(res[j], e, r[j]);
+                }
+        }
+#pragma unroll
+        for (int j = 0; j < Op::NOUT; ++j)
+            st<NT>(reinterpret_cast<V *>(tp.p[Op::out_slot(j)]) + v0, res[j]);
+        return;
+    }
 
     V out[Op::NOUT][UNROLL];
     static_assert(UNROLL * VN <= 32, "one redo bit per element of a lane");

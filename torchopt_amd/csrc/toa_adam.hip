@@ -84,14 +84,28 @@ static_assert(lds_for_waves(kMinWavesPerCU) <= 64 * 1024, "every served level fi
 // 8.8 us capped, 6.5 us uncapped), so such launches run without a reservation.
 constexpr size_t kOneRoundTiles = 256 * kMaxWavesPerCU;
 
+// Residency level of a staged list launch: the op's own figure where it was measured, else the
+// single-tensor level.
+template <class Op, class = void>
+struct StagedListLevel {
+    static constexpr int value = Op::kWavesPerCUStaged;
+};
+template <class Op>
+struct StagedListLevel<Op, decltype((void)Op::kWavesPerCUStagedLists)> {
+    static constexpr int value = Op::kWavesPerCUStagedLists;
+};
+template <class Op>
+constexpr int staged_list_level() {
+    return StagedListLevel<Op>::value;
+}
+
 template <class Op>
 unsigned lds_reservation(bool multi, size_t num_tiles, bool staged = false) {
     const int o = waves_override();
     if (o) return lds_for_waves(o);
     if (num_tiles <= kOneRoundTiles) return 0;
     if constexpr (IsStaged<Op>::value) {
-        // lists run the staged schedule at the single-tensor level
-        if (staged) return lds_for_waves(Op::kWavesPerCUStaged);
+        if (staged) return lds_for_waves(multi ? staged_list_level<Op>() : Op::kWavesPerCUStaged);
     }
     return lds_for_waves(multi ? Op::kWavesPerCUMulti : Op::kWavesPerCU);
 }
@@ -469,9 +483,10 @@ int launch_multi(MakeOp make_op, size_t num_tensors,
             if (mem != nullptr) {
                 const uint32_t total = (uint32_t)tiles_all;
                 const PlanView view = plan_view<Op::NPTR>(mem, seeds, total);
-                // the lookup is two scalar-cache hits, so the launch wants the residency level
-                // of the single-tensor kernel, not the list kernel's raised one
-                const unsigned lds = lds_reservation<Op>(false, total, staged);
+                // the lookup is two scalar-cache hits, so a plain launch wants the residency
+                // level of the single-tensor kernel, not the table kernel's raised one; a staged
+                // launch takes the op's level for staged lists
+                const unsigned lds = lds_reservation<Op>(staged, total, staged);
                 if (staged) {
                     if constexpr (IsStaged<Op>::value)
                         hipLaunchKernelGGL((plan_stream_kernel<T, Op, kUnroll, kNonTemporal, true>),
