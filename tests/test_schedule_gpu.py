@@ -239,3 +239,48 @@ def test_fused_step_list_takes_the_staged_schedule():
         O.fused_step(h[0], h[1], h[2], h[3], B1, B2, 1e-8, 0.0, 2, 1e-3, False, True, 0.01, True)
         for got, exp, name in zip(d, h, ('params', 'updates', 'mu', 'nu')):
             assert_bit_equal(host(got, 'f32'), exp, f'leaf {k} {name}')
+
+
+@pytest.mark.parametrize('tag', ['f32', 'f64', 'f16'])
+@pytest.mark.parametrize('schedule', [1, 2])
+@pytest.mark.parametrize('outside', ['both', 'mu only', 'none'])
+def test_backward_all_both_schedules(tag, schedule, outside):
+    """The one-pass backward equals backward_updates, autograd's additions, backward_mu and
+    backward_nu, whichever order the wave issues its memory operations in."""
+    lib = _lib.load()
+    n = BIG[tag]
+    eps, eps_root, count = (1e-8, 1e-8, 3) if tag in ('f32', 'f64') else (1e-3, 1e-4, 3)
+    g, m, v = draw(tag, n, 51)
+    d_u, d_m, d_v = draw(tag, n, 52)
+    e_mu, e_nu = O.forward_mu(g, m, B1), O.forward_nu(g, v, B2)
+    e_u = O.forward_updates(e_mu, e_nu, B1, B2, eps, eps_root, count)
+    bm, bv = O.backward_updates(d_u, e_u, e_mu, B1, B2, eps_root, count)
+    has_m, has_v = outside in ('both', 'mu only'), outside == 'both'
+    # the sums autograd forms where a gradient reaches new_mu / new_nu from outside as well
+    from torchopt_amd._C import adam_op as A
+
+    def plus(a, b):  # a + b in the element type's own arithmetic, on the GPU
+        return host(dev(a, tag) + dev(b, tag), tag)
+
+    tot_m = plus(d_m, bm) if has_m else bm
+    tot_v = plus(d_v, bv) if has_v else bv
+    gu1, gm = O.backward_mu(tot_m, B1)
+    gu2, gv = O.backward_nu(tot_v, g, B2)
+    want_du = plus(gu1, gu2)
+    t = {k: dev(a, tag) for k, a in (('du', d_u), ('nu_', e_u), ('nm', e_mu), ('g', g),
+                                     ('dm', d_m), ('dv', d_v))}
+    outs = [torch.empty_like(t['g']) for _ in range(3)]
+    lib.toa_adam_set_schedule(schedule)
+    print(f'backward_all {tag} n={n} schedule={schedule} outside gradients: {outside}', flush=True)
+    rc = lib.toa_adam_backward_all(CODE[tag], t['du'].data_ptr(), t['nu_'].data_ptr(),
+                                   t['nm'].data_ptr(), t['g'].data_ptr(),
+                                   t['dm'].data_ptr() if has_m else None,
+                                   t['dv'].data_ptr() if has_v else None, n, B1, B2, eps_root,
+                                   count, outs[0].data_ptr(), outs[1].data_ptr(),
+                                   outs[2].data_ptr(), torch.cuda.current_stream().cuda_stream)
+    lib.toa_adam_set_schedule(0)
+    assert rc == 0, lib.toa_adam_error_string(rc)
+    assert_bit_equal(host(outs[1], tag), gm, f'{tag} {outside} d(mu)')
+    assert_bit_equal(host(outs[2], tag), gv, f'{tag} {outside} d(nu)')
+    assert_bit_equal(host(outs[0], tag), want_du, f'{tag} {outside} d(updates)')
+    del A

@@ -881,15 +881,29 @@ struct BackwardAll {
                          NPTR = NIN + NOUT;
     static constexpr int kWavesPerCU = waves_by_type<T>(10, 10, 11, 14);  // seven to nine streams per wave
     static constexpr int kWavesPerCUMulti = waves_by_type<T>(14, 16, 16);
+    // staged: float32 / float64 only (the 16-bit types are bound by their arithmetic here)
+    static constexpr bool kStaged = sizeof(T) >= 4;
+    // the more streams a wave carries, the fewer waves fill the queues: nine streams 12, seven 16
+    static constexpr int kWavesPerCUStaged = HAS_DM && HAS_DV ? 12 : (HAS_DM || HAS_DV ? 14 : 16);
+    static constexpr bool kStagedLists = false;
     __device__ static constexpr int out_slot(int j) { return NIN + j; }
     T b1, b2, p1, q2;
-    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
-        const T d = in[0], u = in[1], m1 = in[2], g = in[3];
+    __device__ __forceinline__ void set_bias(T, T, T p1_, T q2_) {
+        p1 = p1_;
+        q2 = q2_;
+    }
+    // d(new_mu) and d(new_nu) arriving from the update: backward_updates
+    __device__ __forceinline__ void from_update(T d, T u, T m1, T &tot_m, T &tot_v) const {
         const T r = u / m1;
         const T den = r * p1;
         const bool zero = (m1 == 0);
-        T tot_m = zero ? T(0) : T(d * r);
-        T tot_v = zero ? T(0) : static_cast<T>(-d * u * den * 0.5 * q2 * den);
+        tot_m = zero ? T(0) : T(d * r);
+        tot_v = zero ? T(0) : static_cast<T>(-d * u * den * 0.5 * q2 * den);
+    }
+    __device__ __forceinline__ void operator()(const T (&in)[NIN], T (&out)[NOUT]) const {
+        const T g = in[3];
+        T tot_m, tot_v;
+        from_update(in[0], in[1], in[2], tot_m, tot_v);
         if constexpr (HAS_DM) tot_m = in[4] + tot_m;
         if constexpr (HAS_DV) tot_v = in[HAS_DM ? 5 : 4] + tot_v;
         const T du_from_mu = (1 - b1) * tot_m;
@@ -897,6 +911,44 @@ struct BackwardAll {
         out[0] = du_from_mu + du_from_nu;
         out[1] = b1 * tot_m;
         out[2] = b2 * tot_v;
+    }
+    // load d(new_updates), new_updates | load new_mu [, d(new_mu)] | store d(mu),
+    // load updates [, d(new_nu)] | store d(nu), store d(updates)
+    template <class IO>
+    __device__ __forceinline__ void staged(const IO &io) const {
+        using V = typename Vec<T>::type;
+        constexpr int VN = Vec<T>::N;
+        const V d = io.load(0);
+        const V u = io.load(1);
+        io.wait();
+        const V m1 = io.load(2);
+        V dm, dv;
+        if constexpr (HAS_DM) dm = io.load(4);
+        io.wait();
+        T tot_m[VN], tot_v[VN];
+        V dmu;
+#pragma unroll
+        for (int e = 0; e < VN; ++e) {
+            from_update(Vec<T>::get(d, e), Vec<T>::get(u, e), Vec<T>::get(m1, e), tot_m[e],
+                        tot_v[e]);
+            if constexpr (HAS_DM) tot_m[e] = Vec<T>::get(dm, e) + tot_m[e];
+            Vec<T>::set(dmu, e, b1 * tot_m[e]);
+        }
+        io.store(out_slot(1), dmu);
+        const V g = io.load(3);
+        if constexpr (HAS_DV) dv = io.load(HAS_DM ? 5 : 4);
+        io.wait();
+        V dnu, du;
+#pragma unroll
+        for (int e = 0; e < VN; ++e) {
+            if constexpr (HAS_DV) tot_v[e] = Vec<T>::get(dv, e) + tot_v[e];
+            Vec<T>::set(dnu, e, b2 * tot_v[e]);
+            const T du_from_mu = (1 - b1) * tot_m[e];
+            const T du_from_nu = 2 * (1 - b2) * Vec<T>::get(g, e) * tot_v[e];
+            Vec<T>::set(du, e, du_from_mu + du_from_nu);
+        }
+        io.store(out_slot(2), dnu);
+        io.store(out_slot(0), du);
     }
 };
 
