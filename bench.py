@@ -114,12 +114,18 @@ CONFIGS = {
             dtype='f32', shapes=gpt2_medium_shapes(), eps_root=0.0, count=1, fused_step=True),
     6: dict(name='config6: fused forward_ in place, 268 435 456 float16 elements (arithmetic of '
                  'the reference CPU op on at::Half: every operation rounded to 16 bits), '
-                 'eps=1e-3, count=1000, gradients from eight arrays in rotation',
+                 'eps=1e-3, count=1000, a fresh N(0,1) gradient array every step',
             dtype='f16', n=1 << 28, eps=1e-3, eps_root=0.0, count=1000, fresh_gradients=True),
     7: dict(name='config7: fused forward_ in place, 268 435 456 bfloat16 elements (arithmetic of '
-                 'the reference CPU op on at::BFloat16), eps=1e-3, count=1000, gradients from eight '
-                 'arrays in rotation',
+                 'the reference CPU op on at::BFloat16), eps=1e-3, count=1000, a fresh N(0,1) '
+                 'gradient array every step',
             dtype='bf16', n=1 << 28, eps=1e-3, eps_root=0.0, count=1000, fresh_gradients=True),
+    8: dict(name='config8: multi-tensor forward_ in place over 64 float32 leaves of 4096 x 1024 '
+                 '(16 MiB each, the GPT-2-medium fc weight), the gradient, mu and nu lists each '
+                 'contiguous, so the three arrays of every leaf lie exactly 1 GiB = 64 x 16 MiB '
+                 'apart and meet in the same DRAM banks; count=1',
+            dtype='f32', shapes=[(4096, 1024)] * 64, eps_root=0.0, count=1,
+            lists_contiguous=True),
 }
 ESIZE = {'f32': 4, 'f64': 8, 'f16': 2, 'bf16': 2}
 
@@ -351,22 +357,60 @@ def run_gpu(cfg_id, steps, warmup):
         extra_arrays = 1 if cfg.get('fused_step') else 0
         host = [host_state(cfg_id, k, n, cfg['dtype'], extra=extra_arrays)
                 for k, n in enumerate(sizes)]
-        us = [h[0].cuda() for h in host]
-        ms = [h[1].cuda() for h in host]
-        vs = [h[2].cuda() for h in host]
-        tensors = list(zip(us, ms, vs))
         num = len(sizes)
-        pu = (ctypes.c_void_p * num)(*[t[0].data_ptr() for t in tensors])
-        pm = (ctypes.c_void_p * num)(*[t[1].data_ptr() for t in tensors])
-        pv = (ctypes.c_void_p * num)(*[t[2].data_ptr() for t in tensors])
         ns = (ctypes.c_size_t * num)(*sizes)
-
-        def step():
-            rc = lib.toa_adam_forward_inplace_multi(code, num, pu, pm, pv, ns, B1, B2, EPS,
-                                                    eps_root, None, count, sptr)
-            if rc:
-                raise RuntimeError(lib.toa_adam_error_string(rc).decode())
         extra = {'tensors': num}
+
+        def carve(gap_elems):
+            """The three lists carved from one allocation, each list contiguous, the lists
+            `gap_elems` elements further apart than their own length."""
+            arena = torch.empty(3 * total + 2 * gap_elems, device='cuda', dtype=dtype)
+            lists = []
+            for j in range(3):
+                at, views = j * (total + gap_elems), []
+                for h, n in zip(host, sizes):
+                    views.append(arena[at:at + n])
+                    views[-1].copy_(h[j])
+                    at += n
+                lists.append(views)
+            return lists
+
+        def list_step(us_, ms_, vs_):
+            a, b, c = ((ctypes.c_void_p * num)(*[t.data_ptr() for t in ts])
+                       for ts in (us_, ms_, vs_))
+
+            def one():
+                rc = lib.toa_adam_forward_inplace_multi(code, num, a, b, c, ns, B1, B2, EPS,
+                                                        eps_root, None, count, sptr)
+                if rc:
+                    raise RuntimeError(lib.toa_adam_error_string(rc).decode())
+            return one
+
+        if cfg.get('lists_contiguous'):
+            # beside the timed layout: the same lists 3 MiB further apart, where no leaf's arrays
+            # meet in the same banks -- what the colliding placement costs
+            apart = carve((3 << 20) // esize)
+            other = list_step(*apart)
+            for _ in range(5):
+                other()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(stream)
+            for _ in range(20):
+                other()
+            b.record(stream)
+            torch.cuda.synchronize()
+            apart_ms = a.elapsed_time(b) / 20
+            extra['lists_3_mib_further_apart'] = {
+                'ms_per_step': round(apart_ms, 5),
+                'GB/s': round(bytes_per_elem * total / apart_ms / 1e6, 1)}
+            del apart, other
+            us, ms, vs = carve(0)
+        else:
+            us = [h[0].cuda() for h in host]
+            ms = [h[1].cuda() for h in host]
+            vs = [h[2].cuda() for h in host]
+        step = list_step(us, ms, vs)
+        pu, pm, pv = ((ctypes.c_void_p * num)(*[t.data_ptr() for t in ts]) for ts in (us, ms, vs))
         if cfg.get('fused_step'):
             ps = [h[3].cuda() for h in host]
             pp = (ctypes.c_void_p * num)(*[t.data_ptr() for t in ps])
@@ -401,15 +445,20 @@ def run_gpu(cfg_id, steps, warmup):
 
         extra = {}
         if cfg.get('fresh_gradients'):
-            # A training loop hands the step a new gradient every time; re-applying the step to
-            # its own output instead drives every element towards one fixed point, which no real
-            # run does and which the 16-bit kernels' data-dependent quick route would be timed
-            # on.  So the steps draw their gradients from eight arrays in rotation (a training loop
-            # reuses its gradient buffers too: pages and TLB entries are warm, the values new).
+            # A training loop hands the step a new gradient every time.  The step overwrites its
+            # gradient array with the update, so an array used twice feeds the operator its own
+            # output: over a few dozen steps that drifts the data away from anything a real run
+            # holds, and the 16-bit kernels' data-dependent quick route with it (measured: the same
+            # loop slows by up to 20 % after 150 steps over eight arrays in rotation, and holds
+            # its speed when every step reads a fresh array).  So every step of this run --
+            # warm-up, timed region and the per-step spread pass -- gets an array of its own,
+            # drawn N(0, 1) before the clock starts; only a run longer than kMaxGradientArrays
+            # steps wraps around.
+            kMaxGradientArrays = 160  # 80 GiB of 16-bit gradients at most
             g = torch.Generator(device='cuda')
             g.manual_seed(1000 * cfg_id + 1)
             fresh = [torch.randn(total, device='cuda', generator=g).to(dtype)
-                     for _ in range(min(steps + warmup, 8))]
+                     for _ in range(min(steps + warmup + min(steps, 20), kMaxGradientArrays))]
             ptrs, turn = [t.data_ptr() for t in fresh], [0]
             extra['gradient_arrays'] = len(fresh)
 

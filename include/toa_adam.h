@@ -83,7 +83,8 @@ TOA_API int toa_adam_set_waves_per_cu(int waves);
 TOA_API int toa_adam_set_schedule(int schedule);
 
 /* Lists longer than one kernel-argument table (96 tensors for ops with three pointer slots, 80
- * with four, 64 with five, fewer beyond) run as ONE launch over a device-resident table, a
+ * with four, 64 with five, fewer beyond), and lists of 256 MiB or more per array whatever their
+ * length, run as ONE launch over a device-resident table, a
  * "plan": one 96-byte record per tensor, written by small kernels that carry the records in
  * their arguments and cached per (device, stream, list) in memory the library allocates (at most
  * 4 plans per stream, 64 per process), with a coarse index from tiles to records in the launch's

@@ -231,6 +231,7 @@ int launch_single(const Op &op, T *const (&ptrs)[Op::NPTR], size_t n, void *stre
 // 0 = plans for lists that need more than one kernel-argument table (the default), 1 = never
 // (several launches instead), 2 = for every list (so that small inputs can exercise the path).
 std::atomic<int> g_plan_mode{0};
+constexpr uint64_t kPlanFromTiles = 1u << 18;  // 256 MiB of 1 KiB tiles per array
 
 constexpr size_t kPlanSlotsPerStream = 4;         // cached plans a stream may hold
 constexpr size_t kPlanSlotsTotal = 64;            // and the process as a whole
@@ -453,8 +454,15 @@ int launch_multi(MakeOp make_op, size_t num_tensors,
                 tiles_all += (n[k] + tile - 1) / tile;
             }
         if (live == 0) continue;
+        // Long lists cannot do without a plan; lists that stream 256 MiB or more per array gain
+        // from one whatever their length (the plan's lookup is two scalar-cache hits where the
+        // table's is a search through kernel arguments, whose latency a bandwidth-bound wave
+        // feels: 64 leaves of 16 MiB run 1 to 3 % faster), and its one small fill launch per new
+        // list is lost in a launch of that size.  Short lists of small tensors keep the tables.
         const bool wants_plan =
-            arena != nullptr || (plan_mode != 1 && (plan_mode == 2 || live > (size_t)Table::MAX));
+            arena != nullptr ||
+            (plan_mode != 1 &&
+             (plan_mode == 2 || live > (size_t)Table::MAX || tiles_all >= kPlanFromTiles));
         if (wants_plan && tiles_all < kNoTile && live < kNoTile) {
             seeds.clear();
             seeds.reserve(live);
