@@ -649,9 +649,20 @@ def run_ceiling(array_bytes=1 << 30, reps=20):
     del arrays[3:]
     arena = torch.randn(3 * (array_bytes // 4), device='cuda')
     a0, a1, a2 = (t.data_ptr() for t in arrays)
-    layouts = (('three separate arrays', (a0, a1, a2), 0),
+    layouts = [('three separate arrays', (a0, a1, a2), 0),
                ('one arena, arrays interleaved in 64 KiB pieces', (arena.data_ptr(), None, None),
-                64 << 10))
+                64 << 10)]
+    # ... and on placements inside one allocation that differ only in the distances between the
+    # arrays: the rate is a repeatable function of those distances (how the three streams fall on
+    # DRAM channels and banks), so a ceiling holds for a placement, like the operator's own rate
+    n_elems = array_bytes // 4
+    wide = torch.randn(3 * n_elems + (8 << 20) // 4, device='cuda')
+    phases = ((0, 0), (0, 8), (8, 8), (4, 4), (2048, 4096))
+    for a_kib, b_kib in phases:
+        base = wide.data_ptr()
+        layouts.append((f'one allocation, mu at 1 GiB + {a_kib} KiB, nu at 2 GiB + {b_kib} KiB',
+                        (base, base + array_bytes + (a_kib << 10),
+                         base + 2 * array_bytes + (b_kib << 10)), 0))
     family = {}
     for layout, ptrs3, piece in layouts:
         rows, top = {}, (0.0, None)
@@ -674,6 +685,31 @@ def run_ceiling(array_bytes=1 << 30, reps=20):
                 top = (best[0], name)
         family[layout] = {'shapes': rows, 'best_shape': top[1], 'best_GB/s': round(top[0], 1),
                           'best_frac_of_peak': round(top[0] / HBM_PEAK_GBS, 4)}
+    # The operator itself (float32 forward_ in place, library defaults) on the same placements
+    from torchopt_amd import _lib
+    lib = _lib.load()
+    operator = {}
+    for layout, ptrs3, piece in layouts:
+        if piece:
+            continue
+        views = [torch.empty(0)] * 3
+        if layout == 'three separate arrays':
+            views = arrays[:3]
+        else:
+            views = [wide[(p - wide.data_ptr()) // 4:(p - wide.data_ptr()) // 4 + n_elems]
+                     for p in ptrs3]
+
+        def launch():
+            rc = lib.toa_adam_forward_inplace(_lib.TOA_F32, ptrs3[0], ptrs3[1], ptrs3[2], n_elems,
+                                              B1, B2, EPS, 0.0, 1000, stream.cuda_stream)
+            if rc:
+                raise RuntimeError(lib.toa_adam_error_string(rc).decode())
+        views[0].normal_()
+        views[1].normal_(0, 0.1)
+        views[2].normal_(0, 0.01).abs_()
+        gbs = 6 * array_bytes / (timed(launch) * 1e-3) / 1e9
+        operator[layout] = {'GB/s': round(gbs, 1), 'frac_of_peak': round(gbs / HBM_PEAK_GBS, 4),
+                            'of_the_probe_best_here': round(gbs / family[layout]['best_GB/s'], 4)}
     # The same pass (staged shape, three separate arrays) over other data: the rate depends on the
     # bits that cross the memory interface, so a ceiling holds for the data it was taken on.
     by_data = {}
@@ -693,6 +729,7 @@ def run_ceiling(array_bytes=1 << 30, reps=20):
             'array_bytes': array_bytes, 'launches_timed': reps,
             'device': torch.cuda.get_device_name(0), 'ceilings': out,
             'three_arrays_read_and_written_back': family,
+            'operator_forward_inplace_f32_on_the_same_placements': operator,
             'staged_shape_by_data_GB/s': by_data}
 
 

@@ -879,7 +879,7 @@ template <typename T, bool HAS_DM, bool HAS_DV>
 struct BackwardAll {
     static constexpr int NIN = 4 + (HAS_DM ? 1 : 0) + (HAS_DV ? 1 : 0), NOUT = 3,
                          NPTR = NIN + NOUT;
-    static constexpr int kWavesPerCU = waves_by_type<T>(10, 10, 11, 14);  // seven to nine streams per wave
+    static constexpr int kWavesPerCU = waves_by_type<T>(10, 10, 12, 12);  // seven to nine streams per wave
     static constexpr int kWavesPerCUMulti = waves_by_type<T>(14, 16, 16);
     // staged: float32 / float64 only (the 16-bit types are bound by their arithmetic here)
     static constexpr bool kStaged = sizeof(T) >= 4;
