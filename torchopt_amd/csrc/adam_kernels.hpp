@@ -716,9 +716,10 @@ struct ForwardInplace : AdamSteps<T> {
     static constexpr int kWavesPerCUStaged = waves_by_type<T>(18, 18, 21, 21);
     // A float32 / float64 list gains nothing from the staged schedule (6.5-6.6 TB/s either way
     // on the GPT-2-medium list) unless its arrays collide in DRAM, so such lists are staged only
-    // then; the 16-bit lists gain 5-10 % from it at full residency.
+    // then; the 16-bit lists gain 1-2 % from it at 25 waves per CU (measured after 100 launches of
+    // the same kind: the first 40-50 launches of a 16-bit kernel run up to 6 % slower).
     static constexpr bool kStagedLists = sizeof(T) == 2;
-    static constexpr int kWavesPerCUStagedLists = waves_by_type<T>(18, 18, 32, 32);
+    static constexpr int kWavesPerCUStagedLists = waves_by_type<T>(18, 18, 25, 25);
     // outputs are produced as (mu', nu', updates') and stored in that order
     __device__ static constexpr int out_slot(int j) { return j == 0 ? 1 : (j == 1 ? 2 : 0); }
     static constexpr bool kSpeculative = HasQuickDirection<T>::value;
