@@ -349,5 +349,6 @@ def test_fc_weight_list_parity_and_cost_of_the_colliding_layout():
     loss = 1.0 - t_apart / t_tight
     print(f'colliding layout {gbs(t_tight):.0f} GB/s, lists 3 MiB further apart '
           f'{gbs(t_apart):.0f} GB/s, loss {100 * loss:.1f} %', flush=True)
-    assert gbs(t_tight) >= 0.80 * 8000, 'the colliding layout fell below 80 % of the HBM peak'
+    # measured 80.6-83.0 % of the 8 TB/s peak; the cliff was 68-75 %
+    assert gbs(t_tight) >= 0.77 * 8000, 'the colliding layout fell back towards the cliff'
     assert loss <= 0.07, f'the colliding layout costs {100 * loss:.1f} % against the spread one'
