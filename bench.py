@@ -608,6 +608,8 @@ INPLACE3_SHAPES = (
     ('four tiles per wave, all loads before the first store', 6, (8, 6, 5, 4, 3, 2)),
     ('persistent grid striding over the tiles, next tile loaded before the current one is '
      'stored', 7, (16, 12, 10, 8, 6, 4)),
+    ('staged, two adjacent tiles per wave, one after the other', 8, (32, 25, 21, 18, 16, 14)),
+    ('staged, four adjacent tiles per wave, one after the other', 9, (32, 25, 21, 18, 16, 14)),
 )
 
 

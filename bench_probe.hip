@@ -107,6 +107,25 @@ __global__ __launch_bounds__(kWave) void shape_staged(Three t) {
     PROBE_ST(c, t.at(0, i));
 }
 
+// SEQ tiles per wave, one after the other, each with the staged order (a wave owns SEQ adjacent
+// tiles: what a list kernel would do to spread the cost of finding its tensor over more bytes)
+template <int SEQ>
+__global__ __launch_bounds__(kWave) void shape_staged_seq(Three t) {
+#pragma unroll 1
+    for (int k = 0; k < SEQ; ++k) {
+        const size_t i = ((size_t)blockIdx.x * SEQ + k) * kWave + threadIdx.x;
+        const f4 a = PROBE_LD(t.at(0, i));
+        PROBE_WAIT();
+        const f4 b = PROBE_LD(t.at(1, i));
+        PROBE_WAIT();
+        PROBE_ST(a, t.at(1, i));
+        const f4 c = PROBE_LD(t.at(2, i));
+        PROBE_WAIT();
+        PROBE_ST(b, t.at(2, i));
+        PROBE_ST(c, t.at(0, i));
+    }
+}
+
 // a wait after every load and every store
 __global__ __launch_bounds__(kWave) void shape_serial(Three t) {
     const size_t i = (size_t)blockIdx.x * kWave + threadIdx.x;
@@ -180,7 +199,9 @@ enum {
     PROBE_TILES2 = 5,      // 2 tiles per wave, loads first
     PROBE_TILES4 = 6,      // 4 tiles per wave, loads first
     PROBE_GRIDSTRIDE = 7,  // persistent grid of `param` workgroups per CU x 256 CUs, prefetching
-    PROBE_SHAPES = 8
+    PROBE_STAGED_SEQ2 = 8,  // staged, two adjacent tiles per wave, one after the other
+    PROBE_STAGED_SEQ4 = 9,  // staged, four adjacent tiles per wave, one after the other
+    PROBE_SHAPES = 10
 };
 
 // Three arrays of `bytes` bytes each (a multiple of 4 KiB x the shape's tiles per workgroup)
@@ -227,6 +248,12 @@ extern "C" __attribute__((visibility("default"))) int bench_probe_inplace3(
             if (param < 1 || param > 32) return -2;
             hipLaunchKernelGGL(shape_gridstride, dim3(256u * (unsigned)param), dim3(64), 0, s, t,
                                (unsigned)tiles);
+            break;
+        case PROBE_STAGED_SEQ2:
+            hipLaunchKernelGGL((shape_staged_seq<2>), grid(2), dim3(64), lds_bytes, s, t);
+            break;
+        case PROBE_STAGED_SEQ4:
+            hipLaunchKernelGGL((shape_staged_seq<4>), grid(4), dim3(64), lds_bytes, s, t);
             break;
         default:
             return -1;

@@ -285,17 +285,42 @@ struct Vec<R16<F>> {
     __device__ static void set(type &v, int e, R16<F> x) { v[e] = x.bits; }
 };
 
+// Every array these kernels touch is device memory (the entry points' contract); a pointer that
+// reached the kernel through memory -- a plan's record -- carries no address space the compiler
+// could see, and would be served by FLAT instructions (aperture checks, both memory counters).
+// All accesses therefore go through the global address space explicitly.
+template <typename V>
+__device__ __forceinline__ auto as_global(V *p) {
+    return (V __attribute__((address_space(1))) *)p;
+}
+// one element (the unaligned and ragged paths)
+template <typename T>
+__device__ __forceinline__ T ld_elem(const T *p, size_t i) {
+    return as_global(p)[i];
+}
+template <typename T>
+__device__ __forceinline__ void st_elem(T *p, size_t i, T v) {
+    as_global(p)[i] = v;
+}
+template <class F>
+__device__ __forceinline__ R16<F> ld_elem(const R16<F> *p, size_t i) {
+    return R16<F>::from_bits(as_global(reinterpret_cast<const uint16_t *>(p))[i]);
+}
+template <class F>
+__device__ __forceinline__ void st_elem(R16<F> *p, size_t i, R16<F> v) {
+    as_global(reinterpret_cast<uint16_t *>(p))[i] = v.bits;
+}
 template <bool NT, typename V>
 __device__ __forceinline__ V ld(const V *p) {
-    if constexpr (NT) return __builtin_nontemporal_load(p);
-    return *p;
+    if constexpr (NT) return __builtin_nontemporal_load(as_global(p));
+    return *as_global(p);
 }
 template <bool NT, typename V>
 __device__ __forceinline__ void st(V *p, V v) {
     if constexpr (NT)
-        __builtin_nontemporal_store(v, p);
+        __builtin_nontemporal_store(v, as_global(p));
     else
-        *p = v;
+        *as_global(p) = v;
 }
 
 // Waits until every memory operation this wave has issued is complete; the compiler may not move
@@ -561,8 +586,12 @@ constexpr int waves_by_type(int wide, int half, int bfloat) {
 // The three steps of one Adam update as the reference writes them (adam_op_impl_cpu.cpp:47-61):
 // the two moments, then the step direction from the bias-corrected moments.  Shared by the
 // in-place step and the one-pass differentiable forward.
+// (Ops are aligned to 8 bytes whatever their element type: a kernel argument of 2-byte alignment --
+// an op over a 16-bit type -- would be fetched with a VECTOR load, whose latency the list kernels
+// pay in full before they can even look up their tensor; aligned, it comes through the scalar
+// unit like every other argument.)
 template <typename T>
-struct AdamSteps {
+struct alignas(8) AdamSteps {
     T b1, b2, c1, c2, eps, eps_root;
     __device__ __forceinline__ void set_bias(T c1_, T c2_, T, T) {
         c1 = c1_;
@@ -732,7 +761,7 @@ struct ForwardInplace : AdamSteps<T> {
 
 // adam_op_impl_cpu.cpp:103-108.  Slots: 0 updates, 1 mu, 2 mu_out.
 template <typename T>
-struct ForwardMu {
+struct alignas(8) ForwardMu {
     static constexpr int NIN = 2, NOUT = 1, NPTR = 3;
     static constexpr int kWavesPerCU = 25;
     static constexpr int kWavesPerCUMulti = 32;
@@ -745,7 +774,7 @@ struct ForwardMu {
 
 // adam_op_impl_cpu.cpp:137-143.  Slots: 0 updates, 1 nu, 2 nu_out.
 template <typename T>
-struct ForwardNu {
+struct alignas(8) ForwardNu {
     static constexpr int NIN = 2, NOUT = 1, NPTR = 3;
     static constexpr int kWavesPerCU = waves_by_type<T>(21, 21, 32, 32);
     static constexpr int kWavesPerCUMulti = 32;
@@ -759,7 +788,7 @@ struct ForwardNu {
 
 // adam_op_impl_cpu.cpp:175-181.  Slots: 0 new_mu, 1 new_nu, 2 updates_out.
 template <typename T>
-struct ForwardUpdates {
+struct alignas(8) ForwardUpdates {
     static constexpr int NIN = 2, NOUT = 1, NPTR = 3;
     // root and quotient: the 16-bit types need every wave to hide the ALU time
     static constexpr int kWavesPerCU = waves_by_type<T>(21, 18, 32, 32);
@@ -797,7 +826,7 @@ struct ForwardUpdates {
 
 // adam_op_impl_cpu.cpp:220-226.  Slots: 0 dmu, 1 dupdates_out, 2 dmu_out.
 template <typename T>
-struct BackwardMu {
+struct alignas(8) BackwardMu {
     static constexpr int NIN = 1, NOUT = 2, NPTR = 3;
     static constexpr int kWavesPerCU = 18;
     static constexpr int kWavesPerCUMulti = 25;
@@ -811,7 +840,7 @@ struct BackwardMu {
 
 // adam_op_impl_cpu.cpp:257-264.  Slots: 0 dnu, 1 updates, 2 dupdates_out, 3 dnu_out.
 template <typename T>
-struct BackwardNu {
+struct alignas(8) BackwardNu {
     static constexpr int NIN = 2, NOUT = 2, NPTR = 4;
     static constexpr int kWavesPerCU = 16;
     static constexpr int kWavesPerCUMulti = 25;
@@ -826,7 +855,7 @@ struct BackwardNu {
 // adam_op_impl_cpu.cpp:298-316.  Slots: 0 dupdates, 1 updates, 2 new_mu,
 // 3 dnew_mu_out, 4 dnew_nu_out.  p1 = 1 - b1^count, q2 = 1/(1 - b2^count + eps_root).
 template <typename T>
-struct BackwardUpdates {
+struct alignas(8) BackwardUpdates {
     static constexpr int NIN = 3, NOUT = 2, NPTR = 5;
     static constexpr int kWavesPerCU = waves_by_type<T>(18, 12, 16, 16);
     static constexpr int kWavesPerCUMulti = 25;
@@ -877,7 +906,7 @@ struct ForwardAll : AdamSteps<T> {
 // Slots: 0 d(new_updates), 1 new_updates, 2 new_mu, 3 updates, [d(new_mu)], [d(new_nu)],
 // then outputs d(updates), d(mu), d(nu).
 template <typename T, bool HAS_DM, bool HAS_DV>
-struct BackwardAll {
+struct alignas(8) BackwardAll {
     static constexpr int NIN = 4 + (HAS_DM ? 1 : 0) + (HAS_DV ? 1 : 0), NOUT = 3,
                          NPTR = NIN + NOUT;
     static constexpr int kWavesPerCU = waves_by_type<T>(10, 10, 12, 12);  // seven to nine streams per wave
@@ -974,7 +1003,7 @@ __device__ __forceinline__ float toa_fma(float a, float b, float c) { return __b
 __device__ __forceinline__ double toa_fma(double a, double b, double c) { return __builtin_fma(a, b, c); }
 
 template <typename T, bool WRITE_UPDATES>
-struct FusedStep {
+struct alignas(8) FusedStep {
     static constexpr int NIN = 4, NOUT = WRITE_UPDATES ? 4 : 3, NPTR = 4;
     static constexpr int kWavesPerCU = waves_by_type<T>(12, 10, 12, 12);
     static constexpr int kWavesPerCUMulti = 16;
@@ -1199,7 +1228,8 @@ __device__ __forceinline__ void tile_partial(const Op &op, const TensorPtrs<T, O
     for (uint32_t v = threadIdx.x; v < nvec; v += kBlock) {
         V in[Op::NIN], out[Op::NOUT];
 #pragma unroll
-        for (int i = 0; i < Op::NIN; ++i) in[i] = reinterpret_cast<const V *>(tp.p[i])[vbase + v];
+        for (int i = 0; i < Op::NIN; ++i)
+            in[i] = as_global(reinterpret_cast<const V *>(tp.p[i]))[vbase + v];
 #pragma unroll
         for (int e = 0; e < VN; ++e) {
             T a[Op::NIN], r[Op::NOUT];
@@ -1211,7 +1241,7 @@ __device__ __forceinline__ void tile_partial(const Op &op, const TensorPtrs<T, O
         }
 #pragma unroll
         for (int j = 0; j < Op::NOUT; ++j)
-            reinterpret_cast<V *>(tp.p[Op::out_slot(j)])[vbase + v] = out[j];
+            as_global(reinterpret_cast<V *>(tp.p[Op::out_slot(j)]))[vbase + v] = out[j];
     }
     // the last rem % VN elements, one lane each
     const uint32_t done = nvec * VN;
@@ -1219,10 +1249,10 @@ __device__ __forceinline__ void tile_partial(const Op &op, const TensorPtrs<T, O
         const size_t i0 = base + done + threadIdx.x;
         T a[Op::NIN], r[Op::NOUT];
 #pragma unroll
-        for (int i = 0; i < Op::NIN; ++i) a[i] = tp.p[i][i0];
+        for (int i = 0; i < Op::NIN; ++i) a[i] = ld_elem(tp.p[i], i0);
         op(a, r);
 #pragma unroll
-        for (int j = 0; j < Op::NOUT; ++j) tp.p[Op::out_slot(j)][i0] = r[j];
+        for (int j = 0; j < Op::NOUT; ++j) st_elem(tp.p[Op::out_slot(j)], i0, r[j]);
     }
 }
 
@@ -1239,7 +1269,7 @@ __device__ __forceinline__ void tile_unaligned(const Op &op, const TensorPtrs<T,
             const uint32_t e = e0 + s * kBlock + threadIdx.x;
             if (e < cnt) {
 #pragma unroll
-                for (int i = 0; i < Op::NIN; ++i) a[s][i] = tp.p[i][base + e];
+                for (int i = 0; i < Op::NIN; ++i) a[s][i] = ld_elem(tp.p[i], base + e);
             }
         }
 #pragma unroll
@@ -1249,7 +1279,7 @@ __device__ __forceinline__ void tile_unaligned(const Op &op, const TensorPtrs<T,
                 T r[Op::NOUT];
                 op(a[s], r);
 #pragma unroll
-                for (int j = 0; j < Op::NOUT; ++j) tp.p[Op::out_slot(j)][base + e] = r[j];
+                for (int j = 0; j < Op::NOUT; ++j) st_elem(tp.p[Op::out_slot(j)], base + e, r[j]);
             }
         }
     }
@@ -1469,8 +1499,17 @@ __device__ __forceinline__ PlanRec load_record(const PlanRec *at) {
 template <typename T, class Op, int UNROLL, bool NT, bool STAGED = false>
 __global__ __launch_bounds__(kBlock) void plan_stream_kernel(const Op op, const PlanView plan) {
     const Op live = live_op(op);
-    for (uint32_t tile = blockIdx.x; tile < plan.total; tile += gridDim.x) {
+    // The host launches at most plan.total workgroups, so the first tile needs no bounds check:
+    // a wave's first dependent fetch is its cell, not the total.
+    uint32_t tile = blockIdx.x;
+    do {
         PlanRec rec = load_record(plan.recs + plan.cell[tile >> plan.shift]);
+        // All twelve words of the record are fetched now, in one go (three 32-byte scalar loads
+        // in flight together): left alone, the compiler fetches the four words the walk below
+        // tests, waits, and only then fetches the pointers -- one more round trip to the scalar
+        // cache in every wave's prologue.
+#pragma unroll
+        for (int i = 0; i < kPlanSlots; ++i) asm volatile("" : "+s"(rec.p[i]));
         // a tensor boundary lies between the cell's first tile and this one: walk on (never
         // past the last record)
         while (tile >= rec.next_first && rec.index + 1 < plan.num)
@@ -1481,7 +1520,8 @@ __global__ __launch_bounds__(kBlock) void plan_stream_kernel(const Op op, const 
         const bool aligned = all_aligned16<T, Op>(tp);
         process_tile<T, Op, UNROLL, NT, STAGED>(live, tp, (size_t)rec.n, (size_t)(tile - rec.first),
                                                 aligned);
-    }
+        tile += gridDim.x;
+    } while (tile < plan.total);
 }
 
 // count <- count + (count != INT64_MAX): the reference's inc_count
