@@ -757,6 +757,64 @@ def run_ceiling(array_bytes=1 << 30, reps=20):
             'staged_shape_by_data_GB/s': by_data}
 
 
+def run_placements(reps=10):
+    """The operator (float32 forward_ in place, 2^28 elements, library defaults) over placements of
+    its three arrays inside ONE allocation: mu at 1 GiB + a, nu at 2 GiB + b for a <= b (so the
+    arrays stay disjoint) from a ladder of distances between 0 and 4 MiB.  The rate depends on how
+    the three read and three write streams fall on DRAM channels and banks; this is the table of
+    that dependence."""
+    import torch
+
+    from torchopt_amd import _lib
+
+    lib = _lib.load()
+    stream = torch.cuda.current_stream()
+    n = 1 << 28
+    ladder = (0, 1, 2, 3, 4, 5, 6, 7, 8, 12, 16, 24, 32, 64, 128, 256, 512, 1024, 2048, 4096)  # KiB
+    arena = torch.empty(3 * n + (8 << 20) // 4, device='cuda')
+    preheat(torch)
+    grid, cells = {}, []
+    for a_kib in ladder:
+        row = {}
+        for b_kib in ladder:
+            if b_kib < a_kib:
+                continue
+            u = arena[0:n]
+            mu = arena[n + a_kib * 256:2 * n + a_kib * 256]
+            nu = arena[2 * n + b_kib * 256:3 * n + b_kib * 256]
+            u.normal_()
+            mu.normal_(0, 0.1)
+            nu.normal_(0, 0.01).abs_()
+            ptrs = (u.data_ptr(), mu.data_ptr(), nu.data_ptr())
+
+            def launch():
+                rc = lib.toa_adam_forward_inplace(_lib.TOA_F32, *ptrs, n, B1, B2, EPS, 0.0, 1000,
+                                                  stream.cuda_stream)
+                if rc:
+                    raise RuntimeError(lib.toa_adam_error_string(rc).decode())
+            for _ in range(2):
+                launch()
+            ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            ev0.record(stream)
+            for _ in range(reps):
+                launch()
+            ev1.record(stream)
+            torch.cuda.synchronize()
+            gbs = 24 * n / (ev0.elapsed_time(ev1) / reps) / 1e6
+            row[f'nu +{b_kib} KiB'] = round(gbs)
+            cells.append(gbs)
+        grid[f'mu +{a_kib} KiB'] = row
+    cells.sort()
+    return {'metric': 'forward_inplace_f32_by_placement', 'unit': 'GB/s', 'peak': HBM_PEAK_GBS,
+            'elements': n, 'placements': len(cells), 'launches_timed': reps,
+            'min': round(cells[0], 1), 'median': round(cells[len(cells) // 2], 1),
+            'max': round(cells[-1], 1),
+            'min_frac': round(cells[0] / HBM_PEAK_GBS, 4),
+            'median_frac': round(cells[len(cells) // 2] / HBM_PEAK_GBS, 4),
+            'max_frac': round(cells[-1] / HBM_PEAK_GBS, 4),
+            'device': torch.cuda.get_device_name(0), 'GB/s_by_placement': grid}
+
+
 # ----------------------------------------------------------------------------- CPU baseline
 
 
@@ -1078,6 +1136,10 @@ def main(argv=None):
     ap.add_argument('--ceiling', action='store_true',
                     help='measure the streaming ceilings of this machine (probe kernels with '
                          'the operator\'s launch shape) instead of the operator')
+    ap.add_argument('--placements', action='store_true',
+                    help='time the operator over 210 placements of its three arrays inside one '
+                         'allocation instead of the benchmark (the rate depends on the '
+                         'distances between the arrays)')
     args = ap.parse_args(argv)
 
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
@@ -1088,6 +1150,9 @@ def main(argv=None):
 
     if args.ceiling:
         print(json.dumps(run_ceiling()), flush=True)
+        return 0
+    if args.placements:
+        print(json.dumps(run_placements()), flush=True)
         return 0
 
     host_cores()  # before torch (and with it the OpenMP runtime) loads
