@@ -757,7 +757,7 @@ def run_ceiling(array_bytes=1 << 30, reps=20):
             'staged_shape_by_data_GB/s': by_data}
 
 
-def run_placements(reps=10):
+def run_placements(reps=10, n=1 << 28, ladder=None):
     """The operator (float32 forward_ in place, 2^28 elements, library defaults) over placements of
     its three arrays inside ONE allocation: mu at 1 GiB + a, nu at 2 GiB + b for a <= b (so the
     arrays stay disjoint) from a ladder of distances between 0 and 4 MiB.  The rate depends on how
@@ -769,9 +769,9 @@ def run_placements(reps=10):
 
     lib = _lib.load()
     stream = torch.cuda.current_stream()
-    n = 1 << 28
-    ladder = (0, 1, 2, 3, 4, 5, 6, 7, 8, 12, 16, 24, 32, 64, 128, 256, 512, 1024, 2048, 4096)  # KiB
-    arena = torch.empty(3 * n + (8 << 20) // 4, device='cuda')
+    if ladder is None:  # KiB
+        ladder = (0, 1, 2, 3, 4, 5, 6, 7, 8, 12, 16, 24, 32, 64, 128, 256, 512, 1024, 2048, 4096)
+    arena = torch.empty(3 * n + 2 * max(ladder) * 256, device='cuda')
     preheat(torch)
     grid, cells = {}, []
     for a_kib in ladder:

@@ -41,3 +41,13 @@ def test_ceiling_probe_runs():
     for row in out['ceilings'].values():
         assert row['GB/s'] > 0 and row['waves_per_cu'] in bench.RESIDENCY_LEVELS
     torch.cuda.empty_cache()
+
+
+def test_placement_sweep_runs():
+    """The operator over placements of its arrays inside one allocation (`bench.py --placements`),
+    on small arrays and a short ladder."""
+    out = bench.run_placements(reps=2, n=1 << 22, ladder=(0, 8, 64))
+    assert out['placements'] == 6 and out['unit'] == 'GB/s'
+    assert 0 < out['min'] <= out['median'] <= out['max']
+    assert set(out['GB/s_by_placement']) == {'mu +0 KiB', 'mu +8 KiB', 'mu +64 KiB'}
+    torch.cuda.empty_cache()
