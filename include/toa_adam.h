@@ -44,7 +44,7 @@ extern "C" {
 /* Element types.  TOA_F16 (IEEE half) and TOA_BF16 (bfloat16) follow the arithmetic the
  * reference CPU op performs on at::Half / at::BFloat16 tensors: every operation between two
  * 16-bit values is rounded back to 16 bits, the square root and division of the update run in
- * float and are rounded once.  The fused optimizer step takes TOA_F32 / TOA_F64 only. */
+ * float and are rounded once.  The fused optimizer step takes weight decay for TOA_F32 / TOA_F64 only. */
 enum { TOA_F32 = 0, TOA_F64 = 1, TOA_F16 = 2, TOA_BF16 = 3 };
 
 enum {
@@ -277,7 +277,13 @@ TOA_API int toa_adam_backward_all_multi(int dtype, size_t num_tensors,
  * the result is bit-identical to them.  mu, nu and params are overwritten; `updates` is
  * overwritten with the scaled update only if write_updates != 0 (otherwise it is read only:
  * 28 instead of 32 bytes per float32 element, against 44 and more for the separate passes).
- * TOA_F32 / TOA_F64 only.  No single counterpart in the reference. */
+ * Element types: all four without weight decay.  On TOA_F16 / TOA_BF16 the step is forward_ with
+ * the 16-bit types' per-operation rounding, then the two torch calls as torch evaluates them on
+ * 16-bit tensors: the update times float(-lr) (the scalar is NOT rounded to 16 bits) rounded to
+ * 16 bits, then params plus that, rounded to 16 bits.  With weight_decay != 0 the 16-bit types
+ * return TOA_EDTYPE: Tensor.add_(p, alpha=wd) on 16-bit CPU tensors is not one arithmetic (its
+ * vectorized body and its scalar tails round differently), so there is no result to be identical
+ * to.  No single counterpart in the reference. */
 TOA_API int toa_adam_fused_step(int dtype, void *params, void *updates, void *mu, void *nu,
                                 size_t n, double b1, double b2, double eps, double eps_root,
                                 uint64_t count, double lr, double weight_decay, int decoupled,

@@ -368,6 +368,54 @@ static inline float f32_from_bf16(uint16_t b) { return f32_from((uint32_t)b << 1
 ORACLE_DEFINE_LOWP(f16, f16_from_f32, f32_from_f16)
 ORACLE_DEFINE_LOWP(bf16, bf16_from_f32, f32_from_bf16)
 
+/* The classic in-place optimizer step on 16-bit tensors, WITHOUT weight decay: the chain of
+ * ORACLE_DEFINE_STEP above with forward_ as the low-precision restatement, and the torch calls
+ * around it as torch evaluates them on 16-bit CPU tensors: Tensor.mul_(-lr) widens the tensor
+ * operand to float, takes the Python scalar double -> float (NOT rounded to 16 bits), multiplies
+ * in float and rounds the product to 16 bits; Tensor.add_(u) is a float addition rounded to 16
+ * bits; neg_ is exact.
+ * Weight decay is left out on purpose: Tensor.add_(p, alpha=wd) on 16-bit CPU tensors has no
+ * single arithmetic to restate -- its vectorized body rounds alpha to 16 bits and then works in
+ * float, its scalar tails (the last elements of every thread's chunk) round the product to 16
+ * bits first, so an element's result depends on where it lies in the tensor.  `decay` must be 0;
+ * any other value leaves the arrays untouched and returns -1. */
+#define ORACLE_DEFINE_LOWP_STEP(SFX, TO16, FROM16)                                             \
+    int oracle_adam_fused_step_##SFX(uint16_t *params, uint16_t *updates, uint16_t *mu,        \
+                                     uint16_t *nu, size_t n, double b1_, double b2_,           \
+                                     double eps_, double eps_root_, uint64_t count,            \
+                                     double lr_, double wd_, int decay, int maximize,          \
+                                     int write_updates) {                                      \
+        (void)wd_;                                                                             \
+        if (decay != 0) return -1;                                                             \
+        double s[4];                                                                           \
+        oracle_adam_host_scalars(b1_, b2_, eps_root_, count, s);                               \
+        const float b1 = rnd_##SFX((float)b1_), b2 = rnd_##SFX((float)b2_);                    \
+        const float eps = rnd_##SFX((float)eps_), er = rnd_##SFX((float)eps_root_);            \
+        const float c1 = rnd_##SFX((float)s[0]), c2 = rnd_##SFX((float)s[1]);                  \
+        const float neg_lr = (float)(-lr_);                                                    \
+        PAR_FOR(n)                                                                             \
+        for (size_t i = 0; i < n; ++i) {                                                       \
+            const float p = FROM16(params[i]), m = FROM16(mu[i]), v = FROM16(nu[i]);           \
+            float g = FROM16(updates[i]);                                                      \
+            if (maximize) g = -g;                                                              \
+            const float m1 =                                                                   \
+                rnd_##SFX(rnd_##SFX(b1 * m) + rnd_##SFX(rnd_##SFX(1.0f - b1) * g));            \
+            const float v1 = rnd_##SFX(                                                        \
+                rnd_##SFX(b2 * v) + rnd_##SFX(rnd_##SFX(rnd_##SFX(1.0f - b2) * g) * g));       \
+            const float mh = rnd_##SFX(m1 * c1), vh = rnd_##SFX(v1 * c2);                      \
+            const float u1 = rnd_##SFX(mh / (sqrtf(rnd_##SFX(vh + er)) + eps));                \
+            const float step = rnd_##SFX(u1 * neg_lr);                                         \
+            mu[i] = TO16(m1);                                                                  \
+            nu[i] = TO16(v1);                                                                  \
+            params[i] = TO16(p + step);                                                        \
+            if (write_updates) updates[i] = TO16(step);                                        \
+        }                                                                                      \
+        return 0;                                                                              \
+    }
+
+ORACLE_DEFINE_LOWP_STEP(f16, f16_from_f32, f32_from_f16)
+ORACLE_DEFINE_LOWP_STEP(bf16, bf16_from_f32, f32_from_bf16)
+
 /* conversions, exported so tests can pin them against NumPy's float16 and torch's bfloat16 */
 uint16_t oracle_f16_from_f32(float f) { return f16_from_f32(f); }
 float oracle_f32_from_f16(uint16_t h) { return f32_from_f16(h); }

@@ -96,6 +96,19 @@ void oracle_adam_fused_step_f64(double *params, double *updates, double *mu, dou
                                 double b1, double b2, double eps, double eps_root,
                                 uint64_t count, double lr, double weight_decay, int decay,
                                 int maximize, int write_updates);
+/* ... on float16 / bfloat16 bit patterns, without weight decay (`decay` must be 0, else -1 and
+ * nothing is touched: torch's add_(p, alpha=wd) on 16-bit CPU tensors is not one arithmetic, see
+ * the .c file): forward_ with the per-operation rounding of the 16-bit types; mul_(-lr) in float
+ * with the scalar unrounded, add_ in float, one rounding to 16 bits per call.  Pinned against
+ * those very calls on 16-bit CPU tensors.  Returns 0. */
+int oracle_adam_fused_step_f16(uint16_t *params, uint16_t *updates, uint16_t *mu, uint16_t *nu,
+                               size_t n, double b1, double b2, double eps, double eps_root,
+                               uint64_t count, double lr, double weight_decay, int decay,
+                               int maximize, int write_updates);
+int oracle_adam_fused_step_bf16(uint16_t *params, uint16_t *updates, uint16_t *mu, uint16_t *nu,
+                                size_t n, double b1, double b2, double eps, double eps_root,
+                                uint64_t count, double lr, double weight_decay, int decay,
+                                int maximize, int write_updates);
 
 /* Host-side bias-correction scalars in double, before the cast to the element
  * type (adam_op_impl_cpu.cpp:73-74, 191-192, 328-329).

@@ -149,6 +149,9 @@ def fused_step(params, updates, mu, nu, b1, b2, eps, eps_root, count, lr, maximi
     """Mutates params, mu, nu (and updates when write_updates), like the reference's classic
     in-place chains: [negate], [L2 decay], forward_, [decoupled decay], scale by -lr, apply."""
     decay = 0 if weight_decay == 0.0 else (2 if decoupled else 1)
+    if decay and params.dtype.itemsize == 2:
+        raise ValueError('no weight decay on 16-bit tensors: torch.Tensor.add_(p, alpha=wd) is not '
+                         'one arithmetic there (vectorized body and scalar tails round differently)')
     _fn('fused_step', params.dtype)(_ptr(params), _ptr(updates), _ptr(mu), _ptr(nu),
                                     _SZ(params.size), _D(b1), _D(b2), _D(eps), _D(eps_root),
                                     _U64(count), _D(lr), _D(weight_decay), ctypes.c_int(decay),

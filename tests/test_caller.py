@@ -100,3 +100,15 @@ def test_cpu_leaves_are_refused():
     state = t.init(params)
     with pytest.raises(RuntimeError, match='Not implemented'):
         t.update([torch.ones(3)], state, inplace=True)
+
+
+def test_fused_adam_refuses_weight_decay_on_16_bit_parameters():
+    from torchopt_amd import FusedAdam, FusedAdamW
+
+    p16 = torch.zeros(4, dtype=torch.bfloat16, requires_grad=True)
+    p32 = torch.zeros(4, requires_grad=True)
+    FusedAdam([p16, p32])  # no decay: fine
+    FusedAdamW([p32], weight_decay=0.01)
+    for cls in (FusedAdam, FusedAdamW):
+        with pytest.raises(ValueError, match='float32 and float64 parameters only'):
+            cls([p32, p16], weight_decay=0.01)

@@ -263,3 +263,117 @@ def test_fused_adamw_mask():
             o.step()
     for p, q in zip(net.parameters(), ref.parameters()):
         torch.testing.assert_close(p, q, rtol=2e-5, atol=1e-6)
+
+
+# ---- float16 / bfloat16 -----------------------------------------------------------------------
+# The 16-bit step has no weight decay: Tensor.add_(p, alpha=wd) on 16-bit CPU tensors is not one
+# arithmetic (tests/test_oracle.py shows body and tail of one call disagreeing), so there is no
+# result to be identical to and the library refuses the combination.
+
+TDT = {'f16': torch.float16, 'bf16': torch.bfloat16}
+
+
+def rand4_16(fmt, n, seed):
+    """(params, updates, mu, nu) as host arrays in the oracle's format for `fmt` (NumPy float16,
+    or uint16 bit patterns for bfloat16) and as GPU tensors."""
+    rng = np.random.default_rng(seed)
+    raw = (rng.standard_normal(n), rng.standard_normal(n), 0.1 * rng.standard_normal(n),
+           np.abs(0.01 * rng.standard_normal(n)))
+    ts = [torch.from_numpy(a.astype(np.float32)).to(TDT[fmt]) for a in raw]
+    return [bits16(t, fmt) for t in ts], [t.cuda() for t in ts]
+
+
+def bits16(t, fmt):
+    t = t.detach().cpu().contiguous()
+    if fmt == 'bf16':
+        return t.view(torch.int16).numpy().view(np.uint16).copy()
+    return t.numpy().copy()
+
+
+@pytest.mark.parametrize('fmt', ['f16', 'bf16'])
+@pytest.mark.parametrize('maximize', [False, True])
+@pytest.mark.parametrize('write_updates', [False, True])
+def test_16_bit_single_tensor_against_oracle(fmt, maximize, write_updates):
+    # sizes on both sides of the whole-tile kernel's threshold, ragged tails, odd element counts
+    for k, n in enumerate([1, 3, 511, 512, 513, 4099, 65537, (1 << 22) + 7]):
+        lr, count, eps_root = (1e-3, 1, 0.0) if k % 2 else (0.05, 1000, 1e-4)
+        h, d = rand4_16(fmt, n, 900 + n)
+        print(f'fused_step_ {fmt} n={n} maximize={maximize} write_updates={write_updates}',
+              flush=True)
+        adam_op.fused_step_(d[0], d[1], d[2], d[3], B1, B2, 1e-3, eps_root, count, lr,
+                            maximize=maximize, write_updates=write_updates)
+        O.fused_step(h[0], h[1], h[2], h[3], B1, B2, 1e-3, eps_root, count, lr, maximize,
+                     write_updates)
+        for j, what in enumerate(('params', 'updates', 'mu', 'nu')):
+            assert_bit_equal(bits16(d[j], fmt), h[j], f'{fmt} n={n} {what}')
+
+
+@pytest.mark.parametrize('fmt', ['f16', 'bf16'])
+def test_16_bit_step_equals_the_unfused_chain_on_the_gpu(fmt):
+    """forward_ in place, then PyTorch's own GPU kernels for mul_(-lr) and add_."""
+    n, lr, count = (1 << 21) + 5, 0.05, 9
+    h, d = rand4_16(fmt, n, 77)
+    p, g, m, v = (t.clone() for t in d)
+    adam_op.forward_(g, m, v, B1, B2, 1e-3, 0.0, count)
+    g.mul_(-lr)
+    p.add_(g)
+    adam_op.fused_step_(d[0], d[1], d[2], d[3], B1, B2, 1e-3, 0.0, count, lr, write_updates=True)
+    for got, want, what in zip(d, (p, g, m, v), ('params', 'updates', 'mu', 'nu')):
+        assert_bit_equal(bits16(got, fmt), bits16(want, fmt), f'{fmt} {what}')
+
+
+@pytest.mark.parametrize('fmt', ['f16', 'bf16'])
+def test_16_bit_list_with_ragged_members_and_counts(fmt):
+    sizes = [864, 9216, 33, 4001, 5, 0, 70_001, 1 << 20]
+    counts = [1, 1, 2, 7, 7, 3, 1000, 2]
+    pairs = [rand4_16(fmt, n, 40 + k) for k, n in enumerate(sizes)]
+    hs, ds = [p[0] for p in pairs], [p[1] for p in pairs]
+    print(f'fused_step_multi_ {fmt} ragged list', flush=True)
+    adam_op.fused_step_multi_([d[0] for d in ds], [d[1] for d in ds], [d[2] for d in ds],
+                              [d[3] for d in ds], B1, B2, 1e-3, 1e-4, counts, 0.01,
+                              maximize=True, write_updates=True)
+    for k, (h, d) in enumerate(zip(hs, ds)):
+        O.fused_step(h[0], h[1], h[2], h[3], B1, B2, 1e-3, 1e-4, counts[k], 0.01, True, True)
+        for j, what in enumerate(('params', 'updates', 'mu', 'nu')):
+            assert_bit_equal(bits16(d[j], fmt), h[j], f'{fmt} tensor {k} {what}')
+
+
+@pytest.mark.parametrize('fmt', ['f16', 'bf16'])
+def test_16_bit_step_refuses_weight_decay(fmt):
+    _, d = rand4_16(fmt, 1000, 3)
+    before = [t.clone() for t in d]
+    for decoupled in (False, True):
+        with pytest.raises(RuntimeError, match='weight decay for float32 and float64 only'):
+            adam_op.fused_step_(d[0], d[1], d[2], d[3], B1, B2, 1e-3, 0.0, 1, 0.01,
+                                weight_decay=0.01, decoupled=decoupled)
+        with pytest.raises(RuntimeError, match='weight decay for float32 and float64 only'):
+            adam_op.fused_step_multi_([d[0]], [d[1]], [d[2]], [d[3]], B1, B2, 1e-3, 0.0, 1, 0.01,
+                                      weight_decay=0.01, decoupled=decoupled)
+    torch.cuda.synchronize()
+    assert all(torch.equal(a, b) for a, b in zip(d, before)), 'a refused call touched its tensors'
+
+
+@pytest.mark.parametrize('fmt', ['f16', 'bf16'])
+@pytest.mark.parametrize('capturable', [False, True])
+def test_fused_adam_on_16_bit_parameters(fmt, capturable):
+    """Five optimizer steps on 16-bit parameters, host-counted and with the count on the device,
+    against the oracle step by step."""
+    shapes = [(300, 7), (5,), (64, 64, 3)]
+    rng = np.random.default_rng(21)
+    tdt = TDT[fmt]
+    params = [torch.from_numpy(rng.standard_normal(s).astype(np.float32)).to(tdt).cuda()
+              .requires_grad_(True) for s in shapes]
+    hp = [bits16(p, fmt).reshape(-1) for p in params]
+    hm = [np.zeros_like(a) for a in hp]
+    hv = [np.zeros_like(a) for a in hp]
+    opt = FusedAdam(params, lr=0.01, eps=1e-3, eps_root=1e-4, capturable=capturable)
+    for step in range(1, 6):
+        grads = [torch.from_numpy(rng.standard_normal(s).astype(np.float32)).to(tdt) for s in shapes]
+        for p, g in zip(params, grads):
+            p.grad = g.cuda()
+        opt.step()
+        for k, g in enumerate(grads):
+            O.fused_step(hp[k], bits16(g, fmt).reshape(-1), hm[k], hv[k], B1, B2, 1e-3, 1e-4, step,
+                         0.01)
+            assert_bit_equal(bits16(params[k], fmt).reshape(-1), hp[k],
+                             f'{fmt} step {step} params[{k}]')

@@ -68,9 +68,14 @@ def test_abi_version_and_error_strings():
         assert b'toa_adam' in lib.toa_adam_error_string(code)
     with pytest.raises(RuntimeError, match='unsupported dtype'):
         _lib.check(-1, 'x')
-    # the fused optimizer step serves float32 / float64 only
-    assert lib.toa_adam_fused_step(_lib.TOA_F16, None, None, None, None, 0, 0.9, 0.999, 1e-8, 0.0, 1,
-                                   1e-3, 0.0, 0, 0, 0, None) == -1
+    # the fused optimizer step serves the 16-bit types without weight decay only (n = 0: no launch)
+    for code in (_lib.TOA_F16, _lib.TOA_BF16):
+        assert lib.toa_adam_fused_step(code, None, None, None, None, 0, 0.9, 0.999, 1e-8, 0.0, 1,
+                                       1e-3, 0.0, 0, 0, 0, None) == 0
+        for decoupled in (0, 1):
+            assert lib.toa_adam_fused_step(code, None, None, None, None, 0, 0.9, 0.999, 1e-8, 0.0,
+                                           1, 1e-3, 0.01, decoupled, 0, 0, None) == -1
+    assert b'weight decay' in lib.toa_adam_error_string(-1)
 
 
 def test_argument_errors_need_no_device():

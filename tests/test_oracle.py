@@ -311,6 +311,92 @@ def test_low_precision_oracle_equals_compiled_reference(fmt):
             assert_bit_equal(a, arr(b))
 
 
+@pytest.mark.parametrize('fmt', ['f16', 'bf16'])
+@pytest.mark.parametrize('maximize', [False, True])
+def test_low_precision_fused_step_is_the_reference_chain(fmt, maximize):
+    """The classic in-place step on 16-bit tensors, without weight decay: the very calls the
+    reference's chains make -- [neg_], forward_ (compiled reference where it is built, else the
+    pinned C oracle), mul_(-lr), add_ -- on 16-bit CPU tensors, against the one-pass oracle.  Pins
+    how torch treats the Python scalar there: -lr acts as a float, not as a 16-bit value (0.05 is
+    not representable in either format)."""
+    import torch
+
+    ref = O.load_reference()
+    tdt = torch.float16 if fmt == 'f16' else torch.bfloat16
+    rng = np.random.default_rng(41)
+
+    def tens(a):
+        return torch.from_numpy(np.asarray(a, dtype=np.float32)).to(tdt)
+
+    def arr(t):
+        if fmt == 'bf16':
+            return t.contiguous().view(torch.int16).numpy().view(np.uint16).copy()
+        return t.numpy().copy()
+
+    for n, lr, count, eps_root in [(1, 1e-3, 1, 0.0), (1003, 1e-3, 7, 0.0), (200_003, 0.05, 1000, 1e-4)]:
+        g, m = tens(rng.standard_normal(n)), tens(0.1 * rng.standard_normal(n))
+        v, p = tens(np.abs(0.01 * rng.standard_normal(n))), tens(rng.standard_normal(n))
+        tg, tm, tv, tp = g.clone(), m.clone(), v.clone(), p.clone()
+        if maximize:
+            tg.neg_()
+        if ref is not None:
+            ref.adam_op.forward_(tg, tm, tv, 0.9, 0.999, 1e-3, eps_root, count)
+        else:
+            og, om, ov = arr(tg), arr(tm), arr(tv)
+            O.forward_inplace(og, om, ov, 0.9, 0.999, 1e-3, eps_root, count)
+            for t, a in ((tg, og), (tm, om), (tv, ov)):
+                t.copy_(torch.from_numpy(a.view(np.int16)).view(tdt) if fmt == 'bf16'
+                        else torch.from_numpy(a))
+        tg.mul_(-lr)
+        tp.add_(tg)
+        for write_updates in (True, False):
+            op, og, om, ov = arr(p), arr(g), arr(m), arr(v)
+            O.fused_step(op, og, om, ov, 0.9, 0.999, 1e-3, eps_root, count, lr, maximize,
+                         write_updates)
+            assert_bit_equal(om, arr(tm), 'mu')
+            assert_bit_equal(ov, arr(tv), 'nu')
+            assert_bit_equal(og, arr(tg) if write_updates else arr(g), 'updates')
+            assert_bit_equal(op, arr(tp), 'params')
+    with pytest.raises(ValueError, match='no weight decay on 16-bit'):
+        O.fused_step(arr(p), arr(g), arr(m), arr(v), 0.9, 0.999, 1e-3, 0.0, 1, 1e-3, False, True,
+                     0.01, True)
+
+
+def test_low_precision_step_keeps_its_learning_rate_in_float():
+    """-lr = -0.05 is not representable in float16 or bfloat16: a step scaled by the rounded scalar
+    differs from torch's mul_(-0.05) on a fifth of random elements and more, one scaled by the
+    float scalar on none -- so the distinction is observable and the oracle is on torch's side."""
+    import torch
+
+    rng = np.random.default_rng(5)
+    u = rng.standard_normal(200_000).astype(np.float32)
+    for tdt in (torch.float16, torch.bfloat16):
+        t = torch.from_numpy(u).to(tdt)
+        torch_way = t.clone().mul_(-0.05)
+        rounded_scalar = (t.float() * torch.tensor(-0.05).to(tdt).float()).to(tdt)
+        assert (torch_way != rounded_scalar).sum() > 20_000
+        float_scalar = (t.float() * torch.tensor(-0.05, dtype=torch.float32)).to(tdt)
+        assert torch.equal(torch_way, float_scalar)
+
+
+def test_weight_decay_on_16_bit_cpu_tensors_is_not_one_arithmetic():
+    """Why the 16-bit step leaves weight decay out: torch.Tensor.add_(p, alpha=wd) on a bfloat16
+    CPU tensor rounds alpha to bfloat16 and works in float in its vectorized body, but rounds the
+    product to bfloat16 first in its scalar tail -- the same operands give different results
+    depending on where in the tensor they lie."""
+    import torch
+
+    a = torch.tensor(-0.49609375, dtype=torch.bfloat16)
+    b = torch.tensor(1.984375, dtype=torch.bfloat16)
+    n = 4096 + 1  # the last element falls into the scalar tail
+    ta, tb = a.repeat(n), b.repeat(n)
+    out = ta.clone().add_(tb, alpha=0.03)
+    body, tail = out[0].item(), out[-1].item()
+    if body == tail:
+        pytest.skip('this build of torch evaluates body and tail alike')
+    assert {body, tail} == {-0.435546875, -0.4375}
+
+
 # ---------------------------------------------------------------------------------------------
 # What the mathematics fixes
 # ---------------------------------------------------------------------------------------------

@@ -1001,6 +1001,26 @@ enum : int { kNoDecay = 0, kDecayIntoGradient = 1, kDecayIntoUpdate = 2 };
 
 __device__ __forceinline__ float toa_fma(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 __device__ __forceinline__ double toa_fma(double a, double b, double c) { return __builtin_fma(a, b, c); }
+// 16-bit tensors: PyTorch evaluates Tensor.add_(p, alpha=wd) and Tensor.mul_(-lr) in float -- the
+// Python scalar goes double -> float and is NOT rounded to 16 bits, the tensor operands widen, one
+// float operation (a fused multiply-add for add_), one rounding back to 16 bits.  The float result
+// of these overloads is rounded when it is assigned to the 16-bit type.
+template <class F>
+__device__ __forceinline__ float toa_fma(float a, R16<F> b, R16<F> c) {
+    return __builtin_fmaf(a, (float)b, (float)c);
+}
+// The type the step's two scalars (-lr and the weight decay) are held in: the element type for
+// float32 / float64, float for the 16-bit types.
+template <typename T>
+struct StepScalarOf {
+    using type = T;
+};
+template <class F>
+struct StepScalarOf<R16<F>> {
+    using type = float;
+};
+template <typename T>
+using StepScalar = typename StepScalarOf<T>::type;
 
 template <typename T, bool WRITE_UPDATES>
 struct alignas(8) FusedStep {
@@ -1013,7 +1033,8 @@ struct alignas(8) FusedStep {
     static constexpr bool kStagedLists = true;
     // outputs: mu', nu', params', then the scaled update
     __device__ static constexpr int out_slot(int j) { return j == 3 ? 0 : j + 1; }
-    T b1, b2, c1, c2, eps, eps_root, neg_lr, wd;
+    T b1, b2, c1, c2, eps, eps_root;
+    StepScalar<T> neg_lr, wd;
     int decay;
     bool maximize;
     __device__ __forceinline__ void set_bias(T c1_, T c2_, T, T) {
@@ -1031,6 +1052,13 @@ struct alignas(8) FusedStep {
     __device__ __forceinline__ T direction(T m1, T v1) const {
         const T mh = m1 * c1;
         const T vh = v1 * c2;
+        if constexpr (HasQuickDirection<T>::value) {
+            // the checked shortcut of the 16-bit types; an element it cannot settle takes the
+            // exact chain
+            bool ok;
+            const T quick = adam_direction_quick(mh, vh, eps_root, eps, ok);
+            if (ok) return quick;
+        }
         return adam_direction(mh, vh, eps_root, eps);
     }
     // the scaled update from the direction

@@ -594,20 +594,7 @@ T *mut(const void *p) {
     return static_cast<T *>(const_cast<void *>(p));
 }
 
-// float32 and float64 only (the fused optimizer step)
-#define TOA_DISPATCH(dtype, ...)                  \
-    switch (dtype) {                              \
-        case TOA_F32: {                           \
-            using T = float;                      \
-            return __VA_ARGS__();                 \
-        }                                         \
-        case TOA_F64: {                           \
-            using T = double;                     \
-            return __VA_ARGS__();                 \
-        }                                         \
-        default:                                  \
-            return TOA_EDTYPE;                    \
-    }
+bool is_16_bit(int dtype) { return dtype == TOA_F16 || dtype == TOA_BF16; }
 
 #define CPP(x) reinterpret_cast<const void *const *>(x)
 
@@ -740,7 +727,9 @@ unsigned toa_adam_set_max_grid(unsigned workgroups) {
 const char *toa_adam_error_string(int code) {
     switch (code) {
         case 0: return "success";
-        case TOA_EDTYPE: return "toa_adam: unsupported dtype for this entry point";
+        case TOA_EDTYPE:
+            return "toa_adam: unsupported dtype for this entry point (the fused step takes weight "
+                   "decay for float32 and float64 only)";
         case TOA_ENULL: return "toa_adam: null pointer for a non-empty tensor";
         case TOA_ESIZE: return "toa_adam: tensor too large for one launch";
         case TOA_ELIMIT:
@@ -1002,6 +991,10 @@ int toa_adam_backward_all_multi(int dtype, size_t num_tensors, const void *const
 }
 
 // ---- fused optimizer step ------------------------------------------------------
+// All four element types without weight decay; with it, float32 and float64 only: the chain the
+// step reproduces applies decay with Tensor.add_(p, alpha=wd), which on 16-bit CPU tensors is not
+// one arithmetic (its vectorized body and its scalar tails round differently), so there is no
+// result to be identical to.
 
 int toa_adam_fused_step(int dtype, void *params, void *updates, void *mu, void *nu, size_t n,
                         double b1, double b2, double eps, double eps_root, uint64_t count,
@@ -1010,15 +1003,16 @@ int toa_adam_fused_step(int dtype, void *params, void *updates, void *mu, void *
     const HostScalars s = host_scalars(b1, b2, eps_root, count);
     const int decay = weight_decay == 0.0 ? kNoDecay
                                           : (decoupled ? kDecayIntoUpdate : kDecayIntoGradient);
-    TOA_DISPATCH(dtype, [&] {
+    if (decay != kNoDecay && is_16_bit(dtype)) return TOA_EDTYPE;
+    TOA_DISPATCH_ALL(dtype, [&] {
         T *const p[4] = {(T *)updates, (T *)mu, (T *)nu, (T *)params};
         if (write_updates) {
             const FusedStep<T, true> op{(T)b1,       (T)b2,    (T)s.c1,         (T)s.c2, (T)eps,
-                                        (T)eps_root, (T)(-lr), (T)weight_decay, decay,   maximize != 0};
+                                        (T)eps_root, (StepScalar<T>)(-lr), (StepScalar<T>)weight_decay, decay,   maximize != 0};
             return launch_single<T>(op, p, n, stream);
         }
         const FusedStep<T, false> op{(T)b1,       (T)b2,    (T)s.c1,         (T)s.c2, (T)eps,
-                                     (T)eps_root, (T)(-lr), (T)weight_decay, decay,   maximize != 0};
+                                     (T)eps_root, (StepScalar<T>)(-lr), (StepScalar<T>)weight_decay, decay,   maximize != 0};
         return launch_single<T>(op, p, n, stream);
     });
 }
@@ -1031,13 +1025,14 @@ int toa_adam_fused_step_multi(int dtype, size_t num_tensors, void *const *params
                               int write_updates, void *stream) {
     const int decay = weight_decay == 0.0 ? kNoDecay
                                           : (decoupled ? kDecayIntoUpdate : kDecayIntoGradient);
-    TOA_DISPATCH(dtype, [&] {
+    if (decay != kNoDecay && is_16_bit(dtype)) return TOA_EDTYPE;
+    TOA_DISPATCH_ALL(dtype, [&] {
         const void *const *const lists[4] = {CPP(updates), CPP(mu), CPP(nu), CPP(params)};
         if (write_updates) {
             auto make = [&](uint64_t c) {
                 const HostScalars s = host_scalars(b1, b2, eps_root, c);
                 return FusedStep<T, true>{(T)b1,       (T)b2,    (T)s.c1,         (T)s.c2, (T)eps,
-                                          (T)eps_root, (T)(-lr), (T)weight_decay, decay,
+                                          (T)eps_root, (StepScalar<T>)(-lr), (StepScalar<T>)weight_decay, decay,
                                           maximize != 0};
             };
             return launch_multi<T, FusedStep<T, true>>(make, num_tensors, lists, n, counts,
@@ -1046,7 +1041,7 @@ int toa_adam_fused_step_multi(int dtype, size_t num_tensors, void *const *params
         auto make = [&](uint64_t c) {
             const HostScalars s = host_scalars(b1, b2, eps_root, c);
             return FusedStep<T, false>{(T)b1,       (T)b2,    (T)s.c1,         (T)s.c2, (T)eps,
-                                       (T)eps_root, (T)(-lr), (T)weight_decay, decay,
+                                       (T)eps_root, (StepScalar<T>)(-lr), (StepScalar<T>)weight_decay, decay,
                                        maximize != 0};
         };
         return launch_multi<T, FusedStep<T, false>>(make, num_tensors, lists, n, counts,
@@ -1136,19 +1131,20 @@ int toa_adam_fused_step_devcount(int dtype, void *params, void *updates, void *m
                                  int decoupled, int maximize, int write_updates, void *stream) {
     const int decay = weight_decay == 0.0 ? kNoDecay
                                           : (decoupled ? kDecayIntoUpdate : kDecayIntoGradient);
-    TOA_DISPATCH(dtype, [&] {
+    if (decay != kNoDecay && is_16_bit(dtype)) return TOA_EDTYPE;
+    TOA_DISPATCH_ALL(dtype, [&] {
         StepRef<T> step;
         if (const int rc = make_step_ref<T>(bias_rows, first_count, rows, count, &step)) return rc;
         T *const p[4] = {(T *)updates, (T *)mu, (T *)nu, (T *)params};
         if (write_updates) {
             const AtStep<FusedStep<T, true>, T> op{
-                {(T)b1, (T)b2, T(1), T(1), (T)eps, (T)eps_root, (T)(-lr), (T)weight_decay, decay,
+                {(T)b1, (T)b2, T(1), T(1), (T)eps, (T)eps_root, (StepScalar<T>)(-lr), (StepScalar<T>)weight_decay, decay,
                  maximize != 0},
                 step};
             return launch_single<T>(op, p, n, stream);
         }
         const AtStep<FusedStep<T, false>, T> op{
-            {(T)b1, (T)b2, T(1), T(1), (T)eps, (T)eps_root, (T)(-lr), (T)weight_decay, decay,
+            {(T)b1, (T)b2, T(1), T(1), (T)eps, (T)eps_root, (StepScalar<T>)(-lr), (StepScalar<T>)weight_decay, decay,
              maximize != 0},
             step};
         return launch_single<T>(op, p, n, stream);
@@ -1164,22 +1160,23 @@ int toa_adam_fused_step_multi_devcount(int dtype, size_t num_tensors, void *cons
                                        int maximize, int write_updates, void *stream) {
     const int decay = weight_decay == 0.0 ? kNoDecay
                                           : (decoupled ? kDecayIntoUpdate : kDecayIntoGradient);
-    TOA_DISPATCH(dtype, [&] {
+    if (decay != kNoDecay && is_16_bit(dtype)) return TOA_EDTYPE;
+    TOA_DISPATCH_ALL(dtype, [&] {
         StepRef<T> step;
         if (const int rc = make_step_ref<T>(bias_rows, first_count, rows, count, &step)) return rc;
         const void *const *const lists[4] = {CPP(updates), CPP(mu), CPP(nu), CPP(params)};
         if (write_updates) {
             using Op = AtStep<FusedStep<T, true>, T>;
             auto make = [&](uint64_t) {
-                return Op{{(T)b1, (T)b2, T(1), T(1), (T)eps, (T)eps_root, (T)(-lr),
-                           (T)weight_decay, decay, maximize != 0},
+                return Op{{(T)b1, (T)b2, T(1), T(1), (T)eps, (T)eps_root, (StepScalar<T>)(-lr),
+                           (StepScalar<T>)weight_decay, decay, maximize != 0},
                           step};
             };
             return launch_multi<T, Op>(make, num_tensors, lists, n, nullptr, 0, stream);
         }
         using Op = AtStep<FusedStep<T, false>, T>;
         auto make = [&](uint64_t) {
-            return Op{{(T)b1, (T)b2, T(1), T(1), (T)eps, (T)eps_root, (T)(-lr), (T)weight_decay,
+            return Op{{(T)b1, (T)b2, T(1), T(1), (T)eps, (T)eps_root, (StepScalar<T>)(-lr), (StepScalar<T>)weight_decay,
                        decay, maximize != 0},
                       step};
         };

@@ -48,8 +48,9 @@ __all__ = ['Adam', 'AdamW', 'FusedAdam', 'FusedAdamW']
 
 
 class FusedAdam:
-    """Classic Adam with the fused single-pass step (GPU tensors, float32 / float64).
-    `weight_decay` is the L2 kind: added to the gradient before the moments."""
+    """Classic Adam with the fused single-pass step (GPU tensors; float32 / float64, and float16 /
+    bfloat16 without weight decay).  `weight_decay` is the L2 kind: added to the gradient before
+    the moments."""
 
     _decoupled = False
     _mask = None  # FusedAdamW: which parameters decay
@@ -115,6 +116,14 @@ class FusedAdam:
         self._decays.append([True] * len(group) if mask is None else [bool(m) for m in mask])
         if len(self._decays[-1]) != len(group):
             raise ValueError('mask and parameters differ in length')
+        if self.weight_decay != 0.0:
+            for p, decays in zip(group, self._decays[-1]):
+                if decays and p.dtype in (torch.float16, torch.bfloat16):
+                    # the chain this step reproduces applies decay with Tensor.add_(p, alpha=wd),
+                    # which on 16-bit CPU tensors is not one arithmetic (vectorized body and
+                    # scalar tails round differently): there is no result to be identical to
+                    raise ValueError(f'{type(self).__name__}: weight decay is served for float32 '
+                                     f'and float64 parameters only, got {p.dtype}')
         self._steps.append(None)
         self._stale.append(False)
 
