@@ -453,8 +453,9 @@ def test_error_paths_on_gpu_tensors():
     a = torch.ones(8, device='cuda')
     with pytest.raises(RuntimeError, match='not implemented for'):
         adam_op.forward_mu(a.int(), a.int(), 0.9)
-    with pytest.raises(RuntimeError, match='unsupported dtype'):  # 16-bit: not in the fused step
-        adam_op.fused_step_(a.half(), a.half(), a.half(), a.half(), 0.9, 0.999, 1e-8, 0.0, 1, 1e-3)
+    with pytest.raises(RuntimeError, match='unsupported dtype'):  # 16-bit: no weight decay
+        adam_op.fused_step_(a.half(), a.half(), a.half(), a.half(), 0.9, 0.999, 1e-8, 0.0, 1, 1e-3,
+                            weight_decay=0.01)
     with pytest.raises(RuntimeError, match='scalar type'):
         adam_op.forward_mu(a, a.double(), 0.9)
     with pytest.raises(RuntimeError, match='size mismatch'):
