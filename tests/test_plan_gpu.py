@@ -199,3 +199,68 @@ def test_fused_step_and_one_pass_ops_over_a_long_list():
     check_lists(gp, params, 'fused step params')
     check_lists(g['mu'], h['mu'], 'fused step mu')
     check_lists(g['nu'], h['nu'], 'fused step nu')
+
+
+def test_a_remembered_call_is_only_taken_for_the_very_same_arguments():
+    """A plan remembers the last call it served and serves a byte-for-byte repeat with one launch.
+    Anything else -- one size changed under the same pointers, another op over the same lists,
+    another schedule, a capturing stream -- must go the long way and still be right."""
+    lib = _lib.load()
+    sizes = ragged_sizes(200, 11)
+    h = make_lists(np.float32, sizes, 3)
+    g = to_dev(h)
+    print('remembered calls: repeat, size change, other op, other schedule, capture', flush=True)
+    for step in (1, 2, 3):  # 1 writes the plan, 2 and 3 are repeats
+        step_and_check(g, h, step, f'repeat {step}')
+
+    # the same arrays, one tensor shorter by a few elements: views of the same storage
+    k = len(sizes) // 3
+    short = sizes[k] - 1000
+    gs = {name: list(g[name]) for name in ('updates', 'mu', 'nu')}
+    hs = {name: list(h[name]) for name in ('updates', 'mu', 'nu')}
+    keep = {name: h[name][k][short:].copy() for name in hs}
+    for name in gs:
+        gs[name][k] = g[name][k][:short]
+        hs[name][k] = h[name][k][:short]
+    step_and_check(gs, hs, 4, 'one tensor shorter')
+    for name in keep:  # the tail beyond the shorter length was not touched
+        assert_bit_equal(g[name][k][short:].cpu().numpy(), keep[name], f'{name} beyond the new length')
+    step_and_check(g, h, 5, 'full length again')
+
+    # another op over the same three lists plus parameters
+    hp = [np.random.default_rng(50 + i).standard_normal(n).astype(np.float32)
+          for i, n in enumerate(sizes)]
+    gp = [torch.from_numpy(a).cuda() for a in hp]
+    adam_op.fused_step_multi_(gp, g['updates'], g['mu'], g['nu'], B1, B2, EPS, 0.0, 6, 0.01,
+                              write_updates=True)
+    for i in range(len(sizes)):
+        O.fused_step(hp[i], h['updates'][i], h['mu'][i], h['nu'][i], B1, B2, EPS, 0.0, 6, 0.01)
+    check_lists(gp, hp, 'fused step params')
+    check_lists(g['updates'], h['updates'], 'fused step updates')
+    step_and_check(g, h, 7, 'in-place step after the fused one')
+
+    for schedule in (2, 1, 0):
+        lib.toa_adam_set_schedule(schedule)
+        step_and_check(g, h, 8 + schedule, f'schedule {schedule}')
+        step_and_check(g, h, 12 + schedule, f'schedule {schedule}, repeat')
+    lib.toa_adam_set_schedule(0)
+
+    # a capturing stream must not lean on the remembered plan
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        adam_op.forward_multi_(g['updates'], g['mu'], g['nu'], B1, B2, EPS, 0.0, 20)  # warm, eager
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            adam_op.forward_multi_(g['updates'], g['mu'], g['nu'], B1, B2, EPS, 0.0, 21)
+    torch.cuda.synchronize()
+    for i in range(len(sizes)):
+        O.forward_inplace(h['updates'][i], h['mu'][i], h['nu'][i], B1, B2, EPS, 0.0, 20)
+    assert lib.toa_adam_release_plans() == 0  # the replay below must not need any plan
+    graph.replay()
+    torch.cuda.synchronize()
+    for i in range(len(sizes)):
+        O.forward_inplace(h['updates'][i], h['mu'][i], h['nu'][i], B1, B2, EPS, 0.0, 21)
+    check_lists(g['updates'], h['updates'], 'replayed capture updates')
+    check_lists(g['mu'], h['mu'], 'replayed capture mu')

@@ -285,6 +285,13 @@ struct PlanSlot {
     size_t capacity = 0;
     std::vector<unsigned char> key;  // empty: contents unknown
     uint64_t stamp = 0;
+    // The last call this plan served, remembered whole: the caller's arguments as bytes and the
+    // launch they led to.  A training loop calls with the same lists step after step; when the
+    // arguments are byte for byte those of the last time, every per-tensor decision is known
+    // already and the call is one comparison and one launch (150 ns per tensor otherwise).
+    std::vector<unsigned char> call;  // empty: nothing remembered
+    PlanView view;
+    bool staged = false;
 };
 std::mutex g_plan_mutex;
 std::vector<PlanSlot> g_plan_slots;
@@ -352,12 +359,49 @@ void *plan_cached(const std::vector<PlanSeed<NPTR>> &seeds, size_t tile, hipStre
         use->capacity = capacity;
     }
     use->key.clear();
+    use->call.clear();
     *rc = plan_write<NPTR>(use->mem, seeds, stream);
     if (*rc) return nullptr;
     use->key = std::move(key);
     use->stamp = ++g_plan_stamp;
     return use->mem;
 }
+
+// The remembered call of a cached plan (see PlanSlot::call).
+bool plan_recall(hipStream_t stream, const std::vector<unsigned char> &call, PlanView *view,
+                 bool *staged) {
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) return false;
+    std::lock_guard<std::mutex> lock(g_plan_mutex);
+    for (PlanSlot &slot : g_plan_slots) {
+        if (slot.device != device || slot.stream != stream || slot.call != call) continue;
+        slot.stamp = ++g_plan_stamp;
+        *view = slot.view;
+        *staged = slot.staged;
+        return true;
+    }
+    return false;
+}
+
+void plan_remember(const void *mem, std::vector<unsigned char> &&call, const PlanView &view,
+                   bool staged) {
+    std::lock_guard<std::mutex> lock(g_plan_mutex);
+    for (PlanSlot &slot : g_plan_slots) {
+        if (slot.mem != mem || slot.key.empty()) continue;
+        slot.call = std::move(call);
+        slot.view = view;
+        slot.staged = staged;
+        return;
+    }
+}
+
+// One address per op type: tells the remembered calls of different ops apart.
+template <class Op>
+struct OpTag {
+    static const char tag;
+};
+template <class Op>
+const char OpTag<Op>::tag = 0;
 
 // Memory for the plan of one call, brought by the caller instead of taken from the cache (the
 // entry point that must not allocate).  The plan is rewritten on every call.
@@ -385,6 +429,49 @@ int launch_multi(MakeOp make_op, size_t num_tensors,
     if (n == nullptr) return TOA_ENULL;
     for (int i = 0; i < Op::NPTR; ++i)
         if (lists[i] == nullptr) return TOA_ENULL;
+
+    // A call whose arguments are byte for byte those a cached plan last served: one launch.
+    // (One step count for the whole list, the caller not capturing, plans not switched off;
+    // everything else -- validation, schedule, plan -- was settled when the call was first seen.)
+    std::vector<unsigned char> call;
+    if (counts == nullptr && arena == nullptr && g_plan_mode.load(std::memory_order_relaxed) != 1) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing((hipStream_t)stream, &capturing) == hipSuccess &&
+            capturing == hipStreamCaptureStatusNone) {
+            const uint64_t head[4] = {reinterpret_cast<uintptr_t>(&OpTag<Op>::tag),
+                                      (uint64_t)g_schedule.load(std::memory_order_relaxed),
+                                      (uint64_t)g_plan_mode.load(std::memory_order_relaxed),
+                                      (uint64_t)num_tensors};
+            static_assert(sizeof(size_t) == sizeof(void *), "sizes and pointers copy alike");
+            const size_t row = num_tensors * sizeof(void *);
+            call.resize(sizeof(head) + (Op::NPTR + 1) * row);
+            unsigned char *at = call.data();
+            std::memcpy(at, head, sizeof(head));
+            at += sizeof(head);
+            std::memcpy(at, n, row);
+            at += row;
+            for (int i = 0; i < Op::NPTR; ++i, at += row) std::memcpy(at, lists[i], row);
+            PlanView view;
+            bool staged_before = false;
+            if (plan_recall((hipStream_t)stream, call, &view, &staged_before)) {
+                const Op op = make_op(count_all);
+                const unsigned lds = lds_reservation<Op>(staged_before, view.total, staged_before);
+                if (staged_before) {
+                    if constexpr (IsStaged<Op>::value)
+                        hipLaunchKernelGGL((plan_stream_kernel<T, Op, kUnroll, kNonTemporal, true>),
+                                           dim3(grid_for(view.total)), dim3(kBlock), lds,
+                                           (hipStream_t)stream, op, view);
+                } else {
+                    hipLaunchKernelGGL((plan_stream_kernel<T, Op, kUnroll, kNonTemporal>),
+                                       dim3(grid_for(view.total)), dim3(kBlock), lds,
+                                       (hipStream_t)stream, op, view);
+                }
+                return (int)hipGetLastError();
+            }
+        } else {
+            (void)hipGetLastError();
+        }
+    }
 
     // validate everything before the first launch
     for (size_t k = 0; k < num_tensors; ++k) {
@@ -506,6 +593,7 @@ int launch_multi(MakeOp make_op, size_t num_tensors,
                                        (hipStream_t)stream, op, view);
                 }
                 if (const int rc = (int)hipGetLastError()) return rc;
+                if (arena == nullptr && !call.empty()) plan_remember(mem, std::move(call), view, staged);
                 continue;
             }
         } else if (arena != nullptr) {
