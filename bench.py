@@ -259,10 +259,19 @@ def time_backward_ops(torch, lib, cfg_id, code, dtype, tag, n, esize, eps_root, 
     return res
 
 
-def run_gpu(cfg_id, steps, warmup, operator_preheat=None):
+def run_gpu(cfg_id, steps, warmup, operator_preheat=None, state='library'):
     import torch
 
     from torchopt_amd import _lib
+    from torchopt_amd.placement import state_empty_like
+
+    def moment(host_array, like):
+        """A moment array on the GPU: allocated the way the package's own init allocates state
+        (large arrays 8 KiB off the 16 KiB address phase the allocator gives the gradient), or
+        with --state plain wherever torch's allocator puts it, like the gradient."""
+        if state == 'plain':
+            return host_array.cuda()
+        return state_empty_like(like).copy_(host_array)
 
     if not torch.cuda.is_available():
         raise SystemExit('bench.py needs a GPU: the fused Adam op has no CPU path')
@@ -415,8 +424,9 @@ def run_gpu(cfg_id, steps, warmup, operator_preheat=None):
             us, ms, vs = carve(0)
         else:
             us = [h[0].cuda() for h in host]
-            ms = [h[1].cuda() for h in host]
-            vs = [h[2].cuda() for h in host]
+            ms = [moment(h[1], u) for h, u in zip(host, us)]
+            vs = [moment(h[2], u) for h, u in zip(host, us)]
+            extra['state_allocation'] = state
         step = list_step(us, ms, vs)
         pu, pm, pv = ((ctypes.c_void_p * num)(*[t.data_ptr() for t in ts]) for ts in (us, ms, vs))
         if cfg.get('fused_step'):
@@ -456,10 +466,13 @@ def run_gpu(cfg_id, steps, warmup, operator_preheat=None):
                          three_pass_chain_bytes_per_element=11 * esize)
     else:
         total = cfg['n']
-        u, mu, nu = (a.cuda() for a in host_state(cfg_id, 0, total, cfg['dtype']))
+        h_u, h_mu, h_nu = host_state(cfg_id, 0, total, cfg['dtype'])
+        u = h_u.cuda()
+        mu, nu = moment(h_mu, u), moment(h_nu, u)
         pu, pm, pv = u.data_ptr(), mu.data_ptr(), nu.data_ptr()
 
-        extra = {}
+        extra = {'state_allocation': state,
+                 'address_mod_16KiB': {'updates': pu % 16384, 'mu': pm % 16384, 'nu': pv % 16384}}
         if cfg.get('fresh_gradients'):
             # A training loop hands the step a new gradient every time.  The step overwrites its
             # gradient array with the update, so an array used twice feeds the operator its own
@@ -1148,6 +1161,10 @@ def main(argv=None):
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--config', type=int, default=2, choices=sorted(CONFIGS))
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--state', choices=('library', 'plain'), default='library',
+                    help="how mu and nu are allocated: 'library' = as the package's init does "
+                         '(torchopt_amd.state_zeros_like: large arrays 8 KiB off the 16 KiB '
+                         "address phase of allocator blocks), 'plain' = torch's allocator alone")
     ap.add_argument('--operator-preheat', type=int, default=None,
                     help='launches of the operator on scratch state before the warm-up steps '
                          '(default: 100 for the 16-bit configurations, 0 otherwise)')
@@ -1179,7 +1196,7 @@ def main(argv=None):
 
     host_cores()  # before torch (and with it the OpenMP runtime) loads
 
-    gpu = run_gpu(args.config, args.steps, args.warmup, args.operator_preheat)
+    gpu = run_gpu(args.config, args.steps, args.warmup, args.operator_preheat, args.state)
     cfg = CONFIGS[args.config]
     if args.pmc_calibration:
         import torch

@@ -374,3 +374,43 @@ def test_availability_probe_on_the_gpu():
     assert accelerated_op_available(['cuda', 'cuda:0', 0])
     assert not accelerated_op_available(['cuda', 'meta'])
     assert not accelerated_op_available(['cpu', 'cuda'])  # the CPU is not served here
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float64, torch.bfloat16],
+                         ids=['f32', 'f64', 'bf16'])
+def test_state_of_large_leaves_is_placed_and_steps_like_any_other(dtype):
+    """init puts the moments of a large GPU leaf 8 KiB off the 16 KiB address phase (a view into
+    a slightly larger block), leaves small and non-contiguous leaves to zeros_like, and the steps
+    that follow are the oracle's bit for bit either way."""
+    from torchopt_amd import FusedAdam, state_zeros_like
+
+    n_big = (3 << 20) // torch.empty(0, dtype=dtype).element_size() + 5  # 3 MiB and a ragged end
+    params = [torch.randn(n_big, device='cuda').to(dtype),
+              torch.randn(7, 33, device='cuda').to(dtype),
+              torch.randn(1024, 600, device='cuda').to(dtype).t()]  # large, not contiguous
+    t = scale_by_accelerated_adam(B1, B2, 1e-3, eps_root=0.0)
+    state = t.init(params)
+    for moments in (state.mu, state.nu):
+        big, small, strided = moments
+        assert big.data_ptr() % (16 << 10) == 8 << 10 and big.is_contiguous()
+        assert big.shape == params[0].shape and big.dtype == dtype and not big.any()
+        assert small.storage_offset() == 0 and small.shape == (7, 33)
+        assert strided.stride() == params[2].stride() and strided.storage_offset() == 0
+    assert state_zeros_like(params[0], requires_grad=True).requires_grad
+    if dtype == torch.bfloat16:
+        return  # values of the 16-bit step are covered where its oracle is (test_low_precision_gpu)
+    np_dtype = {torch.float32: np.float32, torch.float64: np.float64}[dtype]
+    h_mu, h_nu = np.zeros(n_big, np_dtype), np.zeros(n_big, np_dtype)
+    for step in (1, 2, 3):
+        g = torch.randn(n_big, device='cuda').to(dtype)
+        h_g = host(g).copy()
+        updates, state = t.update([g, None, None], state, params=params, inplace=True)
+        O.forward_inplace(h_g, h_mu, h_nu, B1, B2, 1e-3, 0.0, step)
+        assert_bit_equal(host(updates[0]), h_g, f'step {step} updates')
+        assert_bit_equal(host(state.mu[0]), h_mu, f'step {step} mu')
+        assert_bit_equal(host(state.nu[0]), h_nu, f'step {step} nu')
+    opt = FusedAdam([torch.nn.Parameter(params[0].clone())], lr=1e-3)
+    opt.param_groups[0][0].grad = torch.randn(n_big, device='cuda').to(dtype)
+    opt.step()
+    s = opt.state_groups[0]
+    assert s.mu[0].data_ptr() % (16 << 10) == 8 << 10 and s.nu[0].data_ptr() % (16 << 10) == 8 << 10

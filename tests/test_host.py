@@ -37,6 +37,7 @@ def test_header_declares_the_expected_surface():
     want |= {'toa_adam_abi_version', 'toa_adam_error_string', 'toa_adam_set_waves_per_cu',
              'toa_adam_fused_step', 'toa_adam_fused_step_multi', 'toa_adam_set_max_grid',
              'toa_adam_set_schedule', 'toa_adam_set_plan_mode', 'toa_adam_release_plans',
+             'toa_adam_state_slack', 'toa_adam_state_shift',
              'toa_adam_forward_inplace_multi_noalloc', 'toa_adam_bias_rows',
              'toa_adam_bias_rows_needed', 'toa_adam_count_advance',
              'toa_adam_forward_inplace_devcount', 'toa_adam_forward_inplace_multi_devcount',
@@ -254,3 +255,23 @@ def test_availability_probe_is_loud_about_the_cpu():
     with pytest.warns(UserWarning, match='no CPU kernels'):
         assert not accelerated_op_available(['cpu', 'cuda'])
     assert not accelerated_op_available('not-a-device')
+
+
+def test_state_placement_advice():
+    """toa_adam_state_shift: the bytes to skip so a state array starts 8 KiB off a 16 KiB phase."""
+    lib = _lib.load()
+    slack = lib.toa_adam_state_slack()
+    assert slack == 16 << 10
+    for base in (0, 256, 8 << 10, (8 << 10) + 512, (16 << 10) - 256, (2 << 20) * 37, 0x7f12_3456_7800):
+        shift = lib.toa_adam_state_shift(base)
+        assert 0 <= shift < slack and shift % 256 == base % 256 == 0
+        assert (base + shift) % slack == 8 << 10
+    # CPU tensors, small tensors and non-contiguous ones are plain zeros_like / empty_like
+    import torch
+
+    from torchopt_amd.placement import state_empty_like, state_zeros_like
+
+    t = torch.ones(3, 5, dtype=torch.float64).t()
+    z = state_zeros_like(t, requires_grad=True)
+    assert z.shape == t.shape and z.stride() == t.stride() and z.requires_grad and not z.any()
+    assert state_empty_like(torch.ones(7)).storage_offset() == 0

@@ -18,7 +18,7 @@ TOA_F32 = 0
 TOA_F64 = 1
 TOA_F16 = 2
 TOA_BF16 = 3
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _vp = ctypes.c_void_p
 _vpp = ctypes.POINTER(ctypes.c_void_p)
@@ -36,6 +36,8 @@ SIGNATURES = {
     'toa_adam_set_schedule': [_i],
     'toa_adam_set_plan_mode': [_i],
     'toa_adam_release_plans': [],
+    'toa_adam_state_slack': [],
+    'toa_adam_state_shift': [_vp],
     'toa_adam_forward_inplace': [_i, _vp, _vp, _vp, _sz, _d, _d, _d, _d, _u64, _vp],
     'toa_adam_forward_mu': [_i, _vp, _vp, _sz, _d, _vp, _vp],
     'toa_adam_forward_nu': [_i, _vp, _vp, _sz, _d, _vp, _vp],
@@ -112,7 +114,9 @@ def load() -> ctypes.CDLL:
         for name, argtypes in SIGNATURES.items():
             fn = getattr(lib, name)
             fn.restype = {'toa_adam_set_max_grid': ctypes.c_uint,
-                          'toa_adam_bias_rows_needed': ctypes.c_size_t}.get(name, _i)
+                          'toa_adam_bias_rows_needed': ctypes.c_size_t,
+                          'toa_adam_state_slack': ctypes.c_size_t,
+                          'toa_adam_state_shift': ctypes.c_size_t}.get(name, _i)
             fn.argtypes = argtypes
         _lib = lib
     return _lib

@@ -147,6 +147,9 @@ bool arrays_disjoint(T *const (&ptrs)[NPTR], size_t n) {
     return true;
 }
 
+// Where state arrays should begin, as an address modulo kStatePeriod (see toa_adam_state_shift).
+constexpr uintptr_t kStatePeriod = 16 << 10, kStatePhase = 8 << 10;
+
 // Workgroups per launch are capped; a tensor with more tiles than the cap is covered by the
 // kernels' stride loop.  The cap is adjustable so that path can be exercised on small inputs.
 std::atomic<unsigned> g_max_grid{kMaxGrid};
@@ -769,7 +772,15 @@ int backward_all_multi(size_t num, const void *const *dnew_updates,
 
 extern "C" {
 
-int toa_adam_abi_version(void) { return 3; }
+int toa_adam_abi_version(void) { return 4; }
+
+// Preferred placement of state arrays: 8 KiB off the 16 KiB phase that large allocations share.
+size_t toa_adam_state_slack(void) { return kStatePeriod; }
+
+size_t toa_adam_state_shift(const void *allocation) {
+    const uintptr_t at = reinterpret_cast<uintptr_t>(allocation) % kStatePeriod;
+    return (size_t)((kStatePhase + kStatePeriod - at) % kStatePeriod);
+}
 
 int toa_adam_set_waves_per_cu(int waves) {
     const int prev = waves_override();
