@@ -57,9 +57,9 @@ BYTES_PER_ELEM = {  # op -> number of arrays streamed (multiply by the element s
 # figures belong to the kernels as they were when the profile was taken; re-record them whenever
 # adam_kernels.hpp or the launch shape changes.
 RECORDED_TRAFFIC = {
-    2: (6442411158, 'profiles/forward_inplace_f32_config2_pmc_traffic.md'),
-    4: (8516318272, 'profiles/forward_inplace_multi_f32_config4_kernel_trace_and_traffic.md'),
-    5: (9935405910, 'profiles/fused_step_multi_f32_config5_kernel_trace_and_traffic.md'),
+    2: (6442420201, 'profiles/forward_inplace_f32_config2_pmc_traffic.md'),
+    4: (8516224043, 'profiles/forward_inplace_multi_f32_config4_kernel_trace_and_traffic.md'),
+    5: (9935413118, 'profiles/fused_step_multi_f32_config5_kernel_trace_and_traffic.md'),
 }
 
 B1, B2, EPS = 0.9, 0.999, 1e-8
