@@ -264,3 +264,23 @@ def test_a_remembered_call_is_only_taken_for_the_very_same_arguments():
         O.forward_inplace(h['updates'][i], h['mu'][i], h['nu'][i], B1, B2, EPS, 0.0, 21)
     check_lists(g['updates'], h['updates'], 'replayed capture updates')
     check_lists(g['mu'], h['mu'], 'replayed capture mu')
+
+
+@pytest.mark.parametrize('sizes_of', ['ragged', 'one_tile_or_less', 'a_giant_among_thousands'])
+def test_thousands_of_small_tensors_start_from_the_finer_index(sizes_of):
+    """More records than twice the cells of the launch's coarse index: the plan carries a finer
+    index in device memory and waves start from that.  Checked like every other list, over two
+    steps (plan written, then found in the cache and the call remembered)."""
+    rng = np.random.default_rng(11)
+    if sizes_of == 'ragged':
+        sizes = [int(x) for x in rng.integers(0, 3000, size=6000)]
+    elif sizes_of == 'one_tile_or_less':
+        sizes = [int(x) for x in rng.integers(1, 257, size=4000)]
+    else:
+        sizes = [int(x) for x in rng.integers(1, 600, size=5000)]
+        sizes[2500] = 256 * 40_000 + 17  # shifts the index to coarser entries
+    h = make_lists(np.float32, sizes, 12)
+    g = to_dev(h)
+    print(f'{len(sizes)} small tensors ({sizes_of}) through a plan with a finer index', flush=True)
+    for step in (1, 2, 3):
+        step_and_check(g, h, step, f'{sizes_of} step {step}')

@@ -503,6 +503,9 @@ __device__ __forceinline__ float load_uniform(const float *p) {
 __device__ __forceinline__ double load_uniform(const double *p) {
     return *(const __attribute__((address_space(4))) double *)p;
 }
+__device__ __forceinline__ uint32_t load_uniform(const uint32_t *p) {
+    return *(const __attribute__((address_space(4))) uint32_t *)p;
+}
 __device__ __forceinline__ int64_t load_uniform(const int64_t *p) {
     return *(const __attribute__((address_space(4))) int64_t *)p;
 }
@@ -1467,10 +1470,15 @@ constexpr int kPlanCells = 832;  // 3328 bytes of kernel arguments
 
 struct PlanView {
     const PlanRec *recs;
-    uint32_t total;  // tiles
-    uint32_t shift;  // log2 of the tiles per cell
-    uint32_t num;    // records
-    uint32_t reserved;
+    // Lists of thousands of small tensors: 832 cells would leave dozens of records per cell for a
+    // wave to walk, so such a plan carries a finer index of the same kind in device memory (one
+    // entry per 2^fine_shift tiles, about two to four entries per record) and waves start from
+    // that; nullptr for every other list.
+    const uint32_t *fine;
+    uint32_t total;       // tiles
+    uint32_t shift;       // log2 of the tiles per cell
+    uint32_t num;         // records
+    uint32_t fine_shift;  // log2 of the tiles per entry of `fine`
     uint32_t cell[kPlanCells];  // record that owns tile (i << shift)
 };
 
@@ -1507,6 +1515,26 @@ __global__ __launch_bounds__(128) void plan_fill_kernel(PlanRec *recs, uint32_t 
 static_assert(PlanSeedChunk<kPlanSlots>::MAX >= 1 && PlanSeedChunk<3>::MAX <= 128,
               "one fill workgroup covers a chunk");
 
+// The finer index of a plan with very many records: entry c = the record that owns tile
+// c << shift, found by bisection over the records' first tiles (strictly increasing: a plan holds
+// non-empty tensors only).
+__global__ __launch_bounds__(256) void plan_index_kernel(const PlanRec *recs, uint32_t num,
+                                                         uint32_t *fine, uint32_t entries,
+                                                         uint32_t shift) {
+    const uint32_t c = blockIdx.x * 256u + threadIdx.x;
+    if (c >= entries) return;
+    const uint32_t tile = c << shift;
+    uint32_t lo = 0, hi = num - 1;  // the largest k with recs[k].first <= tile
+    while (lo < hi) {
+        const uint32_t mid = lo + (hi - lo + 1) / 2;
+        if (recs[mid].first <= tile)
+            lo = mid;
+        else
+            hi = mid - 1;
+    }
+    fine[c] = lo;
+}
+
 // A record read at a wave-uniform address from memory no kernel writes while this one runs:
 // through the constant address space, so the scalar unit fetches it (three 32-byte loads).
 __device__ __forceinline__ PlanRec load_record(const PlanRec *at) {
@@ -1531,7 +1559,9 @@ __global__ __launch_bounds__(kBlock) void plan_stream_kernel(const Op op, const 
     // a wave's first dependent fetch is its cell, not the total.
     uint32_t tile = blockIdx.x;
     do {
-        PlanRec rec = load_record(plan.recs + plan.cell[tile >> plan.shift]);
+        const uint32_t start = plan.fine != nullptr ? load_uniform(plan.fine + (tile >> plan.fine_shift))
+                                                    : plan.cell[tile >> plan.shift];
+        PlanRec rec = load_record(plan.recs + start);
         // All twelve words of the record are fetched now, in one go (three 32-byte scalar loads
         // in flight together): left alone, the compiler fetches the four words the walk below
         // tests, waits, and only then fetches the pointers -- one more round trip to the scalar

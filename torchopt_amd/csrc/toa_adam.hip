@@ -239,9 +239,24 @@ constexpr uint64_t kPlanFromTiles = 1u << 18;  // 256 MiB of 1 KiB tiles per arr
 constexpr size_t kPlanSlotsPerStream = 4;         // cached plans a stream may hold
 constexpr size_t kPlanSlotsTotal = 64;            // and the process as a whole
 
-size_t plan_bytes(size_t num) { return num * sizeof(PlanRec); }
+// A plan of more than kPlanFineFrom records carries a finer index behind its records: one entry
+// per 2^shift tiles, the smallest shift that leaves at most four entries per record.
+constexpr size_t kPlanFineFrom = 2 * kPlanCells;
 
-// Writes the records for `seeds` into `mem` (device memory of at least plan_bytes(seeds.size()))
+uint32_t plan_fine_entries(size_t num, uint64_t total_tiles, uint32_t *shift) {
+    *shift = 0;
+    if (num <= kPlanFineFrom) return 0;
+    while (((total_tiles + ((uint64_t)1 << *shift) - 1) >> *shift) > 4 * (uint64_t)num) ++*shift;
+    return (uint32_t)((total_tiles + ((uint64_t)1 << *shift) - 1) >> *shift);
+}
+
+size_t plan_record_bytes(size_t num) { return (num * sizeof(PlanRec) + 255) / 256 * 256; }
+// records, then the finer index (if any)
+size_t plan_bytes(size_t num, uint32_t fine_entries) {
+    return plan_record_bytes(num) + (size_t)fine_entries * sizeof(uint32_t);
+}
+
+// Writes the records for `seeds` into `mem` (device memory of at least plan_record_bytes(seeds.size()))
 // on `stream`: fill kernels carrying the records in their arguments.
 template <int NPTR>
 int plan_write(void *mem, const std::vector<PlanSeed<NPTR>> &seeds, hipStream_t stream) {
@@ -259,14 +274,21 @@ int plan_write(void *mem, const std::vector<PlanSeed<NPTR>> &seeds, hipStream_t 
     return 0;
 }
 
-// The launch's view of a plan: the coarse index from tile cells to records.
+// The launch's view of a plan: the coarse index from tile cells to records, and the finer one in
+// device memory where the plan has it (`with_fine`: plans from the cache; a caller's arena holds
+// records only).
 template <int NPTR>
-PlanView plan_view(void *mem, const std::vector<PlanSeed<NPTR>> &seeds, uint32_t total) {
+PlanView plan_view(void *mem, const std::vector<PlanSeed<NPTR>> &seeds, uint32_t total,
+                   bool with_fine) {
     PlanView v;
     v.recs = static_cast<const PlanRec *>(mem);
     v.total = total;
     v.num = (uint32_t)seeds.size();
-    v.reserved = 0;
+    v.fine = nullptr;
+    v.fine_shift = 0;
+    if (with_fine && plan_fine_entries(seeds.size(), total, &v.fine_shift) != 0)
+        v.fine = reinterpret_cast<const uint32_t *>(static_cast<const char *>(mem) +
+                                                   plan_record_bytes(seeds.size()));
     v.shift = 0;
     while ((((uint64_t)total + (1u << v.shift) - 1) >> v.shift) > (uint64_t)kPlanCells) ++v.shift;
     uint32_t k = 0;
@@ -333,7 +355,10 @@ void *plan_cached(const std::vector<PlanSeed<NPTR>> &seeds, size_t tile, hipStre
         use->stamp = ++g_plan_stamp;
         return use->mem;
     }
-    const size_t need = plan_bytes(seeds.size());
+    const uint64_t total_tiles = seeds.empty() ? 0 : seeds.back().next_first;
+    uint32_t fine_shift = 0;
+    const uint32_t fine_entries = plan_fine_entries(seeds.size(), total_tiles, &fine_shift);
+    const size_t need = plan_bytes(seeds.size(), fine_entries);
     if (mine >= kPlanSlotsPerStream || (oldest != nullptr && g_plan_slots.size() >= kPlanSlotsTotal)) {
         use = oldest;
         if (use->capacity < need) {
@@ -364,6 +389,14 @@ void *plan_cached(const std::vector<PlanSeed<NPTR>> &seeds, size_t tile, hipStre
     use->key.clear();
     use->call.clear();
     *rc = plan_write<NPTR>(use->mem, seeds, stream);
+    if (*rc == 0 && fine_entries != 0) {
+        hipLaunchKernelGGL(plan_index_kernel, dim3((fine_entries + 255) / 256), dim3(256), 0, stream,
+                           static_cast<const PlanRec *>(use->mem), (uint32_t)seeds.size(),
+                           reinterpret_cast<uint32_t *>(static_cast<char *>(use->mem) +
+                                                        plan_record_bytes(seeds.size())),
+                           fine_entries, fine_shift);
+        *rc = (int)hipGetLastError();
+    }
     if (*rc) return nullptr;
     use->key = std::move(key);
     use->stamp = ++g_plan_stamp;
@@ -569,7 +602,7 @@ int launch_multi(MakeOp make_op, size_t num_tensors,
             }
             void *mem = nullptr;
             if (arena != nullptr) {
-                if (plan_bytes(live) > arena->bytes) return TOA_ELIMIT;
+                if (plan_bytes(live, 0) > arena->bytes) return TOA_ELIMIT;
                 if (const int rc = plan_write<Op::NPTR>(arena->mem, seeds, (hipStream_t)stream))
                     return rc;
                 mem = arena->mem;
@@ -580,7 +613,7 @@ int launch_multi(MakeOp make_op, size_t num_tensors,
             }
             if (mem != nullptr) {
                 const uint32_t total = (uint32_t)tiles_all;
-                const PlanView view = plan_view<Op::NPTR>(mem, seeds, total);
+                const PlanView view = plan_view<Op::NPTR>(mem, seeds, total, arena == nullptr);
                 // the lookup is two scalar-cache hits, so a plain launch wants the residency
                 // level of the single-tensor kernel, not the table kernel's raised one; a staged
                 // launch takes the op's level for staged lists
