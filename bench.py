@@ -850,6 +850,64 @@ def run_placements(reps=10, n=1 << 28, ladder=None):
             'device': torch.cuda.get_device_name(0), 'GB/s_by_placement': grid}
 
 
+def run_state_phases(reps=12, n=1 << 28, step_kib=2, span_kib=32):
+    """The operator (float32 forward_ in place, 2^28 elements, library defaults) on three SEPARATE
+    PyTorch allocations -- what a training loop hands it -- with mu and nu shifted inside their own
+    allocations by every pair of phases from 0 to `span_kib` in steps of `step_kib`; the gradient
+    stays where the allocator put it (a 2 MiB boundary).  After every row the unshifted placement
+    is timed again, so a drift of the machine over the run shows.  This is the measurement behind
+    the phase at which the package allocates state (toa_adam_state_shift)."""
+    import torch
+
+    from torchopt_amd import _lib
+
+    lib = _lib.load()
+    stream = torch.cuda.current_stream()
+    pad = span_kib * 256
+    u = torch.empty(n, device='cuda')
+    mu_block = torch.empty(n + pad, device='cuda')
+    nu_block = torch.empty(n + pad, device='cuda')
+    preheat(torch)
+
+    def timed(a_kib, b_kib):
+        mu = mu_block[a_kib * 256:a_kib * 256 + n]
+        nu = nu_block[b_kib * 256:b_kib * 256 + n]
+        u.normal_()
+        mu.normal_(0, 0.1)
+        nu.normal_(0, 0.01).abs_()
+        ptrs = (u.data_ptr(), mu.data_ptr(), nu.data_ptr())
+
+        def launch():
+            rc = lib.toa_adam_forward_inplace(_lib.TOA_F32, *ptrs, n, B1, B2, EPS, 0.0, 1000,
+                                              stream.cuda_stream)
+            if rc:
+                raise RuntimeError(lib.toa_adam_error_string(rc).decode())
+        for _ in range(3):
+            launch()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record(stream)
+        for _ in range(reps):
+            launch()
+        ev1.record(stream)
+        torch.cuda.synchronize()
+        return 24 * n / (ev0.elapsed_time(ev1) / reps) / 1e6
+
+    phases = list(range(0, span_kib, step_kib))
+    grid, unshifted = {}, []
+    for a in phases:
+        grid[f'mu +{a} KiB'] = {f'nu +{b} KiB': round(timed(a, b)) for b in phases}
+        unshifted.append(round(timed(0, 0)))
+    shift = lib.toa_adam_state_shift(0) // 1024
+    return {'metric': 'forward_inplace_f32_by_state_phase', 'unit': 'GB/s', 'peak': HBM_PEAK_GBS,
+            'elements': n, 'launches_timed': reps, 'device': torch.cuda.get_device_name(0),
+            'address_mod_16KiB': {'updates': u.data_ptr() % 16384,
+                                  'mu_block': mu_block.data_ptr() % 16384,
+                                  'nu_block': nu_block.data_ptr() % 16384},
+            'library_phase_kib': shift,
+            'at_library_phase': grid[f'mu +{shift} KiB'][f'nu +{shift} KiB'],
+            'unshifted_after_each_row': unshifted, 'GB/s_by_phase': grid}
+
+
 # ----------------------------------------------------------------------------- CPU baseline
 
 
@@ -1179,6 +1237,10 @@ def main(argv=None):
                     help='time the operator over 210 placements of its three arrays inside one '
                          'allocation instead of the benchmark (the rate depends on the '
                          'distances between the arrays)')
+    ap.add_argument('--state-phases', action='store_true',
+                    help='time the operator on three separate allocations with mu and nu shifted '
+                         'inside theirs by every pair of phases below 32 KiB (steps of 2 KiB): '
+                         'the measurement behind the phase at which the package allocates state')
     args = ap.parse_args(argv)
 
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
@@ -1192,6 +1254,9 @@ def main(argv=None):
         return 0
     if args.placements:
         print(json.dumps(run_placements()), flush=True)
+        return 0
+    if args.state_phases:
+        print(json.dumps(run_state_phases()), flush=True)
         return 0
 
     host_cores()  # before torch (and with it the OpenMP runtime) loads

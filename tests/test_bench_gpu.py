@@ -51,3 +51,14 @@ def test_placement_sweep_runs():
     assert 0 < out['min'] <= out['median'] <= out['max']
     assert set(out['GB/s_by_placement']) == {'mu +0 KiB', 'mu +8 KiB', 'mu +64 KiB'}
     torch.cuda.empty_cache()
+
+
+def test_state_phase_sweep_runs():
+    """The operator on separate allocations with the moments at a grid of phases
+    (`bench.py --state-phases`), on small arrays and a coarse grid."""
+    out = bench.run_state_phases(reps=2, n=1 << 22, step_kib=8, span_kib=16)
+    assert out['unit'] == 'GB/s' and out['library_phase_kib'] == 8
+    assert set(out['GB/s_by_phase']) == {'mu +0 KiB', 'mu +8 KiB'}
+    assert out['at_library_phase'] == out['GB/s_by_phase']['mu +8 KiB']['nu +8 KiB'] > 0
+    assert len(out['unshifted_after_each_row']) == 2
+    torch.cuda.empty_cache()
