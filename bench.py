@@ -424,8 +424,16 @@ def run_gpu(cfg_id, steps, warmup, operator_preheat=None, state='library'):
             us, ms, vs = carve(0)
         else:
             us = [h[0].cuda() for h in host]
-            ms = [moment(h[1], u) for h, u in zip(host, us)]
-            vs = [moment(h[2], u) for h, u in zip(host, us)]
+            if state == 'plain':
+                ms = [h[1].cuda() for h in host]
+                vs = [h[2].cuda() for h in host]
+            else:  # as the package's init allocates the moments of a tree
+                from torchopt_amd.placement import state_zeros_like_tree
+
+                ms, vs = state_zeros_like_tree(us)
+                for h, m, v in zip(host, ms, vs):
+                    m.copy_(h[1])
+                    v.copy_(h[2])
             extra['state_allocation'] = state
         step = list_step(us, ms, vs)
         pu, pm, pv = ((ctypes.c_void_p * num)(*[t.data_ptr() for t in ts]) for ts in (us, ms, vs))

@@ -397,6 +397,23 @@ def test_state_of_large_leaves_is_placed_and_steps_like_any_other(dtype):
         assert small.storage_offset() == 0 and small.shape == (7, 33)
         assert strided.stride() == params[2].stride() and strided.storage_offset() == 0
     assert state_zeros_like(params[0], requires_grad=True).requires_grad
+    # the large leaves of a tree share one block: first moments, then second moments, disjoint,
+    # a leaf's two moments clear of the multiples of 16 MiB at which arrays collide in DRAM
+    from torchopt_amd import state_zeros_like_tree
+    tree = [params[0], None, params[1], torch.empty(5 << 20, device='cuda', dtype=dtype), params[2]]
+    mu, nu = state_zeros_like_tree(tree, requires_grad=True)
+    assert mu[1] is None and nu[1] is None and mu[2].shape == (7, 33) and mu[4].stride() == params[2].stride()
+    placed = [mu[0], mu[3], nu[0], nu[3]]
+    assert len({x.untyped_storage().data_ptr() for x in placed}) == 1
+    spans = sorted((x.data_ptr(), x.data_ptr() + x.numel() * x.element_size()) for x in placed)
+    assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:]))
+    assert [x.data_ptr() for x in placed] == sorted(x.data_ptr() for x in placed)
+    for got, like in zip(placed, (tree[0], tree[3], tree[0], tree[3])):
+        assert got.data_ptr() % (16 << 10) == 8 << 10 and got.shape == like.shape
+        assert got.requires_grad and got.dtype == dtype and not got.any()
+    apart = (nu[3].data_ptr() - mu[3].data_ptr()) % (16 << 20)
+    assert nu[0].data_ptr() - mu[0].data_ptr() == nu[3].data_ptr() - mu[3].data_ptr()
+    assert (3 << 20) <= apart <= (13 << 20)
     if dtype == torch.bfloat16:
         return  # values of the 16-bit step are covered where its oracle is (test_low_precision_gpu)
     np_dtype = {torch.float32: np.float32, torch.float64: np.float64}[dtype]

@@ -275,3 +275,8 @@ def test_state_placement_advice():
     z = state_zeros_like(t, requires_grad=True)
     assert z.shape == t.shape and z.stride() == t.stride() and z.requires_grad and not z.any()
     assert state_empty_like(torch.ones(7)).storage_offset() == 0
+    from torchopt_amd.placement import state_zeros_like_tree
+
+    mu, nu = state_zeros_like_tree([torch.ones(1 << 19), None, t], requires_grad=True)
+    assert mu[1] is None and nu[1] is None and mu[0].storage_offset() == 0 and nu[2].stride() == t.stride()
+    assert all(x.requires_grad and not x.any() for x in (mu[0], nu[0], mu[2], nu[2]))

@@ -40,7 +40,7 @@ import torch
 
 from torchopt_amd.accelerated_op.adam_op import adam_op
 from torchopt_amd.base import accelerated_only
-from torchopt_amd.placement import state_zeros_like
+from torchopt_amd.placement import state_zeros_like_tree
 from torchopt_amd.transform.scale_by_adam import (INT64_MAX, ScaleByAdamState, _host_value,
                                                  _remember)
 
@@ -179,8 +179,8 @@ class FusedAdam:
                                     0) for p in group)
         self._steps[i] = [0] * len(group)
         self._stale[i] = False
-        return ScaleByAdamState(mu=tuple(state_zeros_like(p) for p in group),
-                                nu=tuple(state_zeros_like(p) for p in group), count=count)
+        mu, nu = state_zeros_like_tree(group)
+        return ScaleByAdamState(mu=tuple(mu), nu=tuple(nu), count=count)
 
     def _sync_counts(self, i: int) -> None:
         """Bring the 0-dim device count tensors of group `i` up to the host's step numbers.

@@ -9,6 +9,11 @@ gradient's phase the float32 step on 2^28 elements runs 0.8-1.0 % faster, 4 and 
 slow distances, and nothing measured is slower at 8 KiB than at 0.  The state this package
 allocates therefore starts at that phase (``toa_adam_state_shift`` of the C ABI names it);
 values, shapes, dtypes and contiguity are those of ``zeros_like``.
+
+A tree's moments come from ONE block per (device, dtype): every mu, then every nu, each leaf at
+the phase, so the slack is 16 KiB per leaf instead of what the allocator's rounding would add to
+separate blocks (2 MiB on a 16 MiB leaf), and a leaf's two moments lie a distance apart that is
+kept clear of the multiples of 16 MiB at which three arrays meet in the same DRAM banks.
 """
 
 from __future__ import annotations
@@ -46,3 +51,59 @@ def state_zeros_like(t: torch.Tensor, *, requires_grad: bool = False) -> torch.T
 def state_empty_like(t: torch.Tensor, *, requires_grad: bool = False) -> torch.Tensor:
     """``empty_like(t)`` at the preferred phase."""
     return _placed(t, False, requires_grad)
+
+
+_COLLISION_PERIOD = 16 << 20   # arrays a multiple of this apart (within 1.5 MiB) collide in DRAM
+_CLEAR_FROM, _CLEAR_TO = 3 << 20, 13 << 20
+
+
+def _eligible(t) -> bool:
+    return (t is not None and t.is_cuda and t.layout == torch.strided and t.is_contiguous()
+            and t.numel() * t.element_size() >= MIN_BYTES)
+
+
+def state_zeros_like_tree(leaves, *, requires_grad: bool = False):
+    """``([zeros_like(t) for t in leaves], [zeros_like(t) for t in leaves])`` -- both moments of
+    a flattened tree (``None`` leaves stay ``None``).  The large contiguous GPU leaves of one
+    device and dtype share one block: all first moments, then all second moments, every leaf at
+    the preferred phase.  Other leaves get plain ``zeros_like``."""
+    leaves = list(leaves)
+    mu = [None] * len(leaves)
+    nu = [None] * len(leaves)
+    groups: dict = {}
+    for k, t in enumerate(leaves):
+        if t is None:
+            continue
+        if _eligible(t):
+            groups.setdefault((t.device, t.dtype), []).append(k)
+        else:
+            mu[k] = torch.zeros_like(t, requires_grad=requires_grad)
+            nu[k] = torch.zeros_like(t, requires_grad=requires_grad)
+    if not groups:
+        return mu, nu
+    lib = _lib.load()
+    period = lib.toa_adam_state_slack()
+    for (device, dtype), members in groups.items():
+        es = leaves[members[0]].element_size()
+        sizes = [leaves[k].numel() * es for k in members]
+        # byte offsets from the first leaf's start, every leaf a whole number of periods on
+        offsets, end = [], 0
+        for n in sizes:
+            end = -(-end // period) * period
+            offsets.append(end)
+            end += n
+        second = -(-end // period) * period  # where the second moments start
+        if max(sizes) >= (4 << 20):  # smaller arrays sit in cache and do not collide
+            apart = second % _COLLISION_PERIOD
+            if apart < _CLEAR_FROM:
+                second += _CLEAR_FROM - apart
+            elif apart > _CLEAR_TO:
+                second += _COLLISION_PERIOD + _CLEAR_FROM - apart
+        block = torch.zeros((second + end + period) // es, dtype=dtype, device=device)
+        first = lib.toa_adam_state_shift(block.data_ptr())
+        for k, off in zip(members, offsets):
+            n, shape = leaves[k].numel(), leaves[k].shape
+            a, b = (first + off) // es, (first + second + off) // es
+            mu[k] = block[a:a + n].view(shape).requires_grad_(requires_grad)
+            nu[k] = block[b:b + n].view(shape).requires_grad_(requires_grad)
+    return mu, nu
