@@ -103,16 +103,17 @@ CONFIGS = {
             dtype='f32', shapes=maml_shapes(), eps_root=1e-8, count=5, differentiable=True),
     2: dict(name='config2: fused forward_ in place, 268 435 456 float32 elements '
                  '(1 GiB per state array), count=1000',
-            dtype='f32', n=1 << 28, eps_root=0.0, count=1000),
+            dtype='f32', n=1 << 28, eps_root=0.0, count=1000, operator_preheat=60),
     3: dict(name='config3: fused forward_ in place, 67 108 864 float64 elements, count=3; beside '
                  'it the backward ops on the same shapes',
-            dtype='f64', n=1 << 26, eps_root=1e-8, count=3, backward=True),
+            dtype='f64', n=1 << 26, eps_root=1e-8, count=3, backward=True, operator_preheat=60),
     4: dict(name='config4: multi-tensor forward_ in place over the GPT-2-medium parameter list '
                  '(float32), count=1',
-            dtype='f32', shapes=gpt2_medium_shapes(), eps_root=0.0, count=1),
+            dtype='f32', shapes=gpt2_medium_shapes(), eps_root=0.0, count=1, operator_preheat=60),
     5: dict(name='config5: classic optimizer step (Adam + scale(-lr) + apply) in one pass over the '
                  'GPT-2-medium parameter list (float32), count=1; beside it the three-pass chain',
-            dtype='f32', shapes=gpt2_medium_shapes(), eps_root=0.0, count=1, fused_step=True),
+            dtype='f32', shapes=gpt2_medium_shapes(), eps_root=0.0, count=1, fused_step=True,
+            operator_preheat=60),
     6: dict(name='config6: fused forward_ in place, 268 435 456 float16 elements (arithmetic of '
                  'the reference CPU op on at::Half: every operation rounded to 16 bits), '
                  'eps=1e-3, count=1000, a fresh N(0,1) gradient array every step',
@@ -128,7 +129,7 @@ CONFIGS = {
                  'contiguous, so the three arrays of every leaf lie exactly 1 GiB = 64 x 16 MiB '
                  'apart and meet in the same DRAM banks; count=1',
             dtype='f32', shapes=[(4096, 1024)] * 64, eps_root=0.0, count=1,
-            lists_contiguous=True),
+            lists_contiguous=True, operator_preheat=60),
     9: dict(name='config9: classic optimizer step (Adam + scale(-lr) + apply) in one pass over the '
                  'GPT-2-medium parameter list in bfloat16 (parameters, gradients and both moments), '
                  'eps=1e-3, count=1; beside it the three-pass chain',
@@ -534,22 +535,31 @@ def run_gpu(cfg_id, steps, warmup, operator_preheat=None, state='library'):
             extra['cold_cache_ms_per_launch'] = round(sorted(cold)[len(cold) // 2], 5)
 
     extra['preheat_launches_on_scratch_arrays'] = preheat(torch)
-    # The 16-bit kernels (more arithmetic per byte) take another ~50 ms of their OWN kind of load
-    # to reach their steady rate, whatever ran before: the first 40-50 steps of a run are up to
-    # 6 % slower, isolated steps on the initial and on a late state take the same time, and 100
-    # launches of the operator on scratch arrays beforehand remove the transient.  So those
-    # configurations preheat with the operator too -- on scratch state, never the benchmark's.
+    # The first launches of the operator in a process are not its steady state, whatever ran
+    # before: launches 1-2 run at the steady rate, launches 4-8 up to 4 % slower (float32 in place:
+    # 0.948, 0.953, 0.960 ... 0.985 ms), and the time settles back over the next 15 (float32) to
+    # 45 (16-bit types) launches -- the clocks boost and settle under this kernel's own mix of
+    # arithmetic and traffic.  Isolated steps on the initial and on a late state take the same
+    # time, so it is not the data.  The bandwidth-bound configurations therefore run the operator
+    # on SCRATCH state of the same shape before the warm-up steps (never on the benchmark's own:
+    # the in-place step would consume it); a fused step, which only reads its gradients, preheats
+    # on its own lists like any warm-up step would.  --operator-preheat 0 switches it off.
     op_launches = cfg.get('operator_preheat', 0) if operator_preheat is None else operator_preheat
-    if op_launches and 'shapes' in cfg:
-        # on the benchmark's own lists with the gradients only read: a fused step preheats on
-        # its state like any warm-up step would (list configurations without a fused step have
-        # no operator preheat)
-        if cfg.get('fused_step'):
-            for _ in range(op_launches):
-                step()
-            torch.cuda.synchronize()
-            extra['preheat_operator_launches'] = op_launches
-    elif op_launches:
+    if op_launches and cfg.get('fused_step'):
+        for _ in range(op_launches):
+            step()
+        torch.cuda.synchronize()
+        extra['preheat_operator_launches'] = op_launches
+    elif op_launches and 'shapes' in cfg and not cfg.get('differentiable'):
+        scratch = [[torch.randn(n, device='cuda').mul_(scale).abs_().to(dtype) for n in sizes]
+                   for scale in (1.0, 0.1, 0.01)]
+        scratch_step = list_step(*scratch)
+        for _ in range(op_launches):
+            scratch_step()
+        torch.cuda.synchronize()
+        del scratch, scratch_step
+        extra['preheat_operator_launches_on_scratch_state'] = op_launches
+    elif op_launches and 'shapes' not in cfg:
         sg = [torch.randn(total, device='cuda').to(dtype) for _ in range(4)]
         sm = (torch.randn(total, device='cuda') * 0.1).to(dtype)
         sv = (torch.randn(total, device='cuda') * 0.01).abs_().to(dtype)
@@ -1233,7 +1243,8 @@ def main(argv=None):
                          "address phase of allocator blocks), 'plain' = torch's allocator alone")
     ap.add_argument('--operator-preheat', type=int, default=None,
                     help='launches of the operator on scratch state before the warm-up steps '
-                         '(default: 100 for the 16-bit configurations, 0 otherwise)')
+                         '(default: 100 for the 16-bit configurations, 60 for the other '
+                         'bandwidth-bound ones, 0 for configs 0 and 1)')
     ap.add_argument('--pmc-calibration', action='store_true',
                     help='after the timed region also run 5 plain device copies of 1 GiB, so a '
                          'rocprofv3 --pmc run holds a kernel of known traffic to scale '
