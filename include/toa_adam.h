@@ -59,8 +59,9 @@ TOA_API int toa_adam_abi_version(void);
 
 /* Tuning knob: how many single-wave workgroups of these kernels may be resident
  * on one compute unit.  The kernels are HBM-bound and run fastest with a bounded
- * number of bytes in flight; each op has its own measured default (12 for the
- * in-place step, 18-32 for the out-of-place ops).  2..32 overrides the default
+ * number of bytes in flight; each op has its own measured default (18 for the
+ * in-place step in its staged schedule, 12 in the plain one, 16-32 for the
+ * out-of-place ops).  2..32 overrides the default
  * of every op, anything else restores the per-op defaults.  The cap works
  * through LDS granules, so the levels that exist are 32, 25, 21, 18, 16, 14,
  * 12, 11, 10, 9, 8 ...; a value in between selects the next level below it.  The environment

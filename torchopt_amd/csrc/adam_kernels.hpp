@@ -18,7 +18,8 @@
 //     reservation made at launch): more bytes in flight than the memory
 //     system needs only lengthens queues and widens the window.  LDS granules
 //     make 32, 25, 21, 18, 16, 14, 12, 11, 10 ... the levels that exist; the
-//     in-place step peaks at 12 waves per CU, the out-of-place ops at 18-32;
+//     in-place step peaks at 18 waves per CU in its staged schedule (12 in the plain one), the
+//     out-of-place ops at 16-32;
 //   * every array is touched once, so loads and stores carry the
 //     non-temporal hint (worth ~10 %);
 //   * the in-place step runs a staged schedule (tile_full_staged): one memory
