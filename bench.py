@@ -57,9 +57,9 @@ BYTES_PER_ELEM = {  # op -> number of arrays streamed (multiply by the element s
 # figures belong to the kernels as they were when the profile was taken; re-record them whenever
 # adam_kernels.hpp or the launch shape changes.
 RECORDED_TRAFFIC = {
-    2: (6442430077, 'profiles/forward_inplace_f32_config2_pmc_traffic.md'),
-    4: (8516224605, 'profiles/forward_inplace_multi_f32_config4_kernel_trace_and_traffic.md'),
-    5: (9935420999, 'profiles/fused_step_multi_f32_config5_kernel_trace_and_traffic.md'),
+    2: (6442426275, 'profiles/forward_inplace_f32_config2_pmc_traffic.md'),
+    4: (8516207551, 'profiles/forward_inplace_multi_f32_config4_kernel_trace_and_traffic.md'),
+    5: (9935417258, 'profiles/fused_step_multi_f32_config5_kernel_trace_and_traffic.md'),
 }
 
 B1, B2, EPS = 0.9, 0.999, 1e-8
@@ -260,19 +260,25 @@ def time_backward_ops(torch, lib, cfg_id, code, dtype, tag, n, esize, eps_root, 
     return res
 
 
-def run_gpu(cfg_id, steps, warmup, operator_preheat=None, state='library'):
+def run_gpu(cfg_id, steps, warmup, operator_preheat=None, state='init'):
     import torch
 
     from torchopt_amd import _lib
-    from torchopt_amd.placement import state_empty_like
+    from torchopt_amd.placement import state_zeros_like_tree
 
-    def moment(host_array, like):
-        """A moment array on the GPU: allocated the way the package's own init allocates state
-        (large arrays 8 KiB off the 16 KiB address phase the allocator gives the gradient), or
-        with --state plain wherever torch's allocator puts it, like the gradient."""
+    def moments(host_mu, host_nu, like):
+        """The two moment arrays on the GPU: allocated the way the package's own init allocates
+        the state of a one-leaf tree (--state init: one block, both moments 8 KiB off the 16 KiB
+        address phase the allocator gives the gradient, a whole even number of MiB apart modulo
+        16 MiB), each in a block of its own at that phase (--state separate), or wherever
+        torch's allocator puts them (--state plain)."""
         if state == 'plain':
-            return host_array.cuda()
-        return state_empty_like(like).copy_(host_array)
+            return host_mu.cuda(), host_nu.cuda()
+        if state == 'separate':
+            from torchopt_amd.placement import state_empty_like
+            return state_empty_like(like).copy_(host_mu), state_empty_like(like).copy_(host_nu)
+        (mu,), (nu,) = state_zeros_like_tree([like])
+        return mu.copy_(host_mu), nu.copy_(host_nu)
 
     if not torch.cuda.is_available():
         raise SystemExit('bench.py needs a GPU: the fused Adam op has no CPU path')
@@ -428,9 +434,12 @@ def run_gpu(cfg_id, steps, warmup, operator_preheat=None, state='library'):
             if state == 'plain':
                 ms = [h[1].cuda() for h in host]
                 vs = [h[2].cuda() for h in host]
-            else:  # as the package's init allocates the moments of a tree
-                from torchopt_amd.placement import state_zeros_like_tree
+            elif state == 'separate':
+                from torchopt_amd.placement import state_empty_like
 
+                ms = [state_empty_like(u).copy_(h[1]) for h, u in zip(host, us)]
+                vs = [state_empty_like(u).copy_(h[2]) for h, u in zip(host, us)]
+            else:  # as the package's init allocates the moments of a tree
                 ms, vs = state_zeros_like_tree(us)
                 for h, m, v in zip(host, ms, vs):
                     m.copy_(h[1])
@@ -477,7 +486,7 @@ def run_gpu(cfg_id, steps, warmup, operator_preheat=None, state='library'):
         total = cfg['n']
         h_u, h_mu, h_nu = host_state(cfg_id, 0, total, cfg['dtype'])
         u = h_u.cuda()
-        mu, nu = moment(h_mu, u), moment(h_nu, u)
+        mu, nu = moments(h_mu, h_nu, u)
         pu, pm, pv = u.data_ptr(), mu.data_ptr(), nu.data_ptr()
 
         extra = {'state_allocation': state,
@@ -1237,10 +1246,12 @@ def main(argv=None):
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--config', type=int, default=2, choices=sorted(CONFIGS))
     ap.add_argument('--no-cpu-baseline', action='store_true')
-    ap.add_argument('--state', choices=('library', 'plain'), default='library',
-                    help="how mu and nu are allocated: 'library' = as the package's init does "
-                         '(torchopt_amd.state_zeros_like: large arrays 8 KiB off the 16 KiB '
-                         "address phase of allocator blocks), 'plain' = torch's allocator alone")
+    ap.add_argument('--state', choices=('init', 'separate', 'plain'), default='init',
+                    help="how mu and nu are allocated: 'init' = as the package's init does "
+                         '(torchopt_amd.state_zeros_like_tree: the moments of a tree in one block, '
+                         'large leaves 8 KiB off the 16 KiB address phase of allocator blocks), '
+                         "'separate' = every moment in a block of its own at that phase "
+                         "(state_zeros_like), 'plain' = torch's allocator alone")
     ap.add_argument('--operator-preheat', type=int, default=None,
                     help='launches of the operator on scratch state before the warm-up steps '
                          '(default: 100 for the 16-bit configurations, 60 for the other '
