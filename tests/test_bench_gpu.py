@@ -28,6 +28,19 @@ def test_bench_config_runs(cfg, capsys):
     torch.cuda.empty_cache()
 
 
+@pytest.mark.parametrize('state', ['init', 'separate', 'plain'])
+def test_bench_state_allocation_modes(state, capsys):
+    """The three ways the benchmark can allocate the moments (as the package's init does, each in a
+    block of its own at the preferred phase, or wherever the allocator puts them)."""
+    assert bench.main(['--config', '0', '--steps', '2', '--warmup', '1', '--no-cpu-baseline',
+                       '--state', state]) == 0
+    line = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    assert line['config']['state_allocation'] == state
+    phases = line['config']['address_mod_16KiB']
+    assert phases['mu'] == phases['nu'] == (0 if state == 'plain' else 8192)
+    torch.cuda.empty_cache()
+
+
 def test_bench_refuses_more_than_one_gpu(capsys):
     assert bench.main(['--gpus', '2']) == 2
     assert 'one GPU' in capsys.readouterr().err
