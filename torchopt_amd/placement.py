@@ -112,7 +112,14 @@ def state_zeros_like_tree(leaves, *, requires_grad: bool = False):
             offsets.append(end)
             end += n
         second = _second_moment_offset(end, max(sizes), period)
-        block = torch.zeros((second + end + period) // es, dtype=dtype, device=device)
+        try:
+            block = torch.zeros((second + end + period) // es, dtype=dtype, device=device)
+        except torch.cuda.OutOfMemoryError:
+            # no room for one block of that size: a block per moment and leaf, as zeros_like would
+            for k in members:
+                mu[k] = state_zeros_like(leaves[k], requires_grad=requires_grad)
+                nu[k] = state_zeros_like(leaves[k], requires_grad=requires_grad)
+            continue
         first = lib.toa_adam_state_shift(block.data_ptr())
         for k, off in zip(members, offsets):
             n, shape = leaves[k].numel(), leaves[k].shape
