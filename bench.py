@@ -935,6 +935,66 @@ def run_state_phases(reps=12, n=1 << 28, step_kib=2, span_kib=32):
             'unshifted_after_each_row': unshifted, 'GB/s_by_phase': grid}
 
 
+def run_state_distances(reps=12, n=1 << 28, distances_mib=None):
+    """The operator (float32 forward_ in place, 2^28 elements, library defaults) with the gradient
+    in a PyTorch allocation of its own and BOTH moments in one block, each 8 KiB off the 16 KiB
+    address phase, the second `n * 4 bytes + d` after the first for a ladder of distances d.  This
+    is the measurement behind the distance at which the package's init places the two moments of
+    a leaf (torchopt_amd/placement.py).  Beside it: each moment in a block of its own at the
+    phase, and at the allocator's placement."""
+    import torch
+
+    from torchopt_amd import _lib
+
+    lib = _lib.load()
+    stream = torch.cuda.current_stream()
+    if distances_mib is None:
+        distances_mib = (0, 0.25, 0.5, 1, 1.5, 2, 2.5, 3, 4, 5, 6, 7, 8, 10, 12, 14, 16, 20, 24, 32)
+    mib = 1 << 18  # float32 elements
+    phase = (8 << 10) // 4
+    u = torch.empty(n, device='cuda')
+    block = torch.empty(2 * n + int(max(distances_mib) * mib) + 2 * phase, device='cuda')
+    own_mu = torch.empty(n + 2 * phase, device='cuda')
+    own_nu = torch.empty(n + 2 * phase, device='cuda')
+    preheat(torch)
+
+    def timed(mu, nu, launches=reps):
+        u.normal_()
+        mu.normal_(0, 0.1)
+        nu.normal_(0, 0.01).abs_()
+        ptrs = (u.data_ptr(), mu.data_ptr(), nu.data_ptr())
+
+        def launch():
+            rc = lib.toa_adam_forward_inplace(_lib.TOA_F32, *ptrs, n, B1, B2, EPS, 0.0, 1000,
+                                              stream.cuda_stream)
+            if rc:
+                raise RuntimeError(lib.toa_adam_error_string(rc).decode())
+        for _ in range(3):
+            launch()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record(stream)
+        for _ in range(launches):
+            launch()
+        ev1.record(stream)
+        torch.cuda.synchronize()
+        return round(24 * n / (ev0.elapsed_time(ev1) / launches) / 1e6)
+
+    def in_block(d):
+        at = n + int(d * mib) + phase
+        return block[phase:phase + n], block[at:at + n]
+
+    timed(*in_block(8), launches=60)  # past the operator's start-up transient
+    rounds = [{f'{d} MiB': timed(*in_block(d)) for d in distances_mib} for _ in range(2)]
+    return {'metric': 'forward_inplace_f32_by_moment_distance', 'unit': 'GB/s',
+            'peak': HBM_PEAK_GBS, 'elements': n, 'launches_timed': reps,
+            'device': torch.cuda.get_device_name(0),
+            'gradient_minus_block_mib': (u.data_ptr() - block.data_ptr()) / 2 ** 20,
+            'GB/s_by_distance_beyond_the_array_size': rounds,
+            'blocks_of_their_own_at_the_phase': timed(own_mu[phase:phase + n],
+                                                      own_nu[phase:phase + n]),
+            'allocator_placement': timed(own_mu[:n], own_nu[:n])}
+
+
 # ----------------------------------------------------------------------------- CPU baseline
 
 
@@ -1271,6 +1331,10 @@ def main(argv=None):
                     help='time the operator on three separate allocations with mu and nu shifted '
                          'inside theirs by every pair of phases below 32 KiB (steps of 2 KiB): '
                          'the measurement behind the phase at which the package allocates state')
+    ap.add_argument('--state-distances', action='store_true',
+                    help='time the operator with both moments in one block over a ladder of '
+                         'distances between them: the measurement behind the distance at which '
+                         "the package's init places the two moments of a leaf")
     args = ap.parse_args(argv)
 
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
@@ -1287,6 +1351,9 @@ def main(argv=None):
         return 0
     if args.state_phases:
         print(json.dumps(run_state_phases()), flush=True)
+        return 0
+    if args.state_distances:
+        print(json.dumps(run_state_distances()), flush=True)
         return 0
 
     host_cores()  # before torch (and with it the OpenMP runtime) loads

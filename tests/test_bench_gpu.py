@@ -75,3 +75,13 @@ def test_state_phase_sweep_runs():
     assert out['at_library_phase'] == out['GB/s_by_phase']['mu +8 KiB']['nu +8 KiB'] > 0
     assert len(out['unshifted_after_each_row']) == 2
     torch.cuda.empty_cache()
+
+
+def test_state_distance_sweep_runs():
+    """The operator with both moments in one block over a ladder of distances
+    (`bench.py --state-distances`), on small arrays and a short ladder."""
+    out = bench.run_state_distances(reps=2, n=1 << 22, distances_mib=(0, 1, 8))
+    assert out['unit'] == 'GB/s' and len(out['GB/s_by_distance_beyond_the_array_size']) == 2
+    assert set(out['GB/s_by_distance_beyond_the_array_size'][0]) == {'0 MiB', '1 MiB', '8 MiB'}
+    assert out['blocks_of_their_own_at_the_phase'] > 0 and out['allocator_placement'] > 0
+    torch.cuda.empty_cache()
