@@ -749,6 +749,16 @@ def run_ceiling(array_bytes=1 << 30, reps=20):
         layouts.append((f'one allocation, mu at 1 GiB + {a_kib} KiB, nu at 2 GiB + {b_kib} KiB',
                         (base, base + array_bytes + (a_kib << 10),
                          base + 2 * array_bytes + (b_kib << 10)), 0))
+    # ... and the placement the package's own init produces for a one-leaf tree: the gradient in
+    # an allocation of its own, both moments in one block, 8 KiB off the 16 KiB phase, an even
+    # number of MiB (8 where cheap) past a multiple of 16 MiB apart
+    from torchopt_amd.placement import state_zeros_like_tree
+    own_grad = torch.randn(n_elems, device='cuda')
+    (own_mu,), (own_nu,) = state_zeros_like_tree([own_grad])
+    own_mu.normal_()
+    own_nu.normal_()
+    init_layout = "a gradient allocation and the moments in one block where the package's init puts them"
+    layouts.append((init_layout, (own_grad.data_ptr(), own_mu.data_ptr(), own_nu.data_ptr()), 0))
     family = {}
     for layout, ptrs3, piece in layouts:
         rows, top = {}, (0.0, None)
@@ -781,6 +791,8 @@ def run_ceiling(array_bytes=1 << 30, reps=20):
         views = [torch.empty(0)] * 3
         if layout == 'three separate arrays':
             views = arrays[:3]
+        elif layout == init_layout:
+            views = [own_grad, own_mu, own_nu]
         else:
             views = [wide[(p - wide.data_ptr()) // 4:(p - wide.data_ptr()) // 4 + n_elems]
                      for p in ptrs3]
