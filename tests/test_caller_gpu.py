@@ -431,3 +431,39 @@ def test_state_of_large_leaves_is_placed_and_steps_like_any_other(dtype):
     opt.step()
     s = opt.state_groups[0]
     assert s.mu[0].data_ptr() % (16 << 10) == 8 << 10 and s.nu[0].data_ptr() % (16 << 10) == 8 << 10
+
+
+@pytest.mark.parametrize('seed', [0, 1, 2])
+def test_tree_state_allocation_invariants_on_random_trees(seed):
+    """Random trees (sizes from empty to 24 MiB, three dtypes, missing leaves): whatever the mix,
+    every moment has its leaf's shape and dtype, holds zeros, shares no byte with another, and
+    the large leaves of one dtype sit at the preferred phase in one block."""
+    from torchopt_amd import state_zeros_like_tree
+
+    rng = np.random.default_rng(seed)
+    dtypes = (torch.float32, torch.float64, torch.bfloat16)
+    tree = []
+    for _ in range(int(rng.integers(1, 40))):
+        kind = rng.integers(0, 10)
+        if kind == 0:
+            tree.append(None)
+            continue
+        n = int(rng.choice([0, 1, 7, 4096, 1 << 18, (1 << 20) + 3, 3 << 20, 6 << 20]))
+        tree.append(torch.empty(n, device='cuda', dtype=dtypes[int(rng.integers(0, 3))]))
+    mu, nu = state_zeros_like_tree(tree)
+    spans, blocks = [], {}
+    for t, a, b in zip(tree, mu, nu):
+        if t is None:
+            assert a is None and b is None
+            continue
+        for x in (a, b):
+            assert x.shape == t.shape and x.dtype == t.dtype and x.device == t.device
+            assert x.is_contiguous() and not x.any()
+            if x.numel():
+                spans.append((x.data_ptr(), x.data_ptr() + x.numel() * x.element_size()))
+            if t.numel() * t.element_size() >= (1 << 20):
+                assert x.data_ptr() % (16 << 10) == 8 << 10
+                blocks.setdefault(t.dtype, set()).add(x.untyped_storage().data_ptr())
+    spans.sort()
+    assert all(p[1] <= q[0] for p, q in zip(spans, spans[1:])), 'two moments overlap'
+    assert all(len(b) == 1 for b in blocks.values()), 'one block per dtype'
