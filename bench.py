@@ -57,7 +57,7 @@ BYTES_PER_ELEM = {  # op -> number of arrays streamed (multiply by the element s
 # figures belong to the kernels as they were when the profile was taken; re-record them whenever
 # adam_kernels.hpp or the launch shape changes.
 RECORDED_TRAFFIC = {
-    2: (6442426275, 'profiles/forward_inplace_f32_config2_pmc_traffic.md'),
+    2: (6442421106, 'profiles/forward_inplace_f32_config2_pmc_traffic.md'),
     4: (8516207551, 'profiles/forward_inplace_multi_f32_config4_kernel_trace_and_traffic.md'),
     5: (9935417258, 'profiles/fused_step_multi_f32_config5_kernel_trace_and_traffic.md'),
 }
@@ -268,15 +268,16 @@ def run_gpu(cfg_id, steps, warmup, operator_preheat=None, state='init'):
 
     def moments(host_mu, host_nu, like):
         """The two moment arrays on the GPU: allocated the way the package's own init allocates
-        the state of a one-leaf tree (--state init: one block, both moments 8 KiB off the 16 KiB
-        address phase the allocator gives the gradient, a whole even number of MiB apart modulo
-        16 MiB), each in a block of its own at that phase (--state separate), or wherever
+        the state of a one-leaf tree (--state init: one block, the first moment 8 KiB past a
+        multiple of 16 KiB, the second at one, a whole even number of MiB plus those 8 KiB apart
+        modulo 16 MiB), each in a block of its own at its phase (--state separate), or wherever
         torch's allocator puts them (--state plain)."""
         if state == 'plain':
             return host_mu.cuda(), host_nu.cuda()
         if state == 'separate':
             from torchopt_amd.placement import state_empty_like
-            return state_empty_like(like).copy_(host_mu), state_empty_like(like).copy_(host_nu)
+            return (state_empty_like(like, moment=0).copy_(host_mu),
+                    state_empty_like(like, moment=1).copy_(host_nu))
         (mu,), (nu,) = state_zeros_like_tree([like])
         return mu.copy_(host_mu), nu.copy_(host_nu)
 
@@ -437,8 +438,8 @@ def run_gpu(cfg_id, steps, warmup, operator_preheat=None, state='init'):
             elif state == 'separate':
                 from torchopt_amd.placement import state_empty_like
 
-                ms = [state_empty_like(u).copy_(h[1]) for h, u in zip(host, us)]
-                vs = [state_empty_like(u).copy_(h[2]) for h, u in zip(host, us)]
+                ms = [state_empty_like(u, moment=0).copy_(h[1]) for h, u in zip(host, us)]
+                vs = [state_empty_like(u, moment=1).copy_(h[2]) for h, u in zip(host, us)]
             else:  # as the package's init allocates the moments of a tree
                 ms, vs = state_zeros_like_tree(us)
                 for h, m, v in zip(host, ms, vs):
@@ -936,14 +937,14 @@ def run_state_phases(reps=12, n=1 << 28, step_kib=2, span_kib=32):
     for a in phases:
         grid[f'mu +{a} KiB'] = {f'nu +{b} KiB': round(timed(a, b)) for b in phases}
         unshifted.append(round(timed(0, 0)))
-    shift = lib.toa_adam_state_shift(0) // 1024
+    shift_mu, shift_nu = (lib.toa_adam_state_shift(0, k) // 1024 for k in (0, 1))
     return {'metric': 'forward_inplace_f32_by_state_phase', 'unit': 'GB/s', 'peak': HBM_PEAK_GBS,
             'elements': n, 'launches_timed': reps, 'device': torch.cuda.get_device_name(0),
             'address_mod_16KiB': {'updates': u.data_ptr() % 16384,
                                   'mu_block': mu_block.data_ptr() % 16384,
                                   'nu_block': nu_block.data_ptr() % 16384},
-            'library_phase_kib': shift,
-            'at_library_phase': grid[f'mu +{shift} KiB'][f'nu +{shift} KiB'],
+            'library_phases_kib': {'mu': shift_mu, 'nu': shift_nu},
+            'at_library_phases': grid[f'mu +{shift_mu} KiB'][f'nu +{shift_nu} KiB'],
             'unshifted_after_each_row': unshifted, 'GB/s_by_phase': grid}
 
 
@@ -964,13 +965,14 @@ def run_state_distances(reps=12, n=1 << 28, distances_mib=None):
         distances_mib = (0, 0.25, 0.5, 1, 1.5, 2, 2.5, 3, 4, 5, 6, 7, 8, 10, 12, 14, 16, 20, 24, 32)
     mib = 1 << 18  # float32 elements
     phase = (8 << 10) // 4
-    u = torch.empty(n, device='cuda')
-    block = torch.empty(2 * n + int(max(distances_mib) * mib) + 2 * phase, device='cuda')
+    u_block = torch.empty(n + 4 * phase, device='cuda')
+    u = u_block[:n]
+    block = torch.empty(2 * n + int(max(distances_mib) * mib) + 4 * phase, device='cuda')
     own_mu = torch.empty(n + 2 * phase, device='cuda')
     own_nu = torch.empty(n + 2 * phase, device='cuda')
     preheat(torch)
 
-    def timed(mu, nu, launches=reps):
+    def timed(mu, nu, launches=reps, u=u):
         u.normal_()
         mu.normal_(0, 0.1)
         nu.normal_(0, 0.01).abs_()
@@ -997,13 +999,26 @@ def run_state_distances(reps=12, n=1 << 28, distances_mib=None):
 
     timed(*in_block(8), launches=60)  # past the operator's start-up transient
     rounds = [{f'{d} MiB': timed(*in_block(d)) for d in distances_mib} for _ in range(2)]
+    # The two moments at one phase against 8 KiB apart (what the package's init does), 8 MiB
+    # beyond the array size apart, with the gradient's own phase shifted: an allocator puts large
+    # blocks on 2 MiB boundaries, but where the physical pages lie is not the caller's to see.
+    by_gradient_phase = {}
+    for name, (a_kib, b_kib) in (('both moments 8 KiB off', (8, 8)),
+                                 ('first moment 8 KiB off, second at 0', (8, 0)),
+                                 ('first moment at 0, second 8 KiB off', (0, 8)),
+                                 ('both moments at 0', (0, 0))):
+        mu = block[a_kib * 256:a_kib * 256 + n]
+        at = n + 8 * mib + b_kib * 256
+        nu = block[at:at + n]
+        by_gradient_phase[name] = {f'gradient +{g} KiB': timed(mu, nu, u=u_block[g * 256:g * 256 + n])
+                                   for g in (0, 4, 8, 12)}
     return {'metric': 'forward_inplace_f32_by_moment_distance', 'unit': 'GB/s',
             'peak': HBM_PEAK_GBS, 'elements': n, 'launches_timed': reps,
             'device': torch.cuda.get_device_name(0),
             'gradient_minus_block_mib': (u.data_ptr() - block.data_ptr()) / 2 ** 20,
             'GB/s_by_distance_beyond_the_array_size': rounds,
-            'blocks_of_their_own_at_the_phase': timed(own_mu[phase:phase + n],
-                                                      own_nu[phase:phase + n]),
+            'GB/s_by_phases_of_the_moments_and_of_the_gradient': by_gradient_phase,
+            'blocks_of_their_own_at_their_phases': timed(own_mu[phase:phase + n], own_nu[:n]),
             'allocator_placement': timed(own_mu[:n], own_nu[:n])}
 
 
@@ -1321,8 +1336,8 @@ def main(argv=None):
     ap.add_argument('--state', choices=('init', 'separate', 'plain'), default='init',
                     help="how mu and nu are allocated: 'init' = as the package's init does "
                          '(torchopt_amd.state_zeros_like_tree: the moments of a tree in one block, '
-                         'large leaves 8 KiB off the 16 KiB address phase of allocator blocks), '
-                         "'separate' = every moment in a block of its own at that phase "
+                         'the two moments of a large leaf 8 KiB apart modulo 16 KiB), '
+                         "'separate' = every moment in a block of its own at its phase "
                          "(state_zeros_like), 'plain' = torch's allocator alone")
     ap.add_argument('--operator-preheat', type=int, default=None,
                     help='launches of the operator on scratch state before the warm-up steps '

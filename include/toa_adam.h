@@ -111,19 +111,21 @@ TOA_API int toa_adam_release_plans(void);
 TOA_API unsigned toa_adam_set_max_grid(unsigned workgroups);
 
 /* Where to put optimizer state.  The in-place step streams three arrays at once, and how their
- * addresses fall on the memory channels moves its rate by up to 3 %: an allocator hands out large
- * blocks on 2 MiB boundaries, so the gradient, mu and nu of a large tensor normally share their
- * address modulo 16 KiB; with mu and nu 8 KiB off that phase the float32 step on 2^28 elements
- * streams 0.8-1.0 % faster (6.85 against 6.79 TB/s), distances of 4 or 12 KiB are the slow ones,
- * and no op or element type measured slower at 8 KiB than at 0.  The caller owns every
- * allocation, so this is advice in callable form:
+ * addresses fall on the memory channels moves its rate by up to 3 %.  Measured on the float32
+ * step over 2^28 elements: with the two moments of a tensor 8 KiB apart modulo 16 KiB the step
+ * streams at 6.80-6.87 TB/s whatever the gradient's own phase; with both at one phase it ranges
+ * from 6.72 to 6.86 with the gradient's phase (an allocator hands out large blocks on 2 MiB
+ * boundaries, so left alone all three arrays share their address modulo 16 KiB: 6.74-6.79).  The
+ * caller owns every allocation, so this is advice in callable form:
  *   toa_adam_state_slack   extra bytes to allocate for a state array (16 KiB);
  *   toa_adam_state_shift   bytes (a multiple of 256, less than the slack) to skip from the start
- *                          of such an allocation so that the array begins at the preferred phase.
+ *                          of such an allocation so that the array begins at the preferred phase
+ *                          of its kind: moment 0 (mu) 8 KiB past a multiple of 16 KiB, moment 1
+ *                          (nu) at a multiple of 16 KiB.
  * No counterpart in the reference (its init_fn calls zeros_like,
  * /root/reference/torchopt/transform/scale_by_adam.py:401-414). */
 TOA_API size_t toa_adam_state_slack(void);
-TOA_API size_t toa_adam_state_shift(const void *allocation);
+TOA_API size_t toa_adam_state_shift(const void *allocation, int moment);
 
 /* Human-readable name of a return code from any function below. */
 TOA_API const char *toa_adam_error_string(int code);

@@ -37,7 +37,7 @@ def test_bench_state_allocation_modes(state, capsys):
     line = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
     assert line['config']['state_allocation'] == state
     phases = line['config']['address_mod_16KiB']
-    assert phases['mu'] == phases['nu'] == (0 if state == 'plain' else 8192)
+    assert (phases['mu'], phases['nu']) == ((0, 0) if state == 'plain' else (8192, 0))
     torch.cuda.empty_cache()
 
 
@@ -70,9 +70,9 @@ def test_state_phase_sweep_runs():
     """The operator on separate allocations with the moments at a grid of phases
     (`bench.py --state-phases`), on small arrays and a coarse grid."""
     out = bench.run_state_phases(reps=2, n=1 << 22, step_kib=8, span_kib=16)
-    assert out['unit'] == 'GB/s' and out['library_phase_kib'] == 8
+    assert out['unit'] == 'GB/s' and out['library_phases_kib'] == {'mu': 8, 'nu': 0}
     assert set(out['GB/s_by_phase']) == {'mu +0 KiB', 'mu +8 KiB'}
-    assert out['at_library_phase'] == out['GB/s_by_phase']['mu +8 KiB']['nu +8 KiB'] > 0
+    assert out['at_library_phases'] == out['GB/s_by_phase']['mu +8 KiB']['nu +0 KiB'] > 0
     assert len(out['unshifted_after_each_row']) == 2
     torch.cuda.empty_cache()
 
@@ -83,5 +83,6 @@ def test_state_distance_sweep_runs():
     out = bench.run_state_distances(reps=2, n=1 << 22, distances_mib=(0, 1, 8))
     assert out['unit'] == 'GB/s' and len(out['GB/s_by_distance_beyond_the_array_size']) == 2
     assert set(out['GB/s_by_distance_beyond_the_array_size'][0]) == {'0 MiB', '1 MiB', '8 MiB'}
-    assert out['blocks_of_their_own_at_the_phase'] > 0 and out['allocator_placement'] > 0
+    assert out['blocks_of_their_own_at_their_phases'] > 0 and out['allocator_placement'] > 0
+    assert len(out['GB/s_by_phases_of_the_moments_and_of_the_gradient']) == 4
     torch.cuda.empty_cache()

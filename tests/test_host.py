@@ -258,14 +258,16 @@ def test_availability_probe_is_loud_about_the_cpu():
 
 
 def test_state_placement_advice():
-    """toa_adam_state_shift: the bytes to skip so a state array starts 8 KiB off a 16 KiB phase."""
+    """toa_adam_state_shift: the bytes to skip so a first moment starts 8 KiB past a multiple of
+    16 KiB and a second moment at one: the two 8 KiB apart modulo 16 KiB."""
     lib = _lib.load()
     slack = lib.toa_adam_state_slack()
     assert slack == 16 << 10
     for base in (0, 256, 8 << 10, (8 << 10) + 512, (16 << 10) - 256, (2 << 20) * 37, 0x7f12_3456_7800):
-        shift = lib.toa_adam_state_shift(base)
-        assert 0 <= shift < slack and shift % 256 == base % 256 == 0
-        assert (base + shift) % slack == 8 << 10
+        for moment, phase in ((0, 8 << 10), (1, 0)):
+            shift = lib.toa_adam_state_shift(base, moment)
+            assert 0 <= shift < slack and shift % 256 == base % 256 == 0
+            assert (base + shift) % slack == phase
     # CPU tensors, small tensors and non-contiguous ones are plain zeros_like / empty_like
     import torch
 

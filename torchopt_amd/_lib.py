@@ -37,7 +37,7 @@ SIGNATURES = {
     'toa_adam_set_plan_mode': [_i],
     'toa_adam_release_plans': [],
     'toa_adam_state_slack': [],
-    'toa_adam_state_shift': [_vp],
+    'toa_adam_state_shift': [_vp, _i],
     'toa_adam_forward_inplace': [_i, _vp, _vp, _vp, _sz, _d, _d, _d, _d, _u64, _vp],
     'toa_adam_forward_mu': [_i, _vp, _vp, _sz, _d, _vp, _vp],
     'toa_adam_forward_nu': [_i, _vp, _vp, _sz, _d, _vp, _vp],

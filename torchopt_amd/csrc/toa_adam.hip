@@ -147,7 +147,8 @@ bool arrays_disjoint(T *const (&ptrs)[NPTR], size_t n) {
     return true;
 }
 
-// Where state arrays should begin, as an address modulo kStatePeriod (see toa_adam_state_shift).
+// Where first moments should begin, as an address modulo kStatePeriod; second moments begin at
+// a multiple of it (see toa_adam_state_shift).
 constexpr uintptr_t kStatePeriod = 16 << 10, kStatePhase = 8 << 10;
 
 // Workgroups per launch are capped; a tensor with more tiles than the cap is covered by the
@@ -807,12 +808,13 @@ extern "C" {
 
 int toa_adam_abi_version(void) { return 4; }
 
-// Preferred placement of state arrays: 8 KiB off the 16 KiB phase that large allocations share.
+// Preferred placement of state arrays: the two moments of a tensor 8 KiB apart modulo 16 KiB.
 size_t toa_adam_state_slack(void) { return kStatePeriod; }
 
-size_t toa_adam_state_shift(const void *allocation) {
+size_t toa_adam_state_shift(const void *allocation, int moment) {
+    const uintptr_t want = moment == 0 ? kStatePhase : 0;
     const uintptr_t at = reinterpret_cast<uintptr_t>(allocation) % kStatePeriod;
-    return (size_t)((kStatePhase + kStatePeriod - at) % kStatePeriod);
+    return (size_t)((want + kStatePeriod - at) % kStatePeriod);
 }
 
 int toa_adam_set_waves_per_cu(int waves) {

@@ -4,17 +4,20 @@ The reference's ``init_fn`` makes its moments with ``zeros_like``
 (/root/reference/torchopt/transform/scale_by_adam.py:401-414) and gets whatever address the
 allocator hands out: for a large tensor a block on a 2 MiB boundary, so gradient, mu and nu share
 their address modulo 16 KiB.  The in-place step streams all three at once, and on MI355X its rate
-moves with how those streams fall on the memory channels: with the two moments 8 KiB off the
-gradient's phase the float32 step on 2^28 elements runs 0.8-1.0 % faster, 4 and 12 KiB are the
-slow distances, and nothing measured is slower at 8 KiB than at 0.  The state this package
-allocates therefore starts at that phase (``toa_adam_state_shift`` of the C ABI names it);
-values, shapes, dtypes and contiguity are those of ``zeros_like``.
+moves with how those streams fall on the memory channels.  Measured on the float32 step over 2^28
+elements: with the two moments 8 KiB apart modulo 16 KiB it runs at 85.0-85.8 % of the HBM peak
+whatever the gradient's own phase (84.2-84.9 % with all three at one phase, as the allocator
+leaves them; 84.0-85.7 % with both moments at one phase 8 KiB off, depending on the gradient's).
+The state this package allocates therefore starts 8 KiB past a multiple of 16 KiB for first
+moments and at a multiple of 16 KiB for second moments (``toa_adam_state_shift`` of the C ABI
+names the phases); values, shapes, dtypes and contiguity are those of ``zeros_like``.
 
 A tree's moments come from ONE block per (device, dtype): every mu, then every nu, each leaf at
-the phase, so the slack is 16 KiB per leaf instead of what the allocator's rounding would add to
+its phase, so the slack is 16 KiB per leaf instead of what the allocator's rounding would add to
 separate blocks (2 MiB on a 16 MiB leaf), and a leaf's two moments lie a whole even number of MiB
-between 4 and 12 apart modulo 16 MiB (8 where that costs little): the distances the step streams
-fastest at, and clear of the multiples of 16 MiB at which arrays meet in the same DRAM banks.
+between 4 and 12, plus those 8 KiB, apart modulo 16 MiB (8 MiB where that costs little): the
+distances the step streams fastest at, and clear of the multiples of 16 MiB at which arrays meet
+in the same DRAM banks.
 """
 
 from __future__ import annotations
@@ -28,7 +31,7 @@ from torchopt_amd import _lib
 MIN_BYTES = 1 << 20
 
 
-def _placed(t: torch.Tensor, zero: bool, requires_grad: bool) -> torch.Tensor:
+def _placed(t: torch.Tensor, zero: bool, requires_grad: bool, moment: int) -> torch.Tensor:
     size = t.numel() * t.element_size()
     if (not t.is_cuda or size < MIN_BYTES or not t.is_contiguous()
             or t.layout != torch.strided):
@@ -38,20 +41,23 @@ def _placed(t: torch.Tensor, zero: bool, requires_grad: bool) -> torch.Tensor:
     slack = lib.toa_adam_state_slack() // t.element_size()
     make = torch.zeros if zero else torch.empty
     block = make(t.numel() + slack, dtype=t.dtype, device=t.device)
-    skip = lib.toa_adam_state_shift(block.data_ptr()) // t.element_size()
+    skip = lib.toa_adam_state_shift(block.data_ptr(), moment) // t.element_size()
     out = block[skip:skip + t.numel()].view(t.shape)
     return out.requires_grad_(requires_grad)
 
 
-def state_zeros_like(t: torch.Tensor, *, requires_grad: bool = False) -> torch.Tensor:
-    """``zeros_like(t)`` at the preferred phase (a view into a slightly larger block when `t` is
-    a contiguous GPU tensor of 1 MiB or more, plain ``zeros_like`` otherwise)."""
-    return _placed(t, True, requires_grad)
+def state_zeros_like(t: torch.Tensor, *, requires_grad: bool = False,
+                     moment: int = 0) -> torch.Tensor:
+    """``zeros_like(t)`` at the preferred phase of a first (``moment=0``) or second
+    (``moment=1``) moment: a view into a slightly larger block when `t` is a contiguous GPU tensor
+    of 1 MiB or more, plain ``zeros_like`` otherwise."""
+    return _placed(t, True, requires_grad, moment)
 
 
-def state_empty_like(t: torch.Tensor, *, requires_grad: bool = False) -> torch.Tensor:
-    """``empty_like(t)`` at the preferred phase."""
-    return _placed(t, False, requires_grad)
+def state_empty_like(t: torch.Tensor, *, requires_grad: bool = False,
+                     moment: int = 0) -> torch.Tensor:
+    """``empty_like(t)`` at the preferred phase of a first or second moment."""
+    return _placed(t, False, requires_grad, moment)
 
 
 # How far apart the two moments of a leaf lie inside the block, modulo 16 MiB.  Measured on the
@@ -66,14 +72,15 @@ _DISTANCES = (8 << 20, 10 << 20, 6 << 20, 12 << 20, 4 << 20)  # in order of pref
 def _second_moment_offset(end: int, largest: int, period: int) -> int:
     """Where the second moments start, `end` being the size of the first moments' region: the
     nearest preferred distance that costs at most 1/32 of the region (2 MiB for small ones) in
-    slack, else the cheapest preferred one.  Small leaves sit in cache; nothing to arrange."""
+    slack, else the cheapest preferred one (small leaves sit in cache: no distance to arrange) --
+    plus the 8 KiB that put the second moments at their own phase."""
     second = -(-end // period) * period
-    if largest < (4 << 20):
-        return second
-    budget = max(2 << 20, end // 32)
-    gaps = [(want - second) % _DISTANCE_PERIOD for want in _DISTANCES]
-    within = [g for g in gaps if g <= budget]
-    return second + (within[0] if within else min(gaps))
+    if largest >= (4 << 20):
+        budget = max(2 << 20, end // 32)
+        gaps = [(want - second) % _DISTANCE_PERIOD for want in _DISTANCES]
+        within = [g for g in gaps if g <= budget]
+        second += within[0] if within else min(gaps)
+    return second + period // 2  # second moments half a period off the first moments' phase
 
 
 def _eligible(t) -> bool:
@@ -117,10 +124,10 @@ def state_zeros_like_tree(leaves, *, requires_grad: bool = False):
         except torch.cuda.OutOfMemoryError:
             # no room for one block of that size: a block per moment and leaf, as zeros_like would
             for k in members:
-                mu[k] = state_zeros_like(leaves[k], requires_grad=requires_grad)
-                nu[k] = state_zeros_like(leaves[k], requires_grad=requires_grad)
+                mu[k] = state_zeros_like(leaves[k], requires_grad=requires_grad, moment=0)
+                nu[k] = state_zeros_like(leaves[k], requires_grad=requires_grad, moment=1)
             continue
-        first = lib.toa_adam_state_shift(block.data_ptr())
+        first = lib.toa_adam_state_shift(block.data_ptr(), 0)
         for k, off in zip(members, offsets):
             n, shape = leaves[k].numel(), leaves[k].shape
             a, b = (first + off) // es, (first + second + off) // es
