@@ -1,13 +1,19 @@
 #!/usr/bin/env python3
 """Benchmark of the fused Adam operator on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config {0,...,7}]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config {0,...,9}]
+                    [--state {init,separate,plain}] [--operator-preheat N]
 
 A "step" is one pass of the hot path over one batch of synthetic state that is already
 resident in HBM: for the default workload (config 2) one fused in-place `forward_` over three
 float32 arrays of 268 435 456 elements (1 GiB each), launched through the C ABI of
 libtoa_adam.so on PyTorch's current stream.  W untimed steps, then exactly K timed steps
-bracketed by `torch.cuda.synchronize()`; one JSON line on stdout.
+bracketed by `torch.cuda.synchronize()`; one JSON line on stdout.  The gradient array is a
+PyTorch allocation; the two moments are allocated as the package's own init allocates state
+(`--state init`: torchopt_amd.state_zeros_like_tree; `separate` and `plain` are there to show what
+that placement is worth).  Before the W warm-up steps the bandwidth-bound configurations run the
+operator 60-100 times on scratch state, past its start-up transient (`--operator-preheat 0`
+switches that off); the line records both.
 
 Beside the headline `value` (elements per second) the line carries
   roofline      achieved HBM bandwidth of the kernel: algorithmic bytes per launch (24 B per
@@ -20,7 +26,10 @@ Beside the headline `value` (elements per second) the line carries
 `--ceiling` measures, instead of the operator, what this machine's HBM delivers to streaming
 kernels of the same launch shape that do next to no arithmetic (bench_probe.hip: R arrays read,
 W arrays written, at every residency level), and prints those ceilings as one JSON line: the
-context for `roofline.frac`.
+context for `roofline.frac`.  `--placements`, `--state-phases` and `--state-distances` time the
+operator over placements of its three arrays (inside one allocation; the moments' address phases
+on separate allocations; the distance between the moments in one block): the measurements behind
+where the package allocates state.
 
 Everything on one GPU: `--gpus N` with N > 1 is refused.
 """
