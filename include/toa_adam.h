@@ -27,7 +27,10 @@
  *   return    0 on success; a positive value is a hipError_t from the launch;
  *             a negative value is one of the TOA_E* argument errors below.
  *             toa_adam_error_string() names either kind.
- *   threads   re-entrant; the only global state is the two tuning knobs below.
+ *   threads   re-entrant.  Global state: the tuning knobs below and the cache of list plans (see
+ *             toa_adam_set_plan_mode), which one mutex guards from the lookup until the launch
+ *             that reads the plan is enqueued -- list calls from several host threads therefore
+ *             take turns for the few microseconds that enqueueing costs.
  */
 #ifndef TOA_ADAM_H
 #define TOA_ADAM_H
@@ -79,7 +82,8 @@ TOA_API int toa_adam_set_waves_per_cu(int waves);
  *   1            never staged;
  *   2            staged wherever it is legal.
  * Staged needs the arrays of a tensor to be disjoint, 16-byte aligned and large enough to be
- * bandwidth-bound; other calls take the plain order whatever the setting (bfloat16 always does).
+ * bandwidth-bound; other calls take the plain order whatever the setting.  (All four element
+ * types have a staged form; lists of the 16-bit types run staged by default.)
  * Returns the previous setting.  No counterpart in the reference. */
 TOA_API int toa_adam_set_schedule(int schedule);
 
@@ -193,7 +197,7 @@ TOA_API int toa_adam_forward_inplace_multi(int dtype, size_t num_tensors, void *
  * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in
  * the reference.  Same arguments, same results bit for bit, always one launch per distinct step
  * count however long the list; the per-tensor records live in a device array built into the
- * library (384 KiB on every GPU the library runs on, held until the process ends) instead of
+ * library (448 KiB on every GPU the library runs on, held until the process ends) instead of
  * cached allocations, and are rewritten by every call.  It calls no hipMalloc, hipFree or other
  * allocating routine and records no memset or copy.
  *   limit    at most 4096 non-empty tensors per call (and device numbers below 64): beyond that

@@ -23,6 +23,7 @@ LIB_PATH = os.path.join(PKG_DIR, 'libtoa_adam.so')
 SOURCES = [os.path.join(PKG_DIR, 'csrc', 'toa_adam.hip')]
 HEADERS = [
     os.path.join(PKG_DIR, 'csrc', 'adam_kernels.hpp'),
+    os.path.join(PKG_DIR, 'csrc', 'plan_cache.hpp'),
     os.path.join(REPO_DIR, 'include', 'toa_adam.h'),
 ]
 

@@ -4,7 +4,12 @@
 // launchers do (/root/reference/src/adam_op/adam_op_impl_cpu.cpp:73-84,
 // 191-206, 328-343: powers, differences and reciprocals in double, then one
 // cast to the element type), picks a grid and enqueues one kernel on the
-// caller's stream.  Nothing here allocates, copies or synchronises.
+// caller's stream.  Nothing here copies or synchronises, and the single-tensor
+// entry points allocate nothing; the list entry points keep the record tables
+// of long lists ("plans") in device memory that the library allocates once per
+// (device, stream, list) and caches (plan_cache.hpp) -- except
+// toa_adam_forward_inplace_multi_noalloc, whose plan lives in a file-scope
+// device array.
 #include "toa_adam.h"
 
 #include <hip/hip_runtime.h>
@@ -18,9 +23,12 @@
 #include <vector>
 
 #include "adam_kernels.hpp"
+#include "plan_cache.hpp"
 
-// Bytes of the file-scope plan array behind toa_adam_forward_inplace_multi_noalloc: 4096 records.
-constexpr size_t toa_noalloc_scratch_bytes = 4096 * 96;
+// Bytes of the file-scope plan array behind toa_adam_forward_inplace_multi_noalloc: 4096 records
+// of 96 bytes and, behind them, the finer tile index of a long list (at most four 4-byte entries
+// per record).
+constexpr size_t toa_noalloc_scratch_bytes = 4096 * 96 + 4 * 4096 * 4;
 
 namespace {
 
@@ -237,9 +245,6 @@ int launch_single(const Op &op, T *const (&ptrs)[Op::NPTR], size_t n, void *stre
 std::atomic<int> g_plan_mode{0};
 constexpr uint64_t kPlanFromTiles = 1u << 18;  // 256 MiB of 1 KiB tiles per array
 
-constexpr size_t kPlanSlotsPerStream = 4;         // cached plans a stream may hold
-constexpr size_t kPlanSlotsTotal = 64;            // and the process as a whole
-
 // A plan of more than kPlanFineFrom records carries a finer index behind its records: one entry
 // per 2^shift tiles, the smallest shift that leaves at most four entries per record.
 constexpr size_t kPlanFineFrom = 2 * kPlanCells;
@@ -275,19 +280,31 @@ int plan_write(void *mem, const std::vector<PlanSeed<NPTR>> &seeds, hipStream_t 
     return 0;
 }
 
-// The launch's view of a plan: the coarse index from tile cells to records, and the finer one in
-// device memory where the plan has it (`with_fine`: plans from the cache; a caller's arena holds
-// records only).
+// The records and, for a plan of more than kPlanFineFrom records, the finer index behind them.
 template <int NPTR>
-PlanView plan_view(void *mem, const std::vector<PlanSeed<NPTR>> &seeds, uint32_t total,
-                   bool with_fine) {
+int plan_write_all(void *mem, const std::vector<PlanSeed<NPTR>> &seeds, uint32_t fine_entries,
+                   uint32_t fine_shift, hipStream_t stream) {
+    if (const int rc = plan_write<NPTR>(mem, seeds, stream)) return rc;
+    if (fine_entries == 0) return 0;
+    hipLaunchKernelGGL(plan_index_kernel, dim3((fine_entries + 255) / 256), dim3(256), 0, stream,
+                       static_cast<const PlanRec *>(mem), (uint32_t)seeds.size(),
+                       reinterpret_cast<uint32_t *>(static_cast<char *>(mem) +
+                                                    plan_record_bytes(seeds.size())),
+                       fine_entries, fine_shift);
+    return (int)hipGetLastError();
+}
+
+// The launch's view of a plan: the coarse index from tile cells to records, and the finer one in
+// device memory where the plan has it (lists of more than kPlanFineFrom records).
+template <int NPTR>
+PlanView plan_view(void *mem, const std::vector<PlanSeed<NPTR>> &seeds, uint32_t total) {
     PlanView v;
     v.recs = static_cast<const PlanRec *>(mem);
     v.total = total;
     v.num = (uint32_t)seeds.size();
     v.fine = nullptr;
     v.fine_shift = 0;
-    if (with_fine && plan_fine_entries(seeds.size(), total, &v.fine_shift) != 0)
+    if (plan_fine_entries(seeds.size(), total, &v.fine_shift) != 0)
         v.fine = reinterpret_cast<const uint32_t *>(static_cast<const char *>(mem) +
                                                    plan_record_bytes(seeds.size()));
     v.shift = 0;
@@ -301,135 +318,84 @@ PlanView plan_view(void *mem, const std::vector<PlanSeed<NPTR>> &seeds, uint32_t
     return v;
 }
 
-// Cached plans.  A plan's memory is written and read by work enqueued on ONE stream, so stream
-// order keeps a rewrite behind the launches that still read the old contents; another stream
-// gets another plan.  Keyed by the exact bytes of the records.
-struct PlanSlot {
-    int device = -1;
-    hipStream_t stream = nullptr;
-    void *mem = nullptr;
-    size_t capacity = 0;
-    std::vector<unsigned char> key;  // empty: contents unknown
-    uint64_t stamp = 0;
-    // The last call this plan served, remembered whole: the caller's arguments as bytes and the
-    // launch they led to.  A training loop calls with the same lists step after step; when the
-    // arguments are byte for byte those of the last time, every per-tensor decision is known
-    // already and the call is one comparison and one launch (150 ns per tensor otherwise).
-    std::vector<unsigned char> call;  // empty: nothing remembered
+// Cached plans (plan_cache.hpp holds the slot state machine and its threading contract): keyed by
+// (device, stream, exact bytes of the records).  A slot also remembers the last call it served,
+// whole -- the caller's arguments as bytes and the launch they led to.  A training loop calls with
+// the same lists step after step; when the arguments are byte for byte those of the last time,
+// every per-tensor decision is known already and the call is one comparison and one launch
+// (150 ns per tensor otherwise).
+struct PlanMemo {
     PlanView view;
     bool staged = false;
 };
-std::mutex g_plan_mutex;
-std::vector<PlanSlot> g_plan_slots;
-uint64_t g_plan_stamp = 0;
 
-// Returns device memory holding the plan for `seeds`, written on `stream` if it was not already
-// there; nullptr when no plan can be had (the caller then launches table by table).
-template <int NPTR>
-void *plan_cached(const std::vector<PlanSeed<NPTR>> &seeds, size_t tile, hipStream_t stream,
-                  int *rc) {
-    *rc = 0;
-    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess ||
-        capturing != hipStreamCaptureStatusNone) {
-        (void)hipGetLastError();
-        return nullptr;  // a captured launch must not lean on memory a later call may rewrite
+struct HipPlanBackend {
+    using Event = hipEvent_t;
+    void *alloc(size_t bytes) {
+        void *p = nullptr;
+        if (hipMalloc(&p, bytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        return p;
     }
-    int device = 0;
-    if (hipGetDevice(&device) != hipSuccess) return nullptr;
+    void free_blocking(int device, void *p) {  // hipFree waits for the device to drain
+        int current = 0;
+        (void)hipGetDevice(&current);
+        if (current != device) (void)hipSetDevice(device);
+        if (hipFree(p) != hipSuccess) (void)hipGetLastError();
+        if (current != device) (void)hipSetDevice(current);
+    }
+    bool record(void *stream, Event *out) {
+        if (hipEventCreateWithFlags(out, hipEventDisableTiming) != hipSuccess) {
+            (void)hipGetLastError();
+            return false;
+        }
+        if (hipEventRecord(*out, (hipStream_t)stream) != hipSuccess) {
+            (void)hipGetLastError();
+            (void)hipEventDestroy(*out);
+            return false;
+        }
+        return true;
+    }
+    bool done(const Event &e) {
+        if (hipEventQuery(e) == hipSuccess) return true;
+        (void)hipGetLastError();  // "not ready" is an answer, not an error to leave behind
+        return false;
+    }
+    void drop(Event &e) { (void)hipEventDestroy(e); }
+};
 
-    std::vector<unsigned char> key(16 + seeds.size() * sizeof(PlanSeed<NPTR>));
+using Plans = PlanCache<HipPlanBackend, PlanMemo>;
+Plans g_plans;
+
+// Called with g_plans.mutex() held.  Returns the slot whose device memory holds the plan for
+// `seeds`, written on `stream` if it was not already there; nullptr when no plan can be had (the
+// caller then launches table by table).  The caller enqueues its launch before it lets go of the
+// mutex.
+template <int NPTR>
+Plans::Slot *plan_cached(const std::vector<PlanSeed<NPTR>> &seeds, size_t tile, int device,
+                         hipStream_t stream, int *rc) {
+    *rc = 0;
+    Plans::Bytes key(16 + seeds.size() * sizeof(PlanSeed<NPTR>));
     const uint64_t head[2] = {(uint64_t)NPTR, (uint64_t)tile};
     std::memcpy(key.data(), head, 16);
     std::memcpy(key.data() + 16, seeds.data(), seeds.size() * sizeof(PlanSeed<NPTR>));
 
-    std::lock_guard<std::mutex> lock(g_plan_mutex);
-    PlanSlot *use = nullptr, *oldest = nullptr;
-    size_t mine = 0;
-    for (PlanSlot &slot : g_plan_slots) {
-        if (slot.device != device || slot.stream != stream) continue;
-        ++mine;
-        if (slot.key == key) use = &slot;
-        if (oldest == nullptr || slot.stamp < oldest->stamp) oldest = &slot;
-    }
-    if (use != nullptr) {
-        use->stamp = ++g_plan_stamp;
-        return use->mem;
-    }
     const uint64_t total_tiles = seeds.empty() ? 0 : seeds.back().next_first;
     uint32_t fine_shift = 0;
     const uint32_t fine_entries = plan_fine_entries(seeds.size(), total_tiles, &fine_shift);
-    const size_t need = plan_bytes(seeds.size(), fine_entries);
-    if (mine >= kPlanSlotsPerStream || (oldest != nullptr && g_plan_slots.size() >= kPlanSlotsTotal)) {
-        use = oldest;
-        if (use->capacity < need) {
-            // grow: the old memory may still be read by launches in flight on this stream
-            if (hipStreamSynchronize(stream) != hipSuccess) return nullptr;
-            (void)hipFree(use->mem);
-            use->mem = nullptr;
-            use->capacity = 0;
-        }
-    } else if (g_plan_slots.size() < kPlanSlotsTotal) {
-        g_plan_slots.emplace_back();
-        use = &g_plan_slots.back();
-        use->device = device;
-        use->stream = stream;
-    } else {
+    bool fresh = false;
+    Plans::Slot *slot = g_plans.acquire(device, (void *)stream, key,
+                                        plan_bytes(seeds.size(), fine_entries), &fresh);
+    if (slot == nullptr || !fresh) return slot;
+    *rc = plan_write_all<NPTR>(slot->mem, seeds, fine_entries, fine_shift, stream);
+    if (*rc) {
+        g_plans.invalidate(slot);
         return nullptr;
     }
-    if (use->mem == nullptr) {
-        const size_t capacity = need + need / 4;
-        if (hipMalloc(&use->mem, capacity) != hipSuccess) {
-            (void)hipGetLastError();
-            use->mem = nullptr;
-            use->key.clear();
-            return nullptr;
-        }
-        use->capacity = capacity;
-    }
-    use->key.clear();
-    use->call.clear();
-    *rc = plan_write<NPTR>(use->mem, seeds, stream);
-    if (*rc == 0 && fine_entries != 0) {
-        hipLaunchKernelGGL(plan_index_kernel, dim3((fine_entries + 255) / 256), dim3(256), 0, stream,
-                           static_cast<const PlanRec *>(use->mem), (uint32_t)seeds.size(),
-                           reinterpret_cast<uint32_t *>(static_cast<char *>(use->mem) +
-                                                        plan_record_bytes(seeds.size())),
-                           fine_entries, fine_shift);
-        *rc = (int)hipGetLastError();
-    }
-    if (*rc) return nullptr;
-    use->key = std::move(key);
-    use->stamp = ++g_plan_stamp;
-    return use->mem;
-}
-
-// The remembered call of a cached plan (see PlanSlot::call).
-bool plan_recall(hipStream_t stream, const std::vector<unsigned char> &call, PlanView *view,
-                 bool *staged) {
-    int device = 0;
-    if (hipGetDevice(&device) != hipSuccess) return false;
-    std::lock_guard<std::mutex> lock(g_plan_mutex);
-    for (PlanSlot &slot : g_plan_slots) {
-        if (slot.device != device || slot.stream != stream || slot.call != call) continue;
-        slot.stamp = ++g_plan_stamp;
-        *view = slot.view;
-        *staged = slot.staged;
-        return true;
-    }
-    return false;
-}
-
-void plan_remember(const void *mem, std::vector<unsigned char> &&call, const PlanView &view,
-                   bool staged) {
-    std::lock_guard<std::mutex> lock(g_plan_mutex);
-    for (PlanSlot &slot : g_plan_slots) {
-        if (slot.mem != mem || slot.key.empty()) continue;
-        slot.call = std::move(call);
-        slot.view = view;
-        slot.staged = staged;
-        return;
-    }
+    g_plans.commit(slot, std::move(key));
+    return slot;
 }
 
 // One address per op type: tells the remembered calls of different ops apart.
@@ -488,22 +454,29 @@ int launch_multi(MakeOp make_op, size_t num_tensors,
             std::memcpy(at, n, row);
             at += row;
             for (int i = 0; i < Op::NPTR; ++i, at += row) std::memcpy(at, lists[i], row);
-            PlanView view;
-            bool staged_before = false;
-            if (plan_recall((hipStream_t)stream, call, &view, &staged_before)) {
-                const Op op = make_op(count_all);
-                const unsigned lds = lds_reservation<Op>(staged_before, view.total, staged_before);
-                if (staged_before) {
-                    if constexpr (IsStaged<Op>::value)
-                        hipLaunchKernelGGL((plan_stream_kernel<T, Op, kUnroll, kNonTemporal, true>),
+            int device = 0;
+            if (hipGetDevice(&device) == hipSuccess) {
+                // lookup and launch are one step under the cache's mutex (plan_cache.hpp)
+                std::lock_guard<std::mutex> lock(g_plans.mutex());
+                if (Plans::Slot *slot = g_plans.find_call(device, stream, call)) {
+                    const PlanView &view = slot->memo.view;
+                    const bool staged_before = slot->memo.staged;
+                    const Op op = make_op(count_all);
+                    const unsigned lds =
+                        lds_reservation<Op>(staged_before, view.total, staged_before);
+                    if (staged_before) {
+                        if constexpr (IsStaged<Op>::value)
+                            hipLaunchKernelGGL(
+                                (plan_stream_kernel<T, Op, kUnroll, kNonTemporal, true>),
+                                dim3(grid_for(view.total)), dim3(kBlock), lds, (hipStream_t)stream,
+                                op, view);
+                    } else {
+                        hipLaunchKernelGGL((plan_stream_kernel<T, Op, kUnroll, kNonTemporal>),
                                            dim3(grid_for(view.total)), dim3(kBlock), lds,
                                            (hipStream_t)stream, op, view);
-                } else {
-                    hipLaunchKernelGGL((plan_stream_kernel<T, Op, kUnroll, kNonTemporal>),
-                                       dim3(grid_for(view.total)), dim3(kBlock), lds,
-                                       (hipStream_t)stream, op, view);
+                    }
+                    return (int)hipGetLastError();
                 }
-                return (int)hipGetLastError();
             }
         } else {
             (void)hipGetLastError();
@@ -601,24 +574,13 @@ int launch_multi(MakeOp make_op, size_t num_tensors,
                 seed.next_first = first;
                 seeds.push_back(seed);
             }
-            void *mem = nullptr;
-            if (arena != nullptr) {
-                if (plan_bytes(live, 0) > arena->bytes) return TOA_ELIMIT;
-                if (const int rc = plan_write<Op::NPTR>(arena->mem, seeds, (hipStream_t)stream))
-                    return rc;
-                mem = arena->mem;
-            } else {
-                int rc = 0;
-                mem = plan_cached<Op::NPTR>(seeds, tile, (hipStream_t)stream, &rc);
-                if (rc) return rc;
-            }
-            if (mem != nullptr) {
-                const uint32_t total = (uint32_t)tiles_all;
-                const PlanView view = plan_view<Op::NPTR>(mem, seeds, total, arena == nullptr);
-                // the lookup is two scalar-cache hits, so a plain launch wants the residency
-                // level of the single-tensor kernel, not the table kernel's raised one; a staged
-                // launch takes the op's level for staged lists
-                const unsigned lds = lds_reservation<Op>(staged, total, staged);
+            const uint32_t total = (uint32_t)tiles_all;
+            // the lookup is two scalar-cache hits, so a plain launch wants the residency level of
+            // the single-tensor kernel, not the table kernel's raised one; a staged launch takes
+            // the op's level for staged lists
+            const unsigned lds = lds_reservation<Op>(staged, total, staged);
+            auto launch_over = [&](void *mem, PlanView *view_out) -> int {
+                const PlanView view = plan_view<Op::NPTR>(mem, seeds, total);
                 if (staged) {
                     if constexpr (IsStaged<Op>::value)
                         hipLaunchKernelGGL((plan_stream_kernel<T, Op, kUnroll, kNonTemporal, true>),
@@ -629,9 +591,41 @@ int launch_multi(MakeOp make_op, size_t num_tensors,
                                        dim3(grid_for(total)), dim3(kBlock), lds,
                                        (hipStream_t)stream, op, view);
                 }
-                if (const int rc = (int)hipGetLastError()) return rc;
-                if (arena == nullptr && !call.empty()) plan_remember(mem, std::move(call), view, staged);
+                if (view_out != nullptr) *view_out = view;
+                return (int)hipGetLastError();
+            };
+            if (arena != nullptr) {
+                uint32_t fine_shift = 0;
+                const uint32_t fine_entries = plan_fine_entries(live, tiles_all, &fine_shift);
+                if (plan_bytes(live, fine_entries) > arena->bytes) return TOA_ELIMIT;
+                if (const int rc = plan_write_all<Op::NPTR>(arena->mem, seeds, fine_entries,
+                                                            fine_shift, (hipStream_t)stream))
+                    return rc;
+                if (const int rc = launch_over(arena->mem, nullptr)) return rc;
                 continue;
+            }
+            int device = 0;
+            hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+            // a captured launch must not lean on memory a later call may rewrite
+            const bool may_cache =
+                hipStreamIsCapturing((hipStream_t)stream, &capturing) == hipSuccess &&
+                capturing == hipStreamCaptureStatusNone && hipGetDevice(&device) == hipSuccess;
+            if (!may_cache) (void)hipGetLastError();
+            if (may_cache) {
+                // lookup, rewrite and the launch that reads the plan: one step under the cache's
+                // mutex (plan_cache.hpp)
+                std::lock_guard<std::mutex> lock(g_plans.mutex());
+                int rc = 0;
+                Plans::Slot *slot =
+                    plan_cached<Op::NPTR>(seeds, tile, device, (hipStream_t)stream, &rc);
+                if (rc) return rc;
+                if (slot != nullptr) {
+                    PlanMemo memo;
+                    memo.staged = staged;
+                    if ((rc = launch_over(slot->mem, &memo.view)) != 0) return rc;
+                    if (!call.empty()) g_plans.remember(slot, std::move(call), memo);
+                    continue;
+                }
             }
         } else if (arena != nullptr) {
             return TOA_ESIZE;
@@ -682,8 +676,10 @@ int launch_multi(MakeOp make_op, size_t num_tensors,
 // gives the address of the current device's copy, once per device.
 // ---------------------------------------------------------------------------
 constexpr size_t kNoAllocMaxTensors = 4096;
-constexpr size_t kNoAllocScratchBytes = kNoAllocMaxTensors * sizeof(PlanRec);  // 384 KiB
-static_assert(kNoAllocScratchBytes == toa_noalloc_scratch_bytes, "the array holds every record");
+constexpr size_t kNoAllocScratchBytes =
+    kNoAllocMaxTensors * sizeof(PlanRec) + 4 * kNoAllocMaxTensors * sizeof(uint32_t);  // 448 KiB
+static_assert(kNoAllocScratchBytes == toa_noalloc_scratch_bytes,
+              "the array holds every record and the finer index of the longest list");
 constexpr int kNoAllocMaxDevices = 64;
 
 }  // namespace
@@ -837,17 +833,9 @@ int toa_adam_set_plan_mode(int mode) {
 }
 
 int toa_adam_release_plans(void) {
-    std::lock_guard<std::mutex> lock(g_plan_mutex);
-    int rc = 0;
-    for (PlanSlot &slot : g_plan_slots) {
-        if (slot.mem == nullptr) continue;
-        int current = 0;
-        (void)hipGetDevice(&current);
-        if (current != slot.device) (void)hipSetDevice(slot.device);
-        if (const int e = (int)hipFree(slot.mem)) rc = e;  // waits for the device to drain
-        if (current != slot.device) (void)hipSetDevice(current);
-    }
-    g_plan_slots.clear();
+    std::lock_guard<std::mutex> lock(g_plans.mutex());
+    g_plans.release_all();
+    const int rc = (int)hipGetLastError();
     return rc;
 }
 
