@@ -132,8 +132,16 @@ def test_count_state_restored_from_elsewhere_is_read_once():
     assert_bit_equal(host(updates[0]), e, 'count 42')
 
 
-def test_differentiable_branch_matches_per_leaf_adam_op():
-    """inplace=False: the list-level autograd Functions give the same values and the same
+@pytest.fixture(params=['native_node', 'python_node'])
+def node(request, monkeypatch):
+    """Both routes of the differentiable list step: the C++ autograd node of the extension
+    module (the default) and the same node written in Python (what `torch.compile` traces)."""
+    monkeypatch.setattr(MultiAdamOp, 'use_native_node', request.param == 'native_node')
+    return request.param
+
+
+def test_differentiable_branch_matches_per_leaf_adam_op(node):
+    """inplace=False: the list-level autograd node gives the same values and the same
     gradients as the reference-shaped per-leaf AdamOp, bit for bit."""
     shapes = bench.maml_shapes()
     rng = np.random.default_rng(11)
@@ -167,7 +175,7 @@ def test_differentiable_branch_matches_per_leaf_adam_op():
 
 
 @pytest.mark.parametrize('which', ['updates_only', 'updates_and_mu', 'ragged'])
-def test_differentiable_branch_with_missing_outside_gradients(which):
+def test_differentiable_branch_with_missing_outside_gradients(which, node):
     """Only some outputs feed the loss: the one-pass backward must give what the per-leaf chain
     gives when autograd has nothing to add at new_mu / new_nu (for all leaves, or for some)."""
     shapes = [(7, 5), (300,), (3, 4, 5), ()]
@@ -205,7 +213,7 @@ def test_differentiable_branch_with_missing_outside_gradients(which):
 
 
 @pytest.mark.parametrize('which', ['no_update_gradient', 'mu_only', 'nothing_for_one_leaf'])
-def test_leaf_whose_update_receives_no_gradient(which):
+def test_leaf_whose_update_receives_no_gradient(which, node):
     """A leaf whose new_updates does not feed the loss: the per-leaf chain never runs
     backward_updates for it, so the infinities its new_updates / new_mu ratio may hold must not
     reach the gradients of the one-pass node either (0 * inf would be NaN), and a -0 outside
@@ -254,6 +262,72 @@ def test_leaf_whose_update_receives_no_gradient(which):
                 assert b.grad is None, f'{which} leaf {k}: {what} got a gradient from nowhere'
             else:
                 assert_bit_equal(host(b.grad), host(a.grad), f'{which} leaf {k} grad wrt {what}')
+
+
+def test_differentiable_branch_with_a_step_count_per_leaf(node):
+    """Leaves that have fallen out of step carry their own count (ints or 0-dim tensors); values
+    and gradients still equal the per-leaf chain's, also for a leaf whose update gets no
+    gradient while its neighbours' counts differ."""
+    rng = np.random.default_rng(44)
+    shapes = [(12, 3), (5,), (2, 2, 2), (31,)]
+    counts = [3, torch.tensor(7, device='cuda'), 3, 1]
+    data = [[np.asarray(rng.standard_normal(s), dtype=np.float64) for _ in range(3)]
+            for s in shapes]
+    cots = [np.asarray(rng.standard_normal(s), dtype=np.float64) for s in shapes]
+
+    def leaves():
+        return [[dev(a).requires_grad_(True) for a in (g, 0.1 * m, np.abs(0.01 * v) + 1e-3)]
+                for g, m, v in data]
+
+    def loss(outs):
+        # leaf 2 contributes through new_mu only: it takes the backward_mu route on its own
+        return sum((o[2] * dev(c)).sum() if k != 2 else (o[0] * dev(c)).sum()
+                   for k, (o, c) in enumerate(zip(outs, cots)))
+
+    single = leaves()
+    op = AdamOp(B1, B2, EPS, eps_root=1e-8, inplace=False)
+    loss([op(m, v, g, int(c)) for (g, m, v), c in zip(single, counts)]).backward()
+    multi = leaves()
+    mop = MultiAdamOp(B1, B2, EPS, eps_root=1e-8, inplace=False)
+    out = mop([x[1] for x in multi], [x[2] for x in multi], [x[0] for x in multi], counts)
+    loss(list(zip(*out))).backward()
+    for k in range(len(shapes)):
+        for a, b, what in zip(single[k], multi[k], ('updates', 'mu', 'nu')):
+            if a.grad is None:
+                assert b.grad is None, f'leaf {k}: {what} got a gradient from nowhere'
+            else:
+                assert_bit_equal(host(b.grad), host(a.grad), f'leaf {k} grad wrt {what}')
+
+
+def test_native_node_contract():
+    """What autograd sees of `adam_op.step_multi`: outputs that require grad exactly when an
+    input does, no graph under no_grad, fresh non-overlapping outputs of the inputs' layout, and
+    list lengths checked before anything is launched."""
+    from torchopt_amd._C import adam_op
+
+    g = [torch.randn(5, 7, device='cuda'), torch.randn(3, device='cuda')]
+    mu = [torch.zeros_like(x) for x in g]
+    nu = [torch.zeros_like(x) for x in g]
+    new_mu, new_nu, new_u = adam_op.step_multi(g, mu, nu, B1, B2, EPS, 0.0, 1)
+    assert isinstance(new_mu, list) and len(new_mu) == len(new_nu) == len(new_u) == 2
+    assert not any(t.requires_grad for t in new_mu + new_nu + new_u)
+    gl = [x.clone().requires_grad_(True) for x in g]
+    out = adam_op.step_multi(gl, mu, nu, B1, B2, EPS, 0.0, 1)
+    assert all(t.requires_grad and t.grad_fn is not None for lst in out for t in lst)
+    with torch.no_grad():
+        out = adam_op.step_multi(gl, mu, nu, B1, B2, EPS, 0.0, 1)
+    assert not any(t.requires_grad for lst in out for t in lst)
+    # outputs do not overlap one another or the inputs, and keep the inputs' shapes
+    spans = sorted((t.data_ptr(), t.data_ptr() + t.numel() * t.element_size())
+                   for lst in (out[0], out[1], out[2], g, mu, nu) for t in lst)
+    assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:]))
+    assert [t.shape for t in out[2]] == [x.shape for x in g]
+    assert all(t.data_ptr() % 16 == 0 for lst in out for t in lst)
+    with pytest.raises(RuntimeError, match='differ in length'):
+        adam_op.step_multi(g, mu[:1], nu, B1, B2, EPS, 0.0, 1)
+    with pytest.raises(RuntimeError, match='counts'):
+        adam_op.step_multi(g, mu, nu, B1, B2, EPS, 0.0, [1, 2, 3])
+    assert adam_op.step_multi([], [], [], B1, B2, EPS, 0.0, 1) == ([], [], [])
 
 
 def test_meta_step_through_the_transformation():
@@ -323,7 +397,7 @@ def test_chain_reduces_to_torch_optim_adam(inplace):
         torch.testing.assert_close(p - p0, q - p0, rtol=25 * 1e-7, atol=25 * 1e-7)
 
 
-def test_expanded_and_permuted_gradients_on_the_differentiable_branch():
+def test_expanded_and_permuted_gradients_on_the_differentiable_branch(node):
     """Gradients straight out of `torch.autograd.grad` may be expanded (stride 0, as the
     gradient of a sum is) or laid out differently from the moments; the list ops bring them to
     the moments' memory order instead of misreading them."""

@@ -123,10 +123,13 @@ class MultiAdamOp:
     (/root/reference/torchopt/transform/scale_by_adam.py:325-332): one launch, and on the
     differentiable path three autograd nodes with three forward and three backward launches,
     per leaf.  This callable takes the flattened tree at once: the in-place branch is one
-    `forward_multi_` call, and the differentiable branch is ONE autograd Function whose forward
+    `forward_multi_` call, and the differentiable branch is ONE autograd node whose forward
     (`forward_all_multi`) and backward (`backward_all_multi`) are one multi-tensor pass each, so
     a tree of any size costs two launches per step instead of six per leaf, and each direction
     reads its operands once.  Values and gradients are bit-identical to the per-leaf `AdamOp`.
+    The node lives in the extension module (`adam_op.step_multi`, a C++ autograd function: no
+    Python runs between autograd's engine and the launches); `StepOp` below is the same node
+    written in Python, the route taken while `torch.compile` traces.
 
     All lists must be free of ``None`` and live on one device with one dtype; the caller groups
     leaves accordingly.  `counts` is one step number for all leaves or one per leaf (ints or
@@ -205,6 +208,10 @@ class MultiAdamOp:
                     dnu[i] = dn[j]
             return (None, None, *dupdates, *dmu, *dnu)
 
+    # False routes the differentiable branch through the Python `StepOp` even outside
+    # `torch.compile` (the tests hold both routes to the per-leaf chain)
+    use_native_node = True
+
     def __init__(
         self,
         b1: float = 0.9,
@@ -230,6 +237,9 @@ class MultiAdamOp:
             adam_op.forward_multi_(updates, mus, nus, self.b1, self.b2, self.eps, self.eps_root,
                                    counts)
             return mus, nus, updates
+        if self.use_native_node and not torch.compiler.is_compiling():
+            return adam_op.step_multi(updates, mus, nus, self.b1, self.b2, self.eps,
+                                      self.eps_root, counts)
         hyper = (self.b1, self.b2, self.eps, self.eps_root, counts)
         out = self.StepOp.apply(hyper, k, *updates, *mus, *nus)
         return list(out[:k]), list(out[k:2 * k]), list(out[2 * k:])

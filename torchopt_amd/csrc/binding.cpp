@@ -24,6 +24,7 @@
 #include <c10/hip/HIPStream.h>
 #include <hip/hip_runtime_api.h>
 #include <pybind11/stl.h>
+#include <torch/csrc/autograd/custom_function.h>
 #include <torch/extension.h>
 
 #include <array>
@@ -431,10 +432,46 @@ Counts parseCounts(const py::object &counts, size_t num) {
     return out;
 }
 
+// Outputs shaped like `donors` (dtype, device, sizes and strides as at::empty_like gives them).
+// Leaves below 1 MiB share ONE allocation per list, each starting on a 256-byte boundary: a tree
+// of small leaves -- where the step is bound by host time, not bandwidth -- then costs one trip
+// to the allocator instead of one per leaf (2 us each, three lists a direction).  The leaves do
+// not overlap; what they share is the storage's lifetime (it lives as long as any of them) and
+// torch.save of a single leaf writing the whole storage.  Larger leaves get an allocation each.
+constexpr size_t kPooledLeafBytes = (size_t)1 << 20;
+
 TensorList emptyLike(const TensorList &donors) {
-    TensorList out;
-    out.reserve(donors.size());
-    for (const Tensor &t : donors) out.push_back(at::empty_like(t));
+    TensorList out(donors.size());
+    std::vector<size_t> at(donors.size());
+    size_t pooled = 0, bytes = 0, first = 0;
+    for (size_t k = 0; k < donors.size(); ++k) {
+        const Tensor &d = donors[k];
+        const size_t need = (size_t)d.numel() * d.element_size();
+        at[k] = SIZE_MAX;
+        if (!d.is_cuda() || need == 0 || need >= kPooledLeafBytes ||
+            !d.is_non_overlapping_and_dense() || d.layout() != at::kStrided)
+            continue;
+        if (pooled != 0 && d.device() != donors[first].device()) continue;
+        if (pooled++ == 0) first = k;
+        at[k] = bytes;
+        bytes += (need + 255) / 256 * 256;
+    }
+    if (pooled >= 2) {
+        const Tensor pool = at::empty({(int64_t)bytes}, donors[first].options().dtype(at::kByte));
+        const c10::Storage &storage = pool.storage();
+        for (size_t k = 0; k < donors.size(); ++k) {
+            if (at[k] == SIZE_MAX) continue;
+            const Tensor &d = donors[k];
+            Tensor t = at::detail::make_tensor<c10::TensorImpl>(c10::Storage(storage),
+                                                                 pool.key_set(), d.dtype());
+            c10::TensorImpl *impl = t.unsafeGetTensorImpl();
+            impl->set_storage_offset((int64_t)(at[k] / d.element_size()));
+            impl->set_sizes_and_strides(d.sizes(), d.strides());
+            out[k] = std::move(t);
+        }
+    }
+    for (size_t k = 0; k < donors.size(); ++k)
+        if (!out[k].defined()) out[k] = at::empty_like(donors[k]);
     return out;
 }
 
@@ -587,9 +624,9 @@ std::tuple<TensorList, TensorList> backwardUpdatesMulti(
     return {dmu_out, dnu_out};
 }
 
-std::tuple<TensorList, TensorList, TensorList> forwardAllMulti(
+std::tuple<TensorList, TensorList, TensorList> forwardAllMultiImpl(
     const TensorList &updates_in, const TensorList &mu, const TensorList &nu_in, double b1,
-    double b2, double eps, double eps_root, const py::object &counts) {
+    double b2, double eps, double eps_root, const Counts &c) {
     const char *name = "adamForwardAllMulti";
     TensorList new_mu = emptyLike(mu), new_nu = emptyLike(mu), new_updates = emptyLike(mu);
     // gradients may arrive expanded or in another memory order: bring them to mu's
@@ -597,7 +634,8 @@ std::tuple<TensorList, TensorList, TensorList> forwardAllMulti(
     const TensorList nu = asLayoutOfEach(nu_in, mu, name);
     Lists l = gateLists(name, {&updates, &mu, &nu, &new_mu, &new_nu, &new_updates});
     if (l.num) {
-        const Counts c = parseCounts(counts, l.num);
+        TORCH_CHECK(c.each.empty() || c.each.size() == l.num, name, ": expected ", l.num,
+                    " counts, got ", c.each.size());
         const OnDeviceOf dev(deviceDonor(mu));
         check(toa_adam_forward_all_multi(l.code, l.num, l.ptr[0].data(), l.ptr[1].data(),
                                          l.ptr[2].data(), l.n.data(), b1, b2, eps, eps_root,
@@ -608,13 +646,20 @@ std::tuple<TensorList, TensorList, TensorList> forwardAllMulti(
     return {new_mu, new_nu, new_updates};
 }
 
+std::tuple<TensorList, TensorList, TensorList> forwardAllMulti(
+    const TensorList &updates_in, const TensorList &mu, const TensorList &nu_in, double b1,
+    double b2, double eps, double eps_root, const py::object &counts) {
+    return forwardAllMultiImpl(updates_in, mu, nu_in, b1, b2, eps, eps_root,
+                               parseCounts(counts, mu.size()));
+}
+
 // dnew_mu / dnew_nu: a list of outside gradients, or None when there are none at all (a list
 // may not mix tensors and None: the caller substitutes -0.0 for the missing members).
-std::tuple<TensorList, TensorList, TensorList> backwardAllMulti(
+std::tuple<TensorList, TensorList, TensorList> backwardAllMultiImpl(
     const TensorList &dnew_updates_in, const c10::optional<TensorList> &dnew_mu_in,
     const c10::optional<TensorList> &dnew_nu_in, const TensorList &new_updates_in,
     const TensorList &new_mu, const TensorList &updates_in, double b1, double b2,
-    double eps_root, const py::object &counts) {
+    double eps_root, const Counts &c) {
     const char *name = "adamBackwardAllMulti";
     TensorList dupdates = emptyLike(new_mu), dmu = emptyLike(new_mu), dnu = emptyLike(new_mu);
     const TensorList du = asLayoutOfEach(dnew_updates_in, new_mu, name);
@@ -635,7 +680,8 @@ std::tuple<TensorList, TensorList, TensorList> backwardAllMulti(
     collect(dnew_mu_in, &ext_m, &pm);
     collect(dnew_nu_in, &ext_v, &pv);
     if (l.num) {
-        const Counts c = parseCounts(counts, l.num);
+        TORCH_CHECK(c.each.empty() || c.each.size() == l.num, name, ": expected ", l.num,
+                    " counts, got ", c.each.size());
         const OnDeviceOf dev(deviceDonor(new_mu));
         check(toa_adam_backward_all_multi(
                   l.code, l.num, l.ptr[0].data(), l.ptr[1].data(), l.ptr[2].data(),
@@ -646,6 +692,188 @@ std::tuple<TensorList, TensorList, TensorList> backwardAllMulti(
               name);
     }
     return {dupdates, dmu, dnu};
+}
+
+std::tuple<TensorList, TensorList, TensorList> backwardAllMulti(
+    const TensorList &dnew_updates_in, const c10::optional<TensorList> &dnew_mu_in,
+    const c10::optional<TensorList> &dnew_nu_in, const TensorList &new_updates_in,
+    const TensorList &new_mu, const TensorList &updates_in, double b1, double b2,
+    double eps_root, const py::object &counts) {
+    return backwardAllMultiImpl(dnew_updates_in, dnew_mu_in, dnew_nu_in, new_updates_in, new_mu,
+                                updates_in, b1, b2, eps_root, parseCounts(counts, new_mu.size()));
+}
+
+// ---- the differentiable step of a whole tree as ONE autograd node ----------------------------
+//
+// (updates, mu, nu) -> (new_mu, new_nu, new_updates) for every leaf: forward_all_multi forward,
+// backward_all_multi backward, one pass each.  Per leaf the values and gradients are those of the
+// reference's three Functions (/root/reference/torchopt/accelerated_op/adam_op.py:36-121):
+//   * saved for backward: new_updates, new_mu, updates (:44, :70, :104 between them);
+//   * a gradient for new_updates runs backward_updates, whose results join the gradients that
+//     reach new_mu / new_nu from outside (autograd's sums), then backward_mu and backward_nu, and
+//     the two contributions to d(updates) are added -- all inside backward_all, rounding for
+//     rounding;
+//   * a leaf whose new_updates received NO gradient never runs backward_updates in the per-leaf
+//     chain, so nothing of new_updates / new_mu (which may hold infinities) may enter: only the
+//     outside gradients flow on, through backward_mu / backward_nu, and a leaf with neither gets
+//     no gradient at all (undefined, not zeros: materialize_grads is off);
+//   * the hyper-parameters and the step numbers get no gradient.
+// Living in C++ it costs the host no Python between autograd's engine and the launch: the
+// same node written in Python spends 0.2 ms per step on a ten-leaf tree (list slicing, per-leaf
+// pybind conversions), twenty times what its two launches take on the device.
+class AdamStepNode : public torch::autograd::Function<AdamStepNode> {
+  public:
+    using variable_list = torch::autograd::variable_list;
+    using Context = torch::autograd::AutogradContext;
+
+    static variable_list forward(Context *ctx, at::TensorList updates, at::TensorList mu,
+                                 at::TensorList nu, double b1, double b2, double eps,
+                                 double eps_root, std::vector<int64_t> counts) {
+        const size_t k = mu.size();
+        auto [new_mu, new_nu, new_updates] = forwardAllMultiImpl(
+            updates.vec(), mu.vec(), nu.vec(), b1, b2, eps, eps_root, countsOf(counts, k));
+        variable_list keep;
+        keep.reserve(3 * k);
+        keep.insert(keep.end(), new_updates.begin(), new_updates.end());
+        keep.insert(keep.end(), new_mu.begin(), new_mu.end());
+        keep.insert(keep.end(), updates.begin(), updates.end());
+        ctx->save_for_backward(std::move(keep));
+        ctx->saved_data["b1"] = b1;
+        ctx->saved_data["b2"] = b2;
+        ctx->saved_data["eps_root"] = eps_root;
+        ctx->saved_data["counts"] = std::move(counts);
+        ctx->set_materialize_grads(false);  // a missing gradient must stay missing
+        variable_list out;
+        out.reserve(3 * k);
+        for (TensorList *l : {&new_mu, &new_nu, &new_updates})
+            for (Tensor &t : *l) out.push_back(std::move(t));
+        return out;
+    }
+
+    static variable_list backward(Context *ctx, variable_list grads) {
+        const variable_list saved = ctx->get_saved_variables();
+        const size_t k = saved.size() / 3;
+        TORCH_CHECK(grads.size() == 3 * k, "adamStep: expected ", 3 * k, " gradients, got ",
+                    grads.size());
+        const double b1 = ctx->saved_data["b1"].toDouble(), b2 = ctx->saved_data["b2"].toDouble(),
+                     eps_root = ctx->saved_data["eps_root"].toDouble();
+        const std::vector<int64_t> counts = ctx->saved_data["counts"].toIntVector();
+        auto part = [&](const variable_list &v, size_t j) {
+            return TensorList(v.begin() + j * k, v.begin() + (j + 1) * k);
+        };
+        const TensorList new_updates = part(saved, 0), new_mu = part(saved, 1),
+                         updates = part(saved, 2);
+        const TensorList g_mu = part(grads, 0), g_nu = part(grads, 1), g_u = part(grads, 2);
+
+        // d(updates), d(mu), d(nu) per leaf, then nothing for the five non-tensor arguments
+        variable_list result(3 * k + 5);
+        Tensor *dupdates = result.data(), *dmu = result.data() + k, *dnu = result.data() + 2 * k;
+
+        std::vector<size_t> live, via_mu, via_nu;
+        for (size_t i = 0; i < k; ++i) {
+            if (g_u[i].defined()) {
+                live.push_back(i);
+            } else {
+                if (g_mu[i].defined()) via_mu.push_back(i);
+                if (g_nu[i].defined()) via_nu.push_back(i);
+            }
+        }
+        auto pick = [](const TensorList &from, const std::vector<size_t> &idx) {
+            if (idx.size() == from.size()) return from;
+            TensorList out;
+            out.reserve(idx.size());
+            for (size_t i : idx) out.push_back(from[i]);
+            return out;
+        };
+        auto counts_of = [&](const std::vector<size_t> &idx) {
+            if (counts.size() <= 1 || idx.size() == k) return countsOf(counts, k);
+            std::vector<int64_t> some;
+            some.reserve(idx.size());
+            for (size_t i : idx) some.push_back(counts[i]);
+            return countsOf(some, idx.size());
+        };
+        if (!live.empty()) {
+            // Gradients reaching new_mu / new_nu from outside the step.  None at all: the kernel
+            // skips the addition, as autograd would.  Some: members without one get -0.0, the
+            // exact identity of IEEE addition (x + -0.0 is x for every x, signed zeros
+            // included), so they too come out as if nothing had been added.
+            auto outside = [&](const TensorList &gs) -> c10::optional<TensorList> {
+                bool any = false;
+                for (size_t i : live) any = any || gs[i].defined();
+                if (!any) return c10::nullopt;
+                TensorList out;
+                out.reserve(live.size());
+                for (size_t i : live)
+                    out.push_back(gs[i].defined() ? gs[i] : at::full_like(new_mu[i], -0.0));
+                return out;
+            };
+            auto [du, dm, dn] = backwardAllMultiImpl(
+                pick(g_u, live), outside(g_mu), outside(g_nu), pick(new_updates, live),
+                pick(new_mu, live), pick(updates, live), b1, b2, eps_root, counts_of(live));
+            for (size_t j = 0; j < live.size(); ++j) {
+                dupdates[live[j]] = std::move(du[j]);
+                dmu[live[j]] = std::move(dm[j]);
+                dnu[live[j]] = std::move(dn[j]);
+            }
+        }
+        if (!via_mu.empty()) {
+            const TensorList donors = pick(updates, via_mu);
+            auto [du, dm] = backwardMuMulti(pick(g_mu, via_mu), donors, donors, b1);
+            for (size_t j = 0; j < via_mu.size(); ++j) {
+                dupdates[via_mu[j]] = std::move(du[j]);
+                dmu[via_mu[j]] = std::move(dm[j]);
+            }
+        }
+        if (!via_nu.empty()) {
+            const TensorList donors = pick(updates, via_nu);
+            auto [du, dn] = backwardNuMulti(pick(g_nu, via_nu), donors, donors, b2);
+            for (size_t j = 0; j < via_nu.size(); ++j) {
+                const size_t i = via_nu[j];
+                // autograd adds the two contributions to d(updates) where both exist
+                dupdates[i] = dupdates[i].defined() ? dupdates[i] + du[j] : std::move(du[j]);
+                dnu[i] = std::move(dn[j]);
+            }
+        }
+        return result;
+    }
+
+  private:
+    static Counts countsOf(const std::vector<int64_t> &values, size_t num) {
+        Counts c;
+        if (values.size() == 1) {
+            c.all = (uint64_t)values[0];
+        } else {
+            TORCH_CHECK(values.size() == num, "adamStep: expected ", num, " counts, got ",
+                        values.size());
+            c.each.assign(values.begin(), values.end());
+        }
+        return c;
+    }
+};
+
+// (new_mu, new_nu, new_updates) as lists, differentiable with respect to every tensor of the
+// three input lists.  `counts` as for the other list functions.
+py::tuple stepMulti(const py::object &updates_o, const py::object &mu_o, const py::object &nu_o,
+                    double b1, double b2, double eps, double eps_root, const py::object &counts) {
+    const TensorList updates = toTensorList(updates_o, "updates");
+    const TensorList mu = toTensorList(mu_o, "mu");
+    const TensorList nu = toTensorList(nu_o, "nu");
+    const size_t k = mu.size();
+    TORCH_CHECK(updates.size() == k && nu.size() == k, "adamStep: tensor lists differ in length");
+    const Counts c = parseCounts(counts, k);
+    std::vector<int64_t> values;
+    if (c.each.empty())
+        values.push_back((int64_t)c.all);
+    else
+        values.assign(c.each.begin(), c.each.end());
+    for (int64_t v : values)
+        if (v < 0) throw py::type_error("counts beyond INT64_MAX are not served here");
+    const auto out = AdamStepNode::apply(at::TensorList(updates), at::TensorList(mu),
+                                         at::TensorList(nu), b1, b2, eps, eps_root, values);
+    py::list lists[3];
+    for (int j = 0; j < 3; ++j)
+        for (size_t i = 0; i < k; ++i) lists[j].append(py::cast(out[j * k + i]));
+    return py::make_tuple(lists[0], lists[1], lists[2]);
 }
 
 py::tuple fusedStepMulti(const py::object &params_o, const py::object &updates_o,
@@ -844,6 +1072,11 @@ PYBIND11_MODULE(_C, mod) {
     m.def("backward_all_multi", &backwardAllMulti, "backward_all over lists", "dnew_updates"_a,
           "dnew_mu"_a, "dnew_nu"_a, "new_updates"_a, "new_mu"_a, "updates"_a, "b1"_a, "b2"_a,
           "eps_root"_a, "counts"_a);
+
+    m.def("step_multi", &stepMulti,
+          "the differentiable step of a whole list as one autograd node -> "
+          "(new_mu, new_nu, new_updates)",
+          "updates"_a, "mu"_a, "nu"_a, "b1"_a, "b2"_a, "eps"_a, "eps_root"_a, "counts"_a);
 
     // the classic in-place optimizer step in one pass
     m.def("fused_step_", &fusedStep,
