@@ -87,6 +87,35 @@ TOA_API int toa_adam_set_waves_per_cu(int waves);
  * Returns the previous setting.  No counterpart in the reference. */
 TOA_API int toa_adam_set_schedule(int schedule);
 
+/* Tuning knob: load order of the staged in-place step on one large tensor.  The staged program
+ * handles the gradient and the two moments one memory operation at a time; which moment goes
+ * first, and whether it is loaded before the gradient, does not change a bit of the result but
+ * moves the rate by up to 1 % with where the three arrays lie:
+ *   0  g | mu | store mu', nu | store nu', store u'      2  mu | g | store mu', nu | ...
+ *   1  g | nu | store nu', mu | store mu', store u'      3  nu | g | store nu', mu | ...
+ *  -1  (default) the library's choice.
+ * bfloat16, lists and the other ops have one order; the setting is ignored there.  Returns the
+ * previous setting.  No counterpart in the reference.
+ *
+ * The library's choice is made per call site -- the in-place step on one set of three arrays of
+ * one length, 64 MiB or more each -- by measurement on the caller's own launches: the first 24
+ * launches of a site go round the four orders (same bits every time), timed with events on the
+ * caller's stream that are polled, never waited for; rounds alternate their direction and the
+ * first two do not count, so a drift of the machine's rate cancels.  The fastest order is kept if
+ * it beats order 0 by more than 0.15 %, order 0 otherwise.  On most placements order 0 wins; on
+ * some another gains 1-2 %.  Up to 64 call sites are remembered.  Nothing is tuned under stream
+ * capture, with an order or a residency level forced, or with a schedule other than 0.
+ *   toa_adam_set_tuning         0 = every site runs order 0; 1 (default; the environment variable
+ *                               TOA_ADAM_TUNING=0 starts with 0) = as above.  Returns the previous
+ *                               setting.
+ *   toa_adam_tuned_load_order   the order kept for that call site of toa_adam_forward_inplace
+ *                               (or its _devcount form uses a site of its own), or -1 while it is
+ *                               unknown or still being explored. */
+TOA_API int toa_adam_set_load_order(int order);
+TOA_API int toa_adam_set_tuning(int on);
+TOA_API int toa_adam_tuned_load_order(int dtype, const void *updates, const void *mu,
+                                      const void *nu, size_t n);
+
 /* Lists longer than one kernel-argument table (96 tensors for ops with three pointer slots, 80
  * with four, 64 with five, fewer beyond), and lists of 256 MiB or more per array whatever their
  * length, run as ONE launch over a device-resident table, a

@@ -32,6 +32,8 @@ def _gpu():
     yield
     lib.toa_adam_set_schedule(0)
     lib.toa_adam_set_waves_per_cu(0)
+    lib.toa_adam_set_load_order(-1)
+    lib.toa_adam_set_tuning(1)
     torch.cuda.synchronize()
 
 
@@ -98,6 +100,116 @@ def test_staged_schedule_at_every_residency_level(levels):
         assert rc == 0, lib.toa_adam_error_string(rc)
         for got, exp, name in zip((du, dm, dv), want, ('updates', 'mu', 'nu')):
             assert_bit_equal(host(got, 'f32'), exp, f'waves {w} {name}')
+
+
+@pytest.mark.parametrize('tag', ['f32', 'f64', 'f16', 'bf16'])
+def test_every_load_order_of_the_staged_step_matches_the_oracle(tag):
+    """Which moment the staged program handles first, and whether it loads it before the
+    gradient, moves the rate with the placement of the arrays and nothing else: all four orders
+    (bfloat16 has one, whatever is asked for), at the three residency levels around the default,
+    give the oracle's bits -- through the host-counted and the device-counted entry point."""
+    lib = _lib.load()
+    n = BIG[tag]
+    eps, eps_root, count = (1e-8, 1e-8, 7) if tag in ('f32', 'f64') else (1e-3, 0.0, 7)
+    u, m, v = draw(tag, n, 21)
+    want = O.forward_inplace(u.copy(), m.copy(), v.copy(), B1, B2, eps, eps_root, count)
+    stream = torch.cuda.current_stream().cuda_stream
+    rows = 4
+    table = torch.empty(rows, 4, dtype=TORCH[tag])
+    assert lib.toa_adam_bias_rows(CODE[tag], B1, B2, eps_root, count - 1, rows,
+                                  table.data_ptr()) == 0
+    table = table.cuda()
+    step = torch.tensor(count, dtype=torch.int64, device='cuda')
+    lib.toa_adam_set_schedule(2)
+    try:
+        for order in range(4):
+            for waves in (16, 18, 21):
+                lib.toa_adam_set_load_order(order)
+                lib.toa_adam_set_waves_per_cu(waves)
+                for devcount in (False, True):
+                    du, dm, dv = (dev(a, tag) for a in (u, m, v))
+                    print(f'forward_inplace {tag} n={n} staged order={order} waves={waves} '
+                          f'devcount={devcount}', flush=True)
+                    if devcount:
+                        rc = lib.toa_adam_forward_inplace_devcount(
+                            CODE[tag], du.data_ptr(), dm.data_ptr(), dv.data_ptr(), n, B1, B2, eps,
+                            eps_root, table.data_ptr(), count - 1, rows, step.data_ptr(), stream)
+                    else:
+                        rc = lib.toa_adam_forward_inplace(
+                            CODE[tag], du.data_ptr(), dm.data_ptr(), dv.data_ptr(), n, B1, B2, eps,
+                            eps_root, count, stream)
+                    assert rc == 0, lib.toa_adam_error_string(rc)
+                    for got, exp, name in zip((du, dm, dv), want, ('updates', 'mu', 'nu')):
+                        assert_bit_equal(host(got, tag), exp,
+                                         f'{tag} order {order} waves {waves} {name}')
+    finally:
+        lib.toa_adam_set_schedule(0)
+        lib.toa_adam_set_load_order(-1)
+        lib.toa_adam_set_waves_per_cu(0)
+
+
+@pytest.mark.parametrize('tag', ['f32', 'f64'])
+def test_the_load_order_is_chosen_per_call_site_and_changes_no_bit(tag):
+    """A call site of 64 MiB per array is explored over its first 24 launches (four orders, six
+    rounds) and then keeps one order; forty steps on it give the bits of forty steps with tuning
+    off (order 0 throughout) -- and, for the first of them, the oracle's.  With tuning off, under
+    a forced order or below the size limit no site is recorded."""
+    lib = _lib.load()
+    esize = {'f32': 4, 'f64': 8}[tag]
+    n = (64 << 20) // esize + 1000  # whole tiles of 64 MiB and a ragged tail
+    u, m, v = draw(tag, n, 31)
+    first = O.forward_inplace(u.copy(), m.copy(), v.copy(), B1, B2, 1e-8, 1e-8, 1)
+    stream = torch.cuda.current_stream().cuda_stream
+    code = CODE[tag]
+
+    def steps(arrays, count):
+        for k in range(count):
+            rc = lib.toa_adam_forward_inplace(code, *[a.data_ptr() for a in arrays], n, B1, B2,
+                                              1e-8, 1e-8, k + 1, stream)
+            assert rc == 0, lib.toa_adam_error_string(rc)
+
+    tuned = [dev(a, tag) for a in (u, m, v)]
+    plain = [dev(a, tag) for a in (u, m, v)]
+    site = lambda arrays: lib.toa_adam_tuned_load_order(code, *[a.data_ptr() for a in arrays], n)
+
+    lib.toa_adam_set_tuning(0)
+    print(f'forward_inplace {tag} n={n} forty steps, tuning off', flush=True)
+    steps(plain, 40)
+    torch.cuda.synchronize()
+    assert site(plain) == -1
+    lib.toa_adam_set_tuning(1)
+    assert site(tuned) == -1
+    print(f'forward_inplace {tag} n={n} first step of a tuned site', flush=True)
+    steps(tuned, 1)
+    torch.cuda.synchronize()
+    for got, exp, name in zip(tuned, first, ('updates', 'mu', 'nu')):
+        assert_bit_equal(host(got, tag), exp, f'{tag} first tuned step {name}')
+    print(f'forward_inplace {tag} n={n} thirty-nine more steps of the tuned site', flush=True)
+    for k in range(1, 40):
+        rc = lib.toa_adam_forward_inplace(code, *[a.data_ptr() for a in tuned], n, B1, B2, 1e-8,
+                                          1e-8, k + 1, stream)
+        assert rc == 0
+        if k in (5, 23):
+            assert site(tuned) == -1 or k == 23  # exploring: nothing is decided before 24 launches
+    torch.cuda.synchronize()
+    assert site(tuned) in (0, 1, 2, 3)  # every sample is back: decided
+    for a, b, name in zip(tuned, plain, ('updates', 'mu', 'nu')):
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32)), f'{tag} tuned != untuned {name}'
+    # no site for a forced order, a forced level, or arrays below the limit
+    others = [dev(a, tag) for a in (u, m, v)]
+    lib.toa_adam_set_load_order(2)
+    steps(others, 2)
+    lib.toa_adam_set_load_order(-1)
+    lib.toa_adam_set_waves_per_cu(18)
+    steps(others, 2)
+    lib.toa_adam_set_waves_per_cu(0)
+    torch.cuda.synchronize()
+    assert site(others) == -1
+    small = [t[:BIG[tag]] for t in others]
+    rc = lib.toa_adam_forward_inplace(code, *[a.data_ptr() for a in small], BIG[tag], B1, B2, 1e-8,
+                                      1e-8, 1, stream)
+    assert rc == 0
+    assert lib.toa_adam_tuned_load_order(code, *[a.data_ptr() for a in small], BIG[tag]) == -1
 
 
 @pytest.mark.parametrize('alias', ['mu is nu', 'all three'])

@@ -34,6 +34,9 @@ SIGNATURES = {
     'toa_adam_set_waves_per_cu': [_i],
     'toa_adam_set_max_grid': [ctypes.c_uint],
     'toa_adam_set_schedule': [_i],
+    'toa_adam_set_load_order': [_i],
+    'toa_adam_set_tuning': [_i],
+    'toa_adam_tuned_load_order': [_i, _vp, _vp, _vp, _sz],
     'toa_adam_set_plan_mode': [_i],
     'toa_adam_release_plans': [],
     'toa_adam_state_slack': [],

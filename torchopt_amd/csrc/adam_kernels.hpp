@@ -543,6 +543,16 @@ __device__ __forceinline__ Op live_op(const Op &op) {
     return live;
 }
 
+// Load orders of an op's staged program (1 unless the op says otherwise).
+template <class Op, class = void>
+struct LoadOrders {
+    static constexpr int value = 1;
+};
+template <class Op>
+struct LoadOrders<Op, decltype((void)Op::kLoadOrders)> {
+    static constexpr int value = Op::kLoadOrders;
+};
+
 // What a staged op sees of its tile: one 128-bit vector per lane of every array.
 template <typename T, class Op, bool NT>
 struct StagedIO {
@@ -642,8 +652,8 @@ struct alignas(8) AdamSteps {
             out = adam_direction(mh, vh, eps_root, eps);
         return ok;
     }
-    // load in0 | load in1 | store out0, load in2 | store out1, store out2
-    template <class Op, class IO>
+    // load in0 | load in1 | store out0, load in2 | store out1, store out2 (ORDER 0; see below)
+    template <class Op, int ORDER = 0, class IO>
     __device__ __forceinline__ void staged_steps(const IO &io) const {
         using V = typename Vec<T>::type;
         constexpr int VN = Vec<T>::N;
@@ -691,16 +701,37 @@ struct alignas(8) AdamSteps {
             }
             io.store(Op::out_slot(2), res);
         } else {
-            const V g = io.load(0);
+            // ORDER picks which moment is handled first and whether it is loaded before the
+            // gradient: 0 = g, mu, nu; 1 = g, nu, mu; 2 = mu, g, nu; 3 = nu, g, mu.  The results
+            // do not depend on it.
+            constexpr bool nu_first = ORDER == 1 || ORDER == 3;
+            constexpr bool moment_before_gradient = ORDER >= 2;
+            constexpr int in_a = nu_first ? 2 : 1, in_b = nu_first ? 1 : 2;
+            constexpr int out_a = nu_first ? 1 : 0, out_b = nu_first ? 0 : 1;
+            auto moment = [&](bool second_moment, const V &gg, const V &x) {
+                return second_moment ? vmap<T>(gg, x, [&](T p, T q) { return second<T>(p, q); })
+                                     : vmap<T>(gg, x, [&](T p, T q) { return first<T>(p, q); });
+            };
+            V g, xa;
+            if constexpr (moment_before_gradient) {
+                xa = io.load(in_a);
+                io.wait();
+                g = io.load(0);
+                io.wait();
+            } else {
+                g = io.load(0);
+                io.wait();
+                xa = io.load(in_a);
+                io.wait();
+            }
+            const V ra = moment(nu_first, g, xa);
+            io.store(Op::out_slot(out_a), ra);
+            const V xb = io.load(in_b);
             io.wait();
-            const V m = io.load(1);
-            io.wait();
-            const V a = vmap<T>(g, m, [&](T x, T y) { return first<T>(x, y); });
-            io.store(Op::out_slot(0), a);
-            const V v = io.load(2);
-            io.wait();
-            const V b = vmap<T>(g, v, [&](T x, T y) { return second<T>(x, y); });
-            io.store(Op::out_slot(1), b);
+            const V rb = moment(!nu_first, g, xb);
+            io.store(Op::out_slot(out_b), rb);
+            const V &a = nu_first ? rb : ra;  // the new first moment
+            const V &b = nu_first ? ra : rb;  // the new second moment
             V c;
             if constexpr (HasQuickDirection<T>::value) {
                 uint32_t redo = 0;
@@ -757,9 +788,16 @@ struct ForwardInplace : AdamSteps<T> {
     __device__ static constexpr int out_slot(int j) { return j == 0 ? 1 : (j == 1 ? 2 : 0); }
     static constexpr bool kSpeculative = HasQuickDirection<T>::value;
     static constexpr bool kPairs = true;
+    // The staged program exists in four load orders (bfloat16, which computes in pairs, in one):
+    // which order streams fastest depends on where the three arrays lie, see staged_steps.
+    static constexpr int kLoadOrders = __is_same(T, bfloat_t) ? 1 : 4;
     template <class IO>
     __device__ __forceinline__ void staged(const IO &io) const {
-        this->template staged_steps<ForwardInplace>(io);
+        this->template staged_steps<ForwardInplace, 0>(io);
+    }
+    template <int ORDER, class IO>
+    __device__ __forceinline__ void staged_in_order(const IO &io) const {
+        this->template staged_steps<ForwardInplace, ORDER>(io);
     }
 };
 
@@ -1241,11 +1279,16 @@ __device__ __forceinline__ void tile_full(const Op &op, const TensorPtrs<T, Op> 
 // next load go out together), every result stored as soon as it exists.  Same arithmetic as
 // tile_full, other order of memory operations -- so the arrays of a tensor must not overlap one
 // another (the host checks; tile_full loads everything before it stores).
-template <typename T, class Op, bool NT>
+template <typename T, class Op, bool NT, int ORDER = 0>
 __device__ __forceinline__ void tile_full_staged(const Op &op, const TensorPtrs<T, Op> &tp,
                                                  size_t vec_base) {
     const StagedIO<T, Op, NT> io{tp.p, vec_base + threadIdx.x};
-    op.staged(io);
+    if constexpr (ORDER != 0) {
+        static_assert(ORDER < LoadOrders<Op>::value, "the op has no such load order");
+        op.template staged_in_order<ORDER>(io);
+    } else {
+        op.staged(io);
+    }
 }
 
 // All pointers 16-byte aligned, tile cut short by the end of the tensor:
@@ -1361,13 +1404,14 @@ __global__ __launch_bounds__(kBlock) void stream_kernel(const Op op, const Tenso
 // The common case without its branches: every pointer 16-byte aligned and only whole tiles,
 // one workgroup per tile.  The host launches this over the whole tiles of a tensor and hands a
 // ragged last tile to stream_kernel.
-template <typename T, class Op, int UNROLL, bool NT, bool STAGED = false>
+template <typename T, class Op, int UNROLL, bool NT, bool STAGED = false, int ORDER = 0>
 __global__ __launch_bounds__(kBlock) void full_tiles_kernel(const Op op,
                                                             const TensorPtrs<T, Op> tp) {
     static_assert(!STAGED || UNROLL == 1, "the staged schedule handles one vector per lane");
+    static_assert(STAGED || ORDER == 0, "load orders belong to the staged schedule");
     const Op live = live_op(op);
     if constexpr (STAGED)
-        tile_full_staged<T, Op, NT>(live, tp, (size_t)blockIdx.x * Tile<T, UNROLL>::VECS);
+        tile_full_staged<T, Op, NT, ORDER>(live, tp, (size_t)blockIdx.x * Tile<T, UNROLL>::VECS);
     else
         tile_full<T, Op, UNROLL, NT>(live, tp, (size_t)blockIdx.x * Tile<T, UNROLL>::VECS);
 }

@@ -432,16 +432,17 @@ Counts parseCounts(const py::object &counts, size_t num) {
     return out;
 }
 
-// Outputs shaped like `donors` (dtype, device, sizes and strides as at::empty_like gives them).
-// Leaves below 1 MiB share ONE allocation per list, each starting on a 256-byte boundary: a tree
-// of small leaves -- where the step is bound by host time, not bandwidth -- then costs one trip
-// to the allocator instead of one per leaf (2 us each, three lists a direction).  The leaves do
-// not overlap; what they share is the storage's lifetime (it lives as long as any of them) and
-// torch.save of a single leaf writing the whole storage.  Larger leaves get an allocation each.
+// `sets` lists of outputs shaped like `donors` (dtype, device, sizes and strides as
+// at::empty_like gives them).  Leaves below 1 MiB share ONE allocation per call, each starting on
+// a 256-byte boundary: a tree of small leaves -- where the step is bound by host time, not
+// bandwidth -- then costs one trip to the allocator instead of one per leaf and list (2-3 us
+// each).  The leaves do not overlap; what they share is the storage's lifetime (it lives as long
+// as any of them) and torch.save of a single leaf writing the whole storage.  Larger leaves get
+// an allocation each.
 constexpr size_t kPooledLeafBytes = (size_t)1 << 20;
 
-TensorList emptyLike(const TensorList &donors) {
-    TensorList out(donors.size());
+std::vector<TensorList> emptyLikeSets(const TensorList &donors, size_t sets) {
+    std::vector<TensorList> out(sets, TensorList(donors.size()));
     std::vector<size_t> at(donors.size());
     size_t pooled = 0, bytes = 0, first = 0;
     for (size_t k = 0; k < donors.size(); ++k) {
@@ -456,24 +457,29 @@ TensorList emptyLike(const TensorList &donors) {
         at[k] = bytes;
         bytes += (need + 255) / 256 * 256;
     }
-    if (pooled >= 2) {
-        const Tensor pool = at::empty({(int64_t)bytes}, donors[first].options().dtype(at::kByte));
+    if (pooled * sets >= 2) {
+        const Tensor pool =
+            at::empty({(int64_t)(bytes * sets)}, donors[first].options().dtype(at::kByte));
         const c10::Storage &storage = pool.storage();
-        for (size_t k = 0; k < donors.size(); ++k) {
-            if (at[k] == SIZE_MAX) continue;
-            const Tensor &d = donors[k];
-            Tensor t = at::detail::make_tensor<c10::TensorImpl>(c10::Storage(storage),
-                                                                 pool.key_set(), d.dtype());
-            c10::TensorImpl *impl = t.unsafeGetTensorImpl();
-            impl->set_storage_offset((int64_t)(at[k] / d.element_size()));
-            impl->set_sizes_and_strides(d.sizes(), d.strides());
-            out[k] = std::move(t);
-        }
+        for (size_t j = 0; j < sets; ++j)
+            for (size_t k = 0; k < donors.size(); ++k) {
+                if (at[k] == SIZE_MAX) continue;
+                const Tensor &d = donors[k];
+                Tensor t = at::detail::make_tensor<c10::TensorImpl>(c10::Storage(storage),
+                                                                     pool.key_set(), d.dtype());
+                c10::TensorImpl *impl = t.unsafeGetTensorImpl();
+                impl->set_storage_offset((int64_t)((j * bytes + at[k]) / d.element_size()));
+                impl->set_sizes_and_strides(d.sizes(), d.strides());
+                out[j][k] = std::move(t);
+            }
     }
-    for (size_t k = 0; k < donors.size(); ++k)
-        if (!out[k].defined()) out[k] = at::empty_like(donors[k]);
+    for (size_t j = 0; j < sets; ++j)
+        for (size_t k = 0; k < donors.size(); ++k)
+            if (!out[j][k].defined()) out[j][k] = at::empty_like(donors[k]);
     return out;
 }
+
+TensorList emptyLike(const TensorList &donors) { return std::move(emptyLikeSets(donors, 1)[0]); }
 
 TensorList asLayoutOfEach(const TensorList &xs, const TensorList &donors, const char *name) {
     TORCH_CHECK(xs.size() == donors.size(), name, ": tensor lists differ in length");
@@ -573,7 +579,8 @@ std::tuple<TensorList, TensorList> backwardMuMulti(const TensorList &dmu_in,
                                                    const TensorList &mu, double b1) {
     const char *name = "adamBackwardMuMulti";
     TORCH_CHECK(updates.size() == mu.size(), name, ": tensor lists differ in length");
-    TensorList dupdates_out = emptyLike(mu), dmu_out = emptyLike(mu);
+    std::vector<TensorList> fresh = emptyLikeSets(mu, 2);
+    TensorList &dupdates_out = fresh[0], &dmu_out = fresh[1];
     const TensorList dmu = asLayoutOfEach(dmu_in, dmu_out, name);
     Lists l = gateLists(name, {&dmu_out, &dmu, &dupdates_out});
     if (l.num) {
@@ -582,14 +589,15 @@ std::tuple<TensorList, TensorList> backwardMuMulti(const TensorList &dmu_in,
                                          l.ptr[2].data(), l.ptr[0].data(), dev.stream()),
               name);
     }
-    return {dupdates_out, dmu_out};
+    return {std::move(dupdates_out), std::move(dmu_out)};
 }
 
 std::tuple<TensorList, TensorList> backwardNuMulti(const TensorList &dnu_in,
                                                    const TensorList &updates_in,
                                                    const TensorList &nu, double b2) {
     const char *name = "adamBackwardNuMulti";
-    TensorList dupdates_out = emptyLike(nu), dnu_out = emptyLike(nu);
+    std::vector<TensorList> fresh = emptyLikeSets(nu, 2);
+    TensorList &dupdates_out = fresh[0], &dnu_out = fresh[1];
     const TensorList dnu = asLayoutOfEach(dnu_in, dnu_out, name);
     const TensorList updates = asLayoutOfEach(updates_in, nu, name);
     Lists l = gateLists(name, {&dnu, &updates, &dupdates_out, &dnu_out});
@@ -600,7 +608,7 @@ std::tuple<TensorList, TensorList> backwardNuMulti(const TensorList &dnu_in,
                                          dev.stream()),
               name);
     }
-    return {dupdates_out, dnu_out};
+    return {std::move(dupdates_out), std::move(dnu_out)};
 }
 
 std::tuple<TensorList, TensorList> backwardUpdatesMulti(
@@ -608,7 +616,8 @@ std::tuple<TensorList, TensorList> backwardUpdatesMulti(
     const TensorList &new_nu, double b1, double b2, double eps_root, const py::object &counts) {
     const char *name = "adamBackwardUpdatesMulti";
     TORCH_CHECK(new_nu.size() == new_mu.size(), name, ": tensor lists differ in length");
-    TensorList dmu_out = emptyLike(new_mu), dnu_out = emptyLike(new_mu);
+    std::vector<TensorList> fresh = emptyLikeSets(new_mu, 2);
+    TensorList &dmu_out = fresh[0], &dnu_out = fresh[1];
     const TensorList dupdates = asLayoutOfEach(dupdates_in, dmu_out, name);
     const TensorList updates = asLayoutOfEach(updates_in, new_mu, name);
     Lists l = gateLists(name, {&dupdates, &updates, &new_mu, &dmu_out, &dnu_out});
@@ -621,14 +630,15 @@ std::tuple<TensorList, TensorList> backwardUpdatesMulti(
                                               dev.stream()),
               name);
     }
-    return {dmu_out, dnu_out};
+    return {std::move(dmu_out), std::move(dnu_out)};
 }
 
 std::tuple<TensorList, TensorList, TensorList> forwardAllMultiImpl(
     const TensorList &updates_in, const TensorList &mu, const TensorList &nu_in, double b1,
     double b2, double eps, double eps_root, const Counts &c) {
     const char *name = "adamForwardAllMulti";
-    TensorList new_mu = emptyLike(mu), new_nu = emptyLike(mu), new_updates = emptyLike(mu);
+    std::vector<TensorList> fresh = emptyLikeSets(mu, 3);
+    TensorList &new_mu = fresh[0], &new_nu = fresh[1], &new_updates = fresh[2];
     // gradients may arrive expanded or in another memory order: bring them to mu's
     const TensorList updates = asLayoutOfEach(updates_in, mu, name);
     const TensorList nu = asLayoutOfEach(nu_in, mu, name);
@@ -643,7 +653,7 @@ std::tuple<TensorList, TensorList, TensorList> forwardAllMultiImpl(
                                          l.ptr[5].data(), dev.stream()),
               name);
     }
-    return {new_mu, new_nu, new_updates};
+    return {std::move(new_mu), std::move(new_nu), std::move(new_updates)};
 }
 
 std::tuple<TensorList, TensorList, TensorList> forwardAllMulti(
@@ -661,7 +671,8 @@ std::tuple<TensorList, TensorList, TensorList> backwardAllMultiImpl(
     const TensorList &new_mu, const TensorList &updates_in, double b1, double b2,
     double eps_root, const Counts &c) {
     const char *name = "adamBackwardAllMulti";
-    TensorList dupdates = emptyLike(new_mu), dmu = emptyLike(new_mu), dnu = emptyLike(new_mu);
+    std::vector<TensorList> fresh = emptyLikeSets(new_mu, 3);
+    TensorList &dupdates = fresh[0], &dmu = fresh[1], &dnu = fresh[2];
     const TensorList du = asLayoutOfEach(dnew_updates_in, new_mu, name);
     const TensorList new_updates = asLayoutOfEach(new_updates_in, new_mu, name);
     const TensorList updates = asLayoutOfEach(updates_in, new_mu, name);
@@ -691,7 +702,7 @@ std::tuple<TensorList, TensorList, TensorList> backwardAllMultiImpl(
                   dev.stream()),
               name);
     }
-    return {dupdates, dmu, dnu};
+    return {std::move(dupdates), std::move(dmu), std::move(dnu)};
 }
 
 std::tuple<TensorList, TensorList, TensorList> backwardAllMulti(
@@ -834,6 +845,10 @@ class AdamStepNode : public torch::autograd::Function<AdamStepNode> {
                 dnu[i] = std::move(dn[j]);
             }
         }
+        // Gradients nobody asked for (torch.autograd.grad with `inputs`, leaves that do not
+        // require grad) are dropped here rather than checked and routed by the engine.
+        for (size_t i = 0; i < 3 * k; ++i)
+            if (result[i].defined() && !ctx->needs_input_grad(i)) result[i] = Tensor();
         return result;
     }
 

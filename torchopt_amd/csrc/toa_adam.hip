@@ -125,6 +125,10 @@ unsigned lds_reservation(bool multi, size_t num_tiles, bool staged = false) {
 // reference's availability probe passes one array three times) take the plain schedule.
 std::atomic<int> g_schedule{0};
 
+// Load order of the staged program of big single-tensor launches (ops that have several, see
+// LoadOrders): -1 = the library's choice, 0 .. 3 = that order wherever the op has it.
+std::atomic<int> g_load_order{-1};
+
 // Arrays of one tensor whose addresses differ by (nearly) a multiple of 16 MiB meet in the same
 // DRAM banks: measured on MI355X the in-place step falls from 6.6 to 5.5-6.1 TB/s when the
 // distance is within 1.5 MiB of such a multiple (GPT-2-medium's 4096 x 1024 float32 weights are
@@ -191,6 +195,213 @@ int make_step_ref(const void *bias_rows, uint64_t first_count, size_t rows, cons
     return 0;
 }
 
+// One address per op type: tells the remembered calls of different ops apart.
+template <class Op>
+struct OpTag {
+    static const char tag;
+};
+template <class Op>
+const char OpTag<Op>::tag = 0;
+
+// ---------------------------------------------------------------------------
+// Which load order a big single-tensor staged launch runs, chosen per call site by measurement.
+//
+// How three read and three write streams fall on the memory channels depends on where the three
+// arrays lie, and with it which of the four load orders of the staged program streams fastest:
+// on most placements the first (g, mu, nu) does, on some another gains 1-2 %.  The results are
+// the same bits in every order, so the library can try them on the caller's own launches: the
+// first kTuneRounds x 4 launches of a call site (one op on one set of arrays of one length) go
+// round the four orders, timed with events on the caller's stream; rounds alternate their
+// direction and the first two do not count, so a drift in the machine's rate (clocks settling
+// under a new load) cancels instead of favouring whatever ran last.  Once every sample has come
+// back -- events are polled, never waited for -- the order with the lowest mean time is kept for
+// the call site if it beats the default order by more than kTuneMargin, the default otherwise.
+// Nothing is tuned under stream capture, with an order or residency level forced, or with
+// tuning switched off; up to kTuneSites call sites are remembered, least recently used first out.
+// ---------------------------------------------------------------------------
+constexpr int kTuneOrders = 4;
+constexpr int kTuneRounds = 6, kTuneSkippedRounds = 2;
+constexpr double kTuneMargin = 0.0015;
+constexpr size_t kTuneSites = 64;
+constexpr size_t kTuneFromBytes = (size_t)64 << 20;  // per array: launches of 60 us and more
+
+std::atomic<int> g_tuning{-1};  // -1 = not yet initialised, 0 = off, 1 = on
+
+bool tuning_on() {
+    int t = g_tuning.load(std::memory_order_relaxed);
+    if (t < 0) {
+        const char *env = std::getenv("TOA_ADAM_TUNING");
+        t = (env != nullptr && env[0] == '0') ? 0 : 1;
+        g_tuning.store(t, std::memory_order_relaxed);
+    }
+    return t != 0;
+}
+
+struct TuneSite {
+    const void *tag = nullptr;  // the op
+    uintptr_t p[3] = {0, 0, 0};
+    size_t n = 0;
+    int device = 0;
+    uint64_t stamp = 0;
+    int decided = -1;  // the order kept, or -1 while the site is being explored
+    int launches = 0;  // exploring launches issued so far
+    double sum[kTuneOrders] = {0, 0, 0, 0};
+    int count[kTuneOrders] = {0, 0, 0, 0};
+    struct Sample {
+        int order;
+        bool counted;
+        hipEvent_t begin, end;
+    };
+    std::vector<Sample> pending;
+};
+std::mutex g_tune_mutex;
+std::vector<TuneSite> g_tune_sites;
+uint64_t g_tune_stamp = 0;
+
+void tune_drop_events(TuneSite &site) {
+    for (TuneSite::Sample &s : site.pending) {
+        (void)hipEventDestroy(s.begin);
+        (void)hipEventDestroy(s.end);
+    }
+    site.pending.clear();
+}
+
+// Collects the samples that have come back; decides once all have.  g_tune_mutex held.
+void tune_collect(TuneSite &site) {
+    size_t kept = 0;
+    for (size_t i = 0; i < site.pending.size(); ++i) {
+        TuneSite::Sample &s = site.pending[i];
+        const hipError_t ready = hipEventQuery(s.end);
+        if (ready == hipErrorNotReady) {
+            (void)hipGetLastError();
+            site.pending[kept++] = s;
+            continue;
+        }
+        float ms = 0.0f;
+        if (ready == hipSuccess && hipEventElapsedTime(&ms, s.begin, s.end) == hipSuccess) {
+            if (s.counted && ms > 0.0f) {
+                site.sum[s.order] += ms;
+                ++site.count[s.order];
+            }
+        } else {
+            (void)hipGetLastError();
+        }
+        (void)hipEventDestroy(s.begin);
+        (void)hipEventDestroy(s.end);
+    }
+    site.pending.resize(kept);
+    if (site.launches < kTuneRounds * kTuneOrders || !site.pending.empty()) return;
+    int best = 0;
+    bool complete = true;
+    double mean[kTuneOrders];
+    for (int o = 0; o < kTuneOrders; ++o) {
+        complete = complete && site.count[o] == kTuneRounds - kTuneSkippedRounds;
+        mean[o] = site.count[o] ? site.sum[o] / site.count[o] : 0.0;
+    }
+    if (complete)
+        for (int o = 1; o < kTuneOrders; ++o)
+            if (mean[o] < mean[best]) best = o;
+    site.decided = (complete && mean[best] < mean[0] * (1.0 - kTuneMargin)) ? best : 0;
+}
+
+TuneSite *tune_find(const void *tag, const uintptr_t (&p)[3], size_t n, int device, bool create) {
+    TuneSite *oldest = nullptr;
+    for (TuneSite &site : g_tune_sites) {
+        if (site.tag == tag && site.n == n && site.device == device && site.p[0] == p[0] &&
+            site.p[1] == p[1] && site.p[2] == p[2]) {
+            site.stamp = ++g_tune_stamp;
+            return &site;
+        }
+        if (oldest == nullptr || site.stamp < oldest->stamp) oldest = &site;
+    }
+    if (!create) return nullptr;
+    TuneSite *site = oldest;
+    if (g_tune_sites.size() < kTuneSites) {
+        g_tune_sites.emplace_back();
+        site = &g_tune_sites.back();
+    } else {
+        tune_drop_events(*site);
+        *site = TuneSite();
+    }
+    site->tag = tag;
+    for (int i = 0; i < 3; ++i) site->p[i] = p[i];
+    site->n = n;
+    site->device = device;
+    site->stamp = ++g_tune_stamp;
+    return site;
+}
+
+// The staged whole-tile kernel in one of the op's load orders.
+template <typename T, class Op>
+void launch_full_staged(int order, const Op &op, const TensorPtrs<T, Op> &tp, size_t whole,
+                        unsigned lds, void *stream) {
+    auto go = [&](auto ORDER) {
+        hipLaunchKernelGGL(
+            (full_tiles_kernel<T, Op, kUnroll, kNonTemporal, true, decltype(ORDER)::value>),
+            dim3((unsigned)whole), dim3(kBlock), lds, (hipStream_t)stream, op, tp);
+    };
+    if constexpr (LoadOrders<Op>::value == 4) {
+        switch (order) {
+            case 1: return go(std::integral_constant<int, 1>{});
+            case 2: return go(std::integral_constant<int, 2>{});
+            case 3: return go(std::integral_constant<int, 3>{});
+            default: break;
+        }
+    }
+    go(std::integral_constant<int, 0>{});
+}
+
+// A big staged launch of an op with several load orders, at the order its call site has settled
+// on, or -- while the site is being explored -- at the next order to try, timed.  False when the
+// launch is not the tuner's to make (the stream is capturing, no device).
+template <typename T, class Op>
+bool launch_tuned(const Op &op, const TensorPtrs<T, Op> &tp, size_t whole, unsigned lds,
+                  void *stream) {
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    int device = 0;
+    if (hipStreamIsCapturing((hipStream_t)stream, &capturing) != hipSuccess ||
+        capturing != hipStreamCaptureStatusNone || hipGetDevice(&device) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    const uintptr_t p[3] = {reinterpret_cast<uintptr_t>(tp.p[0]),
+                            reinterpret_cast<uintptr_t>(tp.p[1]),
+                            reinterpret_cast<uintptr_t>(tp.p[2])};
+    std::unique_lock<std::mutex> lock(g_tune_mutex);
+    TuneSite *site = tune_find(&OpTag<Op>::tag, p, whole, device, true);
+    if (site->decided < 0) tune_collect(*site);
+    if (site->decided >= 0 || site->launches >= kTuneRounds * kTuneOrders) {
+        // settled, or every exploring launch is out and its samples are still on their way
+        const int order = site->decided >= 0 ? site->decided : 0;
+        lock.unlock();
+        launch_full_staged<T, Op>(order, op, tp, whole, lds, stream);
+        return true;
+    }
+    const int round = site->launches / kTuneOrders, at = site->launches % kTuneOrders;
+    TuneSite::Sample sample;
+    sample.order = round % 2 == 0 ? at : kTuneOrders - 1 - at;
+    sample.counted = round >= kTuneSkippedRounds;
+    ++site->launches;
+    const bool timed = hipEventCreate(&sample.begin) == hipSuccess &&
+                       (hipEventCreate(&sample.end) == hipSuccess ||
+                        (hipEventDestroy(sample.begin), false));
+    if (!timed) (void)hipGetLastError();
+    // record, launch, record: one step under the mutex, so no other launch of the library lands
+    // between the two events on this stream
+    bool recorded = timed && hipEventRecord(sample.begin, (hipStream_t)stream) == hipSuccess;
+    launch_full_staged<T, Op>(sample.order, op, tp, whole, lds, stream);
+    const hipError_t launch_rc = hipPeekAtLastError();
+    recorded = recorded && hipEventRecord(sample.end, (hipStream_t)stream) == hipSuccess;
+    if (recorded && launch_rc == hipSuccess) {
+        site->pending.push_back(sample);
+    } else if (timed) {
+        if (launch_rc == hipSuccess) (void)hipGetLastError();  // an event's error, not the launch's
+        (void)hipEventDestroy(sample.begin);
+        (void)hipEventDestroy(sample.end);
+    }
+    return true;
+}
+
 template <typename T, class Op>
 int launch_single(const Op &op, T *const (&ptrs)[Op::NPTR], size_t n, void *stream) {
     if (n == 0) return 0;
@@ -213,11 +424,21 @@ int launch_single(const Op &op, T *const (&ptrs)[Op::NPTR], size_t n, void *stre
         if constexpr (IsStaged<Op>::value)
             staged = g_schedule.load(std::memory_order_relaxed) != 1 && arrays_disjoint(ptrs, n);
         if (staged) {
-            if constexpr (IsStaged<Op>::value)
-                hipLaunchKernelGGL((full_tiles_kernel<T, Op, kUnroll, kNonTemporal, true>),
-                                   dim3((unsigned)whole), dim3(kBlock),
-                                   lds_reservation<Op>(false, whole, true), (hipStream_t)stream, op,
-                                   tp);
+            if constexpr (IsStaged<Op>::value) {
+                const unsigned lds = lds_reservation<Op>(false, whole, true);
+                int order = g_load_order.load(std::memory_order_relaxed);
+                bool launched = false;
+                if constexpr (LoadOrders<Op>::value == kTuneOrders && Op::NPTR == 3) {
+                    if (order < 0 && tuning_on() && waves_override() == 0 &&
+                        g_schedule.load(std::memory_order_relaxed) == 0 &&
+                        whole * tile * sizeof(T) >= kTuneFromBytes)
+                        launched = launch_tuned<T, Op>(op, tp, whole, lds, stream);
+                }
+                if (!launched) {
+                    if (order < 0 || order >= LoadOrders<Op>::value) order = 0;
+                    launch_full_staged<T, Op>(order, op, tp, whole, lds, stream);
+                }
+            }
         } else {
             hipLaunchKernelGGL((full_tiles_kernel<T, Op, kUnroll, kNonTemporal>),
                                dim3((unsigned)whole), dim3(kBlock),
@@ -397,14 +618,6 @@ Plans::Slot *plan_cached(const std::vector<PlanSeed<NPTR>> &seeds, size_t tile, 
     g_plans.commit(slot, std::move(key));
     return slot;
 }
-
-// One address per op type: tells the remembered calls of different ops apart.
-template <class Op>
-struct OpTag {
-    static const char tag;
-};
-template <class Op>
-const char OpTag<Op>::tag = 0;
 
 // Memory for the plan of one call, brought by the caller instead of taken from the cache (the
 // entry point that must not allocate).  The plan is rewritten on every call.
@@ -824,6 +1037,42 @@ int toa_adam_set_schedule(int schedule) {
     const int prev = g_schedule.load(std::memory_order_relaxed);
     g_schedule.store(schedule == 1 || schedule == 2 ? schedule : 0, std::memory_order_relaxed);
     return prev;
+}
+
+int toa_adam_set_load_order(int order) {
+    const int prev = g_load_order.load(std::memory_order_relaxed);
+    g_load_order.store(order >= 0 && order <= 3 ? order : -1, std::memory_order_relaxed);
+    return prev;
+}
+
+int toa_adam_set_tuning(int on) {
+    const int prev = tuning_on() ? 1 : 0;
+    g_tuning.store(on ? 1 : 0, std::memory_order_relaxed);
+    return prev;
+}
+
+int toa_adam_tuned_load_order(int dtype, const void *updates, const void *mu, const void *nu,
+                              size_t n) {
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) {
+        (void)hipGetLastError();
+        return -1;
+    }
+    const uintptr_t p[3] = {reinterpret_cast<uintptr_t>(updates), reinterpret_cast<uintptr_t>(mu),
+                            reinterpret_cast<uintptr_t>(nu)};
+    auto look = [&](const void *tag, size_t tile) {
+        std::lock_guard<std::mutex> lock(g_tune_mutex);
+        TuneSite *site = tune_find(tag, p, n / tile, device, false);
+        if (site == nullptr) return -1;
+        if (site->decided < 0) tune_collect(*site);
+        return site->decided;
+    };
+    switch (dtype) {
+        case TOA_F32: return look(&OpTag<ForwardInplace<float>>::tag, Tile<float, kUnroll>::ELEMS);
+        case TOA_F64: return look(&OpTag<ForwardInplace<double>>::tag, Tile<double, kUnroll>::ELEMS);
+        case TOA_F16: return look(&OpTag<ForwardInplace<half_t>>::tag, Tile<half_t, kUnroll>::ELEMS);
+        default: return -1;
+    }
 }
 
 int toa_adam_set_plan_mode(int mode) {

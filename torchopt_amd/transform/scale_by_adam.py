@@ -80,6 +80,16 @@ def _inc_counts(counts: Sequence[torch.Tensor | None], grads: Sequence[Any]):
 
     Leaves that hold the very same count tensor (as the leaves of one `init` do, see there) are
     advanced together: one addition, one new tensor, shared again by all of them."""
+    first = counts[0] if counts else None
+    if (first is not None and all(c is first for c in counts)
+            and all(g is not None for g in grads)):
+        # the usual case, in one go: every leaf shares the count tensor `init` made and every
+        # leaf has a gradient
+        v = _host_value(first)
+        if v == INT64_MAX:
+            return list(counts), [v] * len(counts)
+        fresh = _remember(first + 1, v + 1)
+        return [fresh] * len(counts), [v + 1] * len(counts)
     values = [None] * len(counts)
     seen: dict[int, int] = {}      # id(count tensor) -> its host value
     bump: dict[int, torch.Tensor] = {}  # id -> tensor to advance
@@ -168,6 +178,9 @@ def _scale_by_accelerated_adam(
     if not 0.0 <= b2 < 1.0:
         raise ValueError(f'Invalid beta parameter at index 1: {b2}')
 
+    ops = {flag: MultiAdamOp(b1=b1, b2=b2, eps=eps, eps_root=eps_root, inplace=flag)
+           for flag in (False, True)}
+
     def flatten(tree):
         # a plain list / tuple of tensors and Nones is its own flattening; the general walk
         # (pure Python in torch.utils._pytree) costs ~3 us per leaf per tree
@@ -240,10 +253,14 @@ def _scale_by_accelerated_adam(
                 groups.setdefault((g.device, g.dtype), []).append(k)
             # a None gradient keeps mu and nu and yields a None update
 
-        op = MultiAdamOp(b1=b1, b2=b2, eps=eps, eps_root=eps_root, inplace=inplace)
+        op = ops[bool(inplace)]
         for ks in groups.values():
             values = [count_values[k] for k in ks]
             counts = values[0] if len(set(values)) == 1 else values
+            if len(ks) == n:  # the whole tree is one group: no re-indexing
+                new_mu, new_nu, new_g = (list(x) for x in op(mu_leaves, nu_leaves, g_leaves,
+                                                             counts))
+                break
             out_mu, out_nu, out_g = op([mu_leaves[k] for k in ks], [nu_leaves[k] for k in ks],
                                        [g_leaves[k] for k in ks], counts)
             for k, m, v, g in zip(ks, out_mu, out_nu, out_g):
