@@ -269,6 +269,123 @@ def time_backward_ops(torch, lib, cfg_id, code, dtype, tag, n, esize, eps_root, 
     return res
 
 
+def timed_region(torch, step, stream, warmup, steps):
+    """`warmup` untimed steps, then exactly `steps` steps between two device synchronisations:
+    (wall-clock ms per step, stream ms per step from events around the same steps)."""
+    for _ in range(warmup):
+        step()
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev0.record(stream)
+    for _ in range(steps):
+        step()
+    ev1.record(stream)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return (t1 - t0) * 1e3 / steps, ev0.elapsed_time(ev1) / steps
+
+
+def sysfs_gpu_state():
+    """What the driver says about the first GPU right now: the current shader and memory clock
+    levels (the starred lines of pp_dpm_sclk / pp_dpm_mclk) and the socket power.  Read while
+    work is queued on the GPU, these describe the state the timings were taken in.  Empty where
+    the files are not readable."""
+    import glob
+
+    out = {}
+    for dev in sorted(glob.glob('/sys/class/drm/card*/device')):
+        if not os.path.exists(os.path.join(dev, 'pp_dpm_sclk')):
+            continue
+        for key, name in (('sclk', 'pp_dpm_sclk'), ('mclk', 'pp_dpm_mclk')):
+            try:
+                with open(os.path.join(dev, name)) as f:
+                    for line in f:
+                        if line.rstrip().endswith('*'):
+                            out[f'{key}_MHz'] = int(''.join(c for c in line.split(':')[1]
+                                                            if c.isdigit()))
+            except (OSError, ValueError, IndexError):
+                pass
+        for path in glob.glob(os.path.join(dev, 'hwmon', '*', 'power1_input')):
+            try:
+                with open(path) as f:
+                    out['power_W'] = round(int(f.read()) / 1e6, 1)
+            except (OSError, ValueError):
+                pass
+        break
+    return out
+
+
+class ClockProbe:
+    """Shader-clock evidence beside a timing: the library's one-lane spin kernel
+    (toa_adam_clock_probe) reports shader-clock ticks and constant-rate (100 MHz) ticks for a
+    fixed spin; their ratio is the shader clock the wave ran at."""
+
+    SPINS = 20000  # ~60 us at 2.4 GHz: long against the counters' granularity, short in a stream
+
+    def __init__(self, torch, lib, slots=16):
+        self.torch, self.lib = torch, lib
+        self.buf = torch.zeros(slots, 3, dtype=torch.int64, device='cuda')
+        self.names = []
+
+    def sample(self, name, stream, spins=None):
+        k = len(self.names)
+        if k >= self.buf.shape[0]:
+            return
+        rc = self.lib.toa_adam_clock_probe(self.buf[k].data_ptr(), spins or self.SPINS,
+                                           stream.cuda_stream)
+        if rc:
+            raise RuntimeError(self.lib.toa_adam_error_string(rc).decode())
+        self.names.append((name, spins or self.SPINS))
+
+    def read(self):
+        host = self.buf.cpu().tolist()
+        out = {}
+        for (name, spins), (core, wall, _) in zip(self.names, host):
+            out[name] = {'spins': spins, 'shader_clock_ticks': core, 'constant_100MHz_ticks': wall,
+                         'shader_MHz': round(100.0 * core / wall, 1) if wall else None}
+        return out
+
+
+def in_situ(torch, step, stream, alg_bytes, iterations=50, busy_ms=5.0):
+    """The operator where an optimizer runs it: ONE launch per iteration, after `busy_ms` of
+    unrelated GPU work (a chain of matrix products on scratch tensors, as a backward pass would
+    leave the caches, clocks and queues), events around the operator's launch alone."""
+    a = torch.randn(4096, 4096, device='cuda')
+    b = torch.randn(4096, 4096, device='cuda') / 64.0  # keeps the chain's values bounded
+    for _ in range(3):
+        torch.matmul(a, b)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(4):
+        torch.matmul(a, b)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    one_ms = e0.elapsed_time(e1) / 4
+    chain = max(1, int(busy_ms / one_ms + 0.999))
+    pairs = []
+    for _ in range(iterations + 5):
+        x = a
+        for _ in range(chain):
+            x = torch.matmul(x, b)
+        p, q = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        p.record(stream)
+        step()
+        q.record(stream)
+        pairs.append((p, q))
+    torch.cuda.synchronize()
+    each = sorted(p.elapsed_time(q) for p, q in pairs[5:])
+    med = each[len(each) // 2]
+    return {'iterations': len(each), 'other_work_ms_per_iteration': round(chain * one_ms, 3),
+            'other_work': f'{chain} float32 matrix products of 4096 x 4096 on scratch tensors',
+            'operator_ms_median': round(med, 5), 'operator_ms_min': round(each[0], 5),
+            'operator_ms_max': round(each[-1], 5),
+            'GB/s_median': round(alg_bytes / med / 1e6, 1),
+            'frac_median': round(alg_bytes / med / 1e6 / HBM_PEAK_GBS, 4),
+            'frac_min_time': round(alg_bytes / each[0] / 1e6 / HBM_PEAK_GBS, 4)}
+
+
 def run_gpu(cfg_id, steps, warmup, operator_preheat=None, state='init'):
     import torch
 
@@ -554,17 +671,48 @@ def run_gpu(cfg_id, steps, warmup, operator_preheat=None, state='init'):
             extra['cold_cache_ms_per_launch'] = round(sorted(cold)[len(cold) // 2], 5)
 
     extra['preheat_launches_on_scratch_arrays'] = preheat(torch)
+    alg_bytes = bytes_per_elem * total
+    beside = {}  # measurements taken beside the headline, in this process
+
+    def leg(wall_ms, kern_ms, **more):
+        return {'ms_per_step_wall': round(wall_ms, 5), 'kernel_ms': round(kern_ms, 5),
+                'frac': round(alg_bytes / kern_ms / 1e6 / HBM_PEAK_GBS, 4),
+                'frac_by_wall_clock': round(alg_bytes / wall_ms / 1e6 / HBM_PEAK_GBS, 4), **more}
+
     # The first launches of the operator in a process are not its steady state, whatever ran
     # before: launches 1-2 run at the steady rate, launches 4-8 up to 4 % slower (float32 in place:
     # 0.948, 0.953, 0.960 ... 0.985 ms), and the time settles back over the next 15 (float32) to
     # 45 (16-bit types) launches -- the clocks boost and settle under this kernel's own mix of
-    # arithmetic and traffic.  Isolated steps on the initial and on a late state take the same
-    # time, so it is not the data.  The bandwidth-bound configurations therefore run the operator
-    # on SCRATCH state of the same shape before the warm-up steps (never on the benchmark's own:
-    # the in-place step would consume it); a fused step, which only reads its gradients, preheats
-    # on its own lists like any warm-up step would.  --operator-preheat 0 switches it off.
+    # arithmetic and traffic (the clock probes below show the shader clock on either side of the
+    # timed region).  Isolated steps on the initial and on a late state take the same time, so it
+    # is not the data.  The bandwidth-bound configurations therefore run the operator before the
+    # warm-up steps, and the line says how often and on what:
+    #   * float32 / float64 single tensors: on the timed arrays themselves, as the first steps of
+    #     a training run would (the library also settles its choice of load order for this call
+    #     site during its first 24 launches); what the same W + K steps read WITHOUT any of that
+    #     is measured first and reported as `cold_start`;
+    #   * the 16-bit single tensors and the lists: on scratch state of the same shape (the 16-bit
+    #     step's speed depends on its data, which a step fed its own output drifts away from);
+    #   * a fused step, which only reads its gradients, on its own lists.
+    # --operator-preheat 0 switches it off.
     op_launches = cfg.get('operator_preheat', 0) if operator_preheat is None else operator_preheat
-    if op_launches and cfg.get('fused_step'):
+    single_wide = ('shapes' not in cfg and not cfg.get('fresh_gradients')
+                   and not alg_small(total * esize))
+    if single_wide:
+        was = lib.toa_adam_set_tuning(0)
+        cold = timed_region(torch, step, stream, warmup, steps)
+        lib.toa_adam_set_tuning(was)
+        beside['cold_start'] = leg(*cold, note=(
+            f'{warmup} + {steps} steps straight after upload and the PyTorch-kernel preheat: no '
+            'launch of the operator before them, load-order tuning off (order 0 throughout)'))
+    if op_launches and single_wide:
+        for _ in range(op_launches):
+            step()
+        torch.cuda.synchronize()
+        extra['preheat_operator_launches_on_the_timed_arrays'] = op_launches
+        extra['load_order_kept_for_this_call_site'] = lib.toa_adam_tuned_load_order(
+            code, pu, pm, pv, total)
+    elif op_launches and cfg.get('fused_step'):
         for _ in range(op_launches):
             step()
         torch.cuda.synchronize()
@@ -591,37 +739,84 @@ def run_gpu(cfg_id, steps, warmup, operator_preheat=None, state='init'):
         torch.cuda.synchronize()
         del sg, sm, sv
         extra['preheat_operator_launches_on_scratch_state'] = op_launches
+
+    # ---- the headline: W warm-up steps, a clock probe, exactly K timed steps, a clock probe
+    bandwidth_bound = not alg_small(total * esize) and not cfg.get('differentiable')
+    probes = ClockProbe(torch, lib)
     for _ in range(warmup):
         step()
-    ev0 = torch.cuda.Event(enable_timing=True)
-    ev1 = torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    ev0.record(stream)
-    for _ in range(steps):
-        step()
-    ev1.record(stream)
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
+    if bandwidth_bound:
+        probes.sample('before_the_timed_region', stream)
+    wall_ms, kern_ms = timed_region(torch, step, stream, 0, steps)
+    if bandwidth_bound:
+        probes.sample('after_the_timed_region', stream)
+        torch.cuda.synchronize()
 
     # per-step spread, from a second short pass with one pair of events per step (outside the
-    # timed region; event overhead makes it meaningless for microsecond steps)
+    # timed region; event overhead makes it meaningless for microsecond steps).  While those steps
+    # are queued the driver's view of the GPU is read, and a long clock probe runs beside them on
+    # a second stream: the clock state INSIDE a region of the same work.
     spread = {}
-    if (t1 - t0) * 1e3 / steps > 0.05:
+    if wall_ms > 0.05:
+        reps = min(steps, 20)
+        side = None
+        if bandwidth_bound:
+            first = probes.read().get('before_the_timed_region')
+            if first and first['shader_clock_ticks'] and first['shader_MHz']:
+                ticks_per_spin = first['shader_clock_ticks'] / first['spins']
+                want_us = 0.6 * reps * kern_ms * 1e3
+                spins = int(min(want_us * first['shader_MHz'] / ticks_per_spin, 1 << 27))
+                side = torch.cuda.Stream()
+                probes.sample('beside_the_per_step_pass', side, spins=max(spins, 1000))
         pairs = []
-        for _ in range(min(steps, 20)):
+        for _ in range(reps):
             a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             a.record(stream)
             step()
             b.record(stream)
             pairs.append((a, b))
+        busy_state = sysfs_gpu_state() if bandwidth_bound else {}
         torch.cuda.synchronize()
         each = sorted(a.elapsed_time(b) for a, b in pairs)
-        spread = {'step_ms_min': round(each[0], 5), 'step_ms_median': round(each[len(each) // 2], 5)}
+        spread = {'step_ms_min': round(each[0], 5), 'step_ms_median': round(each[len(each) // 2], 5),
+                  'step_ms_max': round(each[-1], 5)}
+        if bandwidth_bound:
+            beside['clock'] = {
+                'probes': probes.read(),
+                'probe': 'toa_adam_clock_probe: one lane, a fixed spin of dependent integer '
+                         'multiply-adds; shader-clock ticks against ticks of the constant 100 MHz '
+                         'counter.  before / after: on the timed stream, either side of the timed '
+                         'region; beside: on a second stream while 20 further steps of the same '
+                         'work run',
+                'driver_while_steps_are_queued': busy_state}
 
-    wall_ms = (t1 - t0) * 1e3 / steps
-    kern_ms = ev0.elapsed_time(ev1) / steps  # stream time per launch (launches are back to back)
-    alg_bytes = bytes_per_elem * total
+    # ---- the same W + K steps with the moments where the ALLOCATOR puts them (what a caller
+    # gets whose state comes from zeros_like, as through the reference's own init)
+    if single_wide and state != 'plain':
+        p_mu, p_nu = h_mu.cuda(), h_nu.cuda()
+
+        def plain_step():
+            rc = lib.toa_adam_forward_inplace(code, pu, p_mu.data_ptr(), p_nu.data_ptr(), total,
+                                              B1, B2, eps, eps_root, count, sptr)
+            if rc:
+                raise RuntimeError(lib.toa_adam_error_string(rc).decode())
+        for _ in range(op_launches):
+            plain_step()
+        torch.cuda.synchronize()
+        beside['state_where_the_allocator_puts_it'] = leg(
+            *timed_region(torch, plain_step, stream, warmup, steps),
+            address_mod_16KiB={'updates': pu % 16384, 'mu': p_mu.data_ptr() % 16384,
+                               'nu': p_nu.data_ptr() % 16384},
+            load_order_kept=lib.toa_adam_tuned_load_order(code, pu, p_mu.data_ptr(),
+                                                          p_nu.data_ptr(), total),
+            note=f'{op_launches} launches on these arrays first, then {warmup} + {steps} steps')
+        del p_mu, p_nu
+
+    # ---- one launch per iteration between other kernels
+    if bandwidth_bound:
+        beside['one_launch_per_iteration_between_other_work'] = in_situ(torch, step, stream,
+                                                                        alg_bytes)
+
     achieved = alg_bytes / (kern_ms * 1e-3) / 1e9
     traffic, traffic_source = RECORDED_TRAFFIC.get(cfg_id, (None, None))
     return {
@@ -634,9 +829,11 @@ def run_gpu(cfg_id, steps, warmup, operator_preheat=None, state='init'):
             'traffic_source': (f'recorded in {traffic_source} (rocprofv3 --pmc), not measured in '
                                'this run' if traffic_source else None),
             'kernel_ms': round(kern_ms, 5), 'algorithmic_bytes_per_launch': alg_bytes,
-            'bytes_per_element': bytes_per_elem, **spread,
+            'bytes_per_element': bytes_per_elem,
+            'frac_by_wall_clock': round(alg_bytes / wall_ms / 1e6 / HBM_PEAK_GBS, 4), **spread,
         },
         'extra': extra,
+        'beside': beside,
         'device': torch.cuda.get_device_name(0),
     }
 
@@ -839,6 +1036,104 @@ def run_ceiling(array_bytes=1 << 30, reps=20):
             'three_arrays_read_and_written_back': family,
             'operator_forward_inplace_f32_on_the_same_placements': operator,
             'staged_shape_by_data_GB/s': by_data}
+
+
+def run_ceiling_backward(n=1 << 26, reps=20):
+    """The out-of-place backward ops in float64 on n elements (config 3's shape) beside
+    arithmetic-free passes of the same pattern -- 1 array read and 2 written (backward_mu), 2 and
+    2 (backward_nu), 3 and 2 (backward_updates), 6 and 3 (backward_all with both outside
+    gradients) -- over the same arrays, every residency level for the probe, library defaults for
+    the operator.  Three rounds, alternating, so that neither side always runs on a warmer
+    machine."""
+    import ctypes
+
+    import torch
+
+    from torchopt_amd import _lib
+
+    if not os.path.exists(PROBE_LIB):
+        build_probe()
+    probe = ctypes.CDLL(PROBE_LIB)
+    probe.bench_probe_stream.restype = ctypes.c_int
+    probe.bench_probe_stream.argtypes = [ctypes.c_int, ctypes.c_int,
+                                         ctypes.POINTER(ctypes.c_void_p), ctypes.c_size_t,
+                                         ctypes.c_uint, ctypes.c_void_p]
+    lib = _lib.load()
+    stream = torch.cuda.current_stream()
+    s = stream.cuda_stream
+    code, count, eps_root = _lib.TOA_F64, 3, 1e-8
+    array_bytes = 8 * n
+    g, mu, nu, d_mu, d_nu, d_u = (a.cuda() for a in host_state(3, 0, n, 'f64', extra=3))
+    new_mu, new_nu, new_u = (torch.empty_like(g) for _ in range(3))
+    rc = lib.toa_adam_forward_all(code, g.data_ptr(), mu.data_ptr(), nu.data_ptr(), n, B1, B2, EPS,
+                                  eps_root, count, new_mu.data_ptr(), new_nu.data_ptr(),
+                                  new_u.data_ptr(), s)
+    assert rc == 0
+    del mu, nu, new_nu
+    outs = [torch.empty_like(g) for _ in range(3)]
+    o = [t.data_ptr() for t in outs]
+    preheat(torch)
+
+    def timed(launch):
+        for _ in range(6):
+            launch()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record(stream)
+        for _ in range(reps):
+            launch()
+        ev1.record(stream)
+        torch.cuda.synchronize()
+        return ev0.elapsed_time(ev1) / reps
+
+    def must(rc):
+        if rc:
+            raise RuntimeError(f'launch failed: {rc}')
+
+    patterns = {
+        'backward_mu': (1, 2, [d_mu], outs[:2], lambda: must(lib.toa_adam_backward_mu(
+            code, d_mu.data_ptr(), n, B1, o[0], o[1], s))),
+        'backward_nu': (2, 2, [d_nu, g], outs[:2], lambda: must(lib.toa_adam_backward_nu(
+            code, d_nu.data_ptr(), g.data_ptr(), n, B2, o[0], o[1], s))),
+        'backward_updates': (3, 2, [d_u, new_u, new_mu], outs[:2],
+                             lambda: must(lib.toa_adam_backward_updates(
+                                 code, d_u.data_ptr(), new_u.data_ptr(), new_mu.data_ptr(), n, B1,
+                                 B2, eps_root, count, o[0], o[1], s))),
+        'backward_all': (6, 3, [d_u, new_u, new_mu, g, d_mu, d_nu], outs,
+                         lambda: must(lib.toa_adam_backward_all(
+                             code, d_u.data_ptr(), new_u.data_ptr(), new_mu.data_ptr(),
+                             g.data_ptr(), d_mu.data_ptr(), d_nu.data_ptr(), n, B1, B2, eps_root,
+                             count, o[0], o[1], o[2], s))),
+    }
+    result = {}
+    for name, (reads, writes, ins, outs_, op_launch) in patterns.items():
+        ptrs = (ctypes.c_void_p * (reads + writes))(*[t.data_ptr() for t in ins + list(outs_)])
+        alg = (reads + writes) * array_bytes
+        op_gbs, probe_by_level = [], {}
+        for rnd in range(3):
+            if rnd % 2 == 0:
+                op_gbs.append(alg / (timed(op_launch) * 1e-3) / 1e9)
+            for waves in RESIDENCY_LEVELS[:9]:
+                def launch():
+                    must(probe.bench_probe_stream(reads, writes, ptrs, array_bytes,
+                                                  lds_for_waves(waves), s))
+                probe_by_level.setdefault(waves, []).append(alg / (timed(launch) * 1e-3) / 1e9)
+            if rnd % 2 == 1:
+                op_gbs.append(alg / (timed(op_launch) * 1e-3) / 1e9)
+        levels = {w: sorted(v)[len(v) // 2] for w, v in probe_by_level.items()}
+        best_level = max(levels, key=levels.get)
+        op_med = sorted(op_gbs)[len(op_gbs) // 2]
+        result[name] = {
+            'pattern': f'{reads}R{writes}W', 'algorithmic_bytes': alg,
+            'operator_GB/s': round(op_med, 1), 'operator_frac_of_peak': round(op_med / HBM_PEAK_GBS, 4),
+            'probe_best_GB/s': round(levels[best_level], 1), 'probe_best_waves_per_cu': best_level,
+            'probe_frac_of_peak': round(levels[best_level] / HBM_PEAK_GBS, 4),
+            'operator_of_probe_best': round(op_med / levels[best_level], 4),
+            'probe_GB/s_by_waves_per_cu': {str(w): round(x, 1) for w, x in levels.items()},
+            'output_address_mod_16KiB': [p % 16384 for p in o[:writes]],
+        }
+    return {'metric': 'backward_ops_against_their_pattern_ceiling', 'unit': 'GB/s',
+            'peak': HBM_PEAK_GBS, 'dtype': 'f64', 'elements': n,
+            'device': torch.cuda.get_device_name(0), 'ops': result}
 
 
 def run_placements(reps=10, n=1 << 28, ladder=None):
@@ -1056,7 +1351,7 @@ def host_cores():
 _HOST_CORES = None
 
 
-CPU_SAMPLE_ELEMS = 1 << 26  # most elements the CPU leg works on (3 x 256 MiB of float32 state)
+CPU_SAMPLE_ELEMS = 1 << 28  # most elements the CPU leg works on: all of config 2 (3 x 1 GiB)
 
 
 def cpu_model():
@@ -1144,27 +1439,35 @@ class CpuOps:
             self._np(d), self._np(u), self._np(m), B1, B2, eps_root, count)]
 
 
-def ulp_report(pairs):
+def ulp_report(pairs, chunk=1 << 24):
     """(GPU tensor, CPU tensor) pairs -> elements checked, elements that differ, largest distance
-    in units in the last place (NaNs of any payload count as equal)."""
+    in units in the last place (NaNs of any payload count as equal).  Works through the arrays
+    in pieces, so whole configurations can be compared without holding 64-bit copies of them."""
     import numpy as np
     import torch
 
     checked = differing = worst = 0
     for got, want in pairs:
-        got = got.detach().cpu()
-        bits = {2: torch.int16, 4: torch.int32, 8: torch.int64}[got.element_size()]
-        nan = torch.isnan(got.float() if got.element_size() == 2 else got) & torch.isnan(
-            want.float() if want.element_size() == 2 else want)
-        a = got.contiguous().view(bits).numpy().astype(np.int64)
-        b = want.contiguous().view(bits).numpy().astype(np.int64)
-        lo = int(np.iinfo({2: np.int16, 4: np.int32, 8: np.int64}[got.element_size()]).min)
-        a, b = np.where(a < 0, lo - a, a), np.where(b < 0, lo - b, b)  # monotone integer line
-        d = np.abs(a - b)
-        d[nan.numpy()] = 0
-        checked += d.size
-        differing += int(np.count_nonzero(d))
-        worst = max(worst, int(d.max(initial=0)))
+        got = got.detach().cpu().contiguous().view(-1)
+        want = want.contiguous().view(-1)
+        size = got.element_size()
+        bits = {2: torch.int16, 4: torch.int32, 8: torch.int64}[size]
+        lo = int(np.iinfo({2: np.int16, 4: np.int32, 8: np.int64}[size]).min)
+        for at in range(0, got.numel(), chunk):
+            g, w = got[at:at + chunk], want[at:at + chunk]
+            if torch.equal(g.view(bits), w.view(bits)):  # the usual case: the same bits
+                checked += g.numel()
+                continue
+            nan = torch.isnan(g.float() if size == 2 else g) & torch.isnan(
+                w.float() if size == 2 else w)
+            a = g.view(bits).numpy().astype(np.int64)
+            b = w.view(bits).numpy().astype(np.int64)
+            a, b = np.where(a < 0, lo - a, a), np.where(b < 0, lo - b, b)  # monotone integer line
+            d = np.abs(a - b)
+            d[nan.numpy()] = 0
+            checked += d.size
+            differing += int(np.count_nonzero(d))
+            worst = max(worst, int(d.max(initial=0)))
     return {'elements_checked': checked, 'differing': differing, 'max_ulp': worst}
 
 
@@ -1210,14 +1513,17 @@ def run_cpu_baseline(cfg_id, budget_s=12.0):
             leaves.append([a.clone() for a in host_state(cfg_id, k, n, tag, extra=extra)])
             taken += n
         full = sum(sizes)
-        what = f'the first {len(leaves)} of {len(sizes)} tensors ({taken} of {full} elements)'
+        what = (f'the first {len(leaves)} of {len(sizes)} tensors ({taken} of {full} elements)'
+                if taken < full else
+                f'all: the whole configuration, {len(sizes)} tensors, {full} elements')
     else:
         full = cfg['n']
         n = min(full, CPU_SAMPLE_ELEMS)
         extra = 3 if cfg.get('backward') else 0
         leaves = [[a[:n].clone() for a in host_state(cfg_id, 0, full, tag, extra=extra)]]
         taken = n
-        what = (f'the first {n} of {full} elements' if n < full else f'all {full} elements')
+        what = (f'the first {n} of {full} elements' if n < full
+                else f'all: the whole configuration, {full} elements')
     dev = [[a.cuda() for a in leaf] for leaf in leaves]
     num = len(leaves)
 
@@ -1359,6 +1665,9 @@ def main(argv=None):
     ap.add_argument('--ceiling', action='store_true',
                     help='measure the streaming ceilings of this machine (probe kernels with '
                          'the operator\'s launch shape) instead of the operator')
+    ap.add_argument('--ceiling-backward', action='store_true',
+                    help='time the float64 backward ops on 2^26 elements beside arithmetic-free '
+                         'passes of the same read / write pattern')
     ap.add_argument('--placements', action='store_true',
                     help='time the operator over 210 placements of its three arrays inside one '
                          'allocation instead of the benchmark (the rate depends on the '
@@ -1381,6 +1690,9 @@ def main(argv=None):
 
     if args.ceiling:
         print(json.dumps(run_ceiling()), flush=True)
+        return 0
+    if args.ceiling_backward:
+        print(json.dumps(run_ceiling_backward()), flush=True)
         return 0
     if args.placements:
         print(json.dumps(run_placements()), flush=True)
@@ -1424,6 +1736,7 @@ def main(argv=None):
                    'eps': cfg.get('eps', EPS), 'eps_root': cfg['eps_root'], 'count': cfg['count'],
                    'device': gpu['device'], **gpu['extra']},
         'roofline': gpu['roofline'],
+        'beside_the_headline': gpu['beside'],
     }
     if not args.no_cpu_baseline:
         line['cpu_baseline'] = run_cpu_baseline(args.config)

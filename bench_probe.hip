@@ -12,7 +12,7 @@ namespace {
 
 typedef float f4 __attribute__((ext_vector_type(4)));
 constexpr int kWave = 64;
-constexpr int kMaxArrays = 8;
+constexpr int kMaxArrays = 9;
 
 #define PROBE_LD(p) __builtin_nontemporal_load(p)
 #define PROBE_ST(v, p) __builtin_nontemporal_store(v, p)
@@ -171,7 +171,8 @@ __global__ __launch_bounds__(kWave) void shape_gridstride(Three t, unsigned tile
 
 // One pass reading `reads` arrays and writing `writes` arrays of `bytes` bytes each (a multiple
 // of 16), `ptrs` = device pointers, reads first.  `lds_bytes` of dynamic LDS are reserved per
-// workgroup to cap residency.  Served shapes: (1,0) (3,0) (0,1) (0,3) (1,1) (2,1) (3,3) (4,3).
+// workgroup to cap residency.  Served shapes: (1,0) (3,0) (0,1) (0,3) (1,1) (2,1) (3,3) (4,3),
+// and the backward ops' (1,2) (2,2) (3,2) (6,3).
 extern "C" __attribute__((visibility("default"))) int bench_probe_stream(
     int reads, int writes, void *const *ptrs, size_t bytes, unsigned lds_bytes, void *stream) {
     if (ptrs == nullptr || bytes % 16 != 0) return -2;
@@ -183,6 +184,10 @@ extern "C" __attribute__((visibility("default"))) int bench_probe_stream(
         case 3: return launch<0, 3>(ptrs, bytes, lds_bytes, s);
         case 11: return launch<1, 1>(ptrs, bytes, lds_bytes, s);
         case 21: return launch<2, 1>(ptrs, bytes, lds_bytes, s);
+        case 12: return launch<1, 2>(ptrs, bytes, lds_bytes, s);
+        case 22: return launch<2, 2>(ptrs, bytes, lds_bytes, s);
+        case 32: return launch<3, 2>(ptrs, bytes, lds_bytes, s);
+        case 63: return launch<6, 3>(ptrs, bytes, lds_bytes, s);
         case 33: return launch<3, 3>(ptrs, bytes, lds_bytes, s);
         case 43: return launch<4, 3>(ptrs, bytes, lds_bytes, s);
         default: return -1;

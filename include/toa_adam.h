@@ -108,9 +108,9 @@ TOA_API int toa_adam_set_schedule(int schedule);
  *   toa_adam_set_tuning         0 = every site runs order 0; 1 (default; the environment variable
  *                               TOA_ADAM_TUNING=0 starts with 0) = as above.  Returns the previous
  *                               setting.
- *   toa_adam_tuned_load_order   the order kept for that call site of toa_adam_forward_inplace
- *                               (or its _devcount form uses a site of its own), or -1 while it is
- *                               unknown or still being explored. */
+ *   toa_adam_tuned_load_order   the order kept for that call site of toa_adam_forward_inplace, or
+ *                               -1 while it is unknown or still being explored (the _devcount
+ *                               form of the step keeps sites of its own). */
 TOA_API int toa_adam_set_load_order(int order);
 TOA_API int toa_adam_set_tuning(int on);
 TOA_API int toa_adam_tuned_load_order(int dtype, const void *updates, const void *mu,
@@ -159,6 +159,14 @@ TOA_API unsigned toa_adam_set_max_grid(unsigned workgroups);
  * /root/reference/torchopt/transform/scale_by_adam.py:401-414). */
 TOA_API size_t toa_adam_state_slack(void);
 TOA_API size_t toa_adam_state_shift(const void *allocation, int moment);
+
+/* Measurement aid: enqueues a one-lane kernel on `stream` that runs `spins` (at most 2^28)
+ * dependent integer multiply-adds and writes three 64-bit words to device memory at `out`: the
+ * shader-clock ticks the spin took, the ticks of the device's constant-rate counter (100 MHz)
+ * over the same span, and the spin's result.  ticks / constant ticks * 100 MHz is the shader
+ * clock the wave ran at -- what a benchmark records beside its timings to show the clock state
+ * they were taken in.  No counterpart in the reference. */
+TOA_API int toa_adam_clock_probe(uint64_t *out, uint32_t spins, void *stream);
 
 /* Human-readable name of a return code from any function below. */
 TOA_API const char *toa_adam_error_string(int code);

@@ -36,7 +36,7 @@ def test_header_declares_the_expected_surface():
     want = {f'toa_adam_{s}' for s in singles} | {f'toa_adam_{s}_multi' for s in singles}
     want |= {'toa_adam_abi_version', 'toa_adam_error_string', 'toa_adam_set_waves_per_cu',
              'toa_adam_fused_step', 'toa_adam_fused_step_multi', 'toa_adam_set_max_grid',
-             'toa_adam_set_schedule', 'toa_adam_set_load_order', 'toa_adam_set_tuning', 'toa_adam_tuned_load_order',
+             'toa_adam_set_schedule', 'toa_adam_clock_probe', 'toa_adam_set_load_order', 'toa_adam_set_tuning', 'toa_adam_tuned_load_order',
              'toa_adam_set_plan_mode', 'toa_adam_release_plans',
              'toa_adam_state_slack', 'toa_adam_state_shift',
              'toa_adam_forward_inplace_multi_noalloc', 'toa_adam_bias_rows',

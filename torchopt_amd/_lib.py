@@ -37,6 +37,7 @@ SIGNATURES = {
     'toa_adam_set_load_order': [_i],
     'toa_adam_set_tuning': [_i],
     'toa_adam_tuned_load_order': [_i, _vp, _vp, _vp, _sz],
+    'toa_adam_clock_probe': [_vp, ctypes.c_uint32, _vp],
     'toa_adam_set_plan_mode': [_i],
     'toa_adam_release_plans': [],
     'toa_adam_state_slack': [],

@@ -1636,4 +1636,24 @@ __global__ __launch_bounds__(64) void count_advance_kernel(int64_t *count) {
     }
 }
 
+// Clock evidence for a measurement: one lane runs `spins` dependent integer multiply-adds and
+// reports how many shader-clock ticks (s_memtime) and how many ticks of the constant-rate
+// counter (s_memrealtime, 100 MHz) that took.  The ratio is the shader clock the wave ran at;
+// the constant-rate ticks for a fixed spin say the same without trusting either counter's name.
+__global__ __launch_bounds__(64) void clock_probe_kernel(uint64_t *out, uint32_t spins) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    const uint64_t wall0 = wall_clock64();
+    const uint64_t core0 = clock64();
+    uint32_t x = spins | 1u;
+    for (uint32_t i = 0; i < spins; ++i) {
+        x = x * 1664525u + 1013904223u;
+        asm volatile("" : "+v"(x));  // keeps the chain: one multiply-add after the other
+    }
+    const uint64_t core1 = clock64();
+    const uint64_t wall1 = wall_clock64();
+    out[0] = core1 - core0;
+    out[1] = wall1 - wall0;
+    out[2] = x;
+}
+
 }  // namespace toa

@@ -1075,6 +1075,13 @@ int toa_adam_tuned_load_order(int dtype, const void *updates, const void *mu, co
     }
 }
 
+int toa_adam_clock_probe(uint64_t *out, uint32_t spins, void *stream) {
+    if (out == nullptr) return TOA_ENULL;
+    if (spins > (1u << 28)) return TOA_ESIZE;  // bounded: a few hundred milliseconds at most
+    hipLaunchKernelGGL(clock_probe_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, out, spins);
+    return (int)hipGetLastError();
+}
+
 int toa_adam_set_plan_mode(int mode) {
     const int prev = g_plan_mode.load(std::memory_order_relaxed);
     g_plan_mode.store(mode == 1 || mode == 2 ? mode : 0, std::memory_order_relaxed);
