@@ -23,14 +23,6 @@ Beside the headline `value` (elements per second) the line carries
                 host's cores on a bounded sample of the same workload, and with it the parity of
                 the GPU's result with the CPU's on that sample (differing elements, max ulp).
 
-`--ceiling` measures, instead of the operator, what this machine's HBM delivers to streaming
-kernels of the same launch shape that do next to no arithmetic (bench_probe.hip: R arrays read,
-W arrays written, at every residency level), and prints those ceilings as one JSON line: the
-context for `roofline.frac`.  `--placements`, `--state-phases` and `--state-distances` time the
-operator over placements of its three arrays (inside one allocation; the moments' address phases
-on separate allocations; the distance between the moments in one block): the measurements behind
-where the package allocates state.
-
 Everything on one GPU: `--gpus N` with N > 1 is refused.
 """
 
@@ -838,494 +830,6 @@ def run_gpu(cfg_id, steps, warmup, operator_preheat=None, state='init'):
     }
 
 
-# ----------------------------------------------------------------------------- HBM ceilings
-
-PROBE_SRC = os.path.join(REPO, 'bench_probe.hip')
-PROBE_LIB = os.path.join(REPO, 'bench_probe.so')
-RESIDENCY_LEVELS = (32, 25, 21, 18, 16, 14, 12, 11, 10, 9, 8)  # floor(128 / LDS granules)
-
-
-def build_probe():
-    """hipcc -> bench_probe.so (cross-compiles without a GPU)."""
-    import subprocess
-
-    subprocess.run(['hipcc', '-O3', '-std=c++17', '--offload-arch=gfx950', '-fPIC', '-shared',
-                    '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
-                    '-fvisibility=hidden', '-o', PROBE_LIB, PROBE_SRC], check=True,
-                   stderr=subprocess.DEVNULL)
-    return PROBE_LIB
-
-
-def lds_for_waves(waves):
-    """Dynamic LDS per single-wave workgroup that caps a gfx950 CU (128 granules of 1280 B) at
-    `waves` resident workgroups."""
-    return 0 if waves >= 32 else (128 // (waves + 1) + 1) * 1280
-
-
-# Launch shapes of bench_probe_inplace3 (three arrays read and written back) and the residency
-# levels each is swept over: workgroups per compute unit through the LDS reservation, except for
-# the persistent grid, whose level is its grid size per compute unit.
-INPLACE3_SHAPES = (
-    ('one wave per workgroup, one 1 KiB tile per wave (the plain schedule)', 0,
-     (32, 25, 21, 18, 16, 14, 12, 11, 10, 9, 8)),
-    ('same, one memory operation of a wave at a time (the staged schedule)', 1,
-     (32, 25, 21, 18, 16, 14, 12)),
-    ('same, a wait after every load and store', 2, (32, 25, 21, 18, 16)),
-    ('256-thread workgroups, one tile per wave', 3, (8, 6, 5, 4, 3, 2)),
-    ('512-thread workgroups, one tile per wave', 4, (4, 3, 2)),
-    ('two tiles per wave, all loads before the first store', 5, (16, 12, 10, 8, 7, 6, 5, 4)),
-    ('four tiles per wave, all loads before the first store', 6, (8, 6, 5, 4, 3, 2)),
-    ('persistent grid striding over the tiles, next tile loaded before the current one is '
-     'stored', 7, (16, 12, 10, 8, 6, 4)),
-    ('staged, two adjacent tiles per wave, one after the other', 8, (32, 25, 21, 18, 16, 14)),
-    ('staged, four adjacent tiles per wave, one after the other', 9, (32, 25, 21, 18, 16, 14)),
-)
-
-
-def run_ceiling(array_bytes=1 << 30, reps=20):
-    import ctypes
-
-    import torch
-
-    if not os.path.exists(PROBE_LIB):
-        build_probe()
-    probe = ctypes.CDLL(PROBE_LIB)
-    probe.bench_probe_stream.restype = ctypes.c_int
-    probe.bench_probe_stream.argtypes = [ctypes.c_int, ctypes.c_int,
-                                         ctypes.POINTER(ctypes.c_void_p), ctypes.c_size_t,
-                                         ctypes.c_uint, ctypes.c_void_p]
-    probe.bench_probe_inplace3.restype = ctypes.c_int
-    probe.bench_probe_inplace3.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
-                                           ctypes.c_void_p, ctypes.c_size_t, ctypes.c_size_t,
-                                           ctypes.c_uint, ctypes.c_int, ctypes.c_void_p]
-    stream = torch.cuda.current_stream()
-    # normally distributed like the operator's state: throughput depends on the bits moved
-    arrays = [torch.randn(array_bytes // 4, device='cuda') for _ in range(7)]
-    torch.cuda.synchronize()
-
-    def timed(launch):
-        for _ in range(4):
-            launch()
-        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        ev0.record(stream)
-        for _ in range(reps):
-            launch()
-        ev1.record(stream)
-        torch.cuda.synchronize()
-        return ev0.elapsed_time(ev1) / reps
-
-    out = {}
-    shapes = [(r, w, False) for r, w in ((1, 0), (3, 0), (0, 1), (0, 3), (1, 1), (2, 1), (3, 3),
-                                         (4, 3))]
-    shapes += [(3, 3, True), (4, 3, True)]  # written back over the arrays just read, as forward_
-    for reads, writes, in_place in shapes:
-        order = list(range(reads)) + (list(range(reads - writes, reads)) if in_place
-                                      else list(range(reads, reads + writes)))
-        ptrs = (ctypes.c_void_p * (reads + writes))(*[arrays[k].data_ptr() for k in order])
-        best = (0.0, None)
-        for waves in RESIDENCY_LEVELS:
-            def launch():
-                rc = probe.bench_probe_stream(reads, writes, ptrs, array_bytes,
-                                              lds_for_waves(waves), stream.cuda_stream)
-                if rc:
-                    raise RuntimeError(f'bench_probe_stream({reads}, {writes}) returned {rc}')
-            gbs = (reads + writes) * array_bytes / (timed(launch) * 1e-3) / 1e9
-            if gbs > best[0]:
-                best = (gbs, waves)
-        out[f'{reads}R{writes}W' + (' in place' if in_place else '')] = {'GB/s': round(best[0], 1), 'frac_of_peak': round(
-            best[0] / HBM_PEAK_GBS, 4), 'waves_per_cu': best[1]}
-
-    # The in-place step's pattern under a family of launch shapes, on two placements of the same
-    # three arrays: separate allocations as the allocator hands them out (what the operator
-    # gets), and one arena in which they interleave in 64 KiB pieces (the most favourable
-    # placement found: every wave's three tiles then sit in different DRAM banks).
-    del arrays[3:]
-    arena = torch.randn(3 * (array_bytes // 4), device='cuda')
-    a0, a1, a2 = (t.data_ptr() for t in arrays)
-    layouts = [('three separate arrays', (a0, a1, a2), 0),
-               ('one arena, arrays interleaved in 64 KiB pieces', (arena.data_ptr(), None, None),
-                64 << 10)]
-    # ... and on placements inside one allocation that differ only in the distances between the
-    # arrays: the rate is a repeatable function of those distances (how the three streams fall on
-    # DRAM channels and banks), so a ceiling holds for a placement, like the operator's own rate
-    n_elems = array_bytes // 4
-    wide = torch.randn(3 * n_elems + (8 << 20) // 4, device='cuda')
-    phases = ((0, 0), (0, 8), (8, 8), (4, 4), (2048, 4096))
-    for a_kib, b_kib in phases:
-        base = wide.data_ptr()
-        layouts.append((f'one allocation, mu at 1 GiB + {a_kib} KiB, nu at 2 GiB + {b_kib} KiB',
-                        (base, base + array_bytes + (a_kib << 10),
-                         base + 2 * array_bytes + (b_kib << 10)), 0))
-    # ... and the placement the package's own init produces for a one-leaf tree: the gradient in
-    # an allocation of its own, both moments in one block, 8 KiB off the 16 KiB phase, an even
-    # number of MiB (8 where cheap) past a multiple of 16 MiB apart
-    from torchopt_amd.placement import state_zeros_like_tree
-    own_grad = torch.randn(n_elems, device='cuda')
-    (own_mu,), (own_nu,) = state_zeros_like_tree([own_grad])
-    own_mu.normal_()
-    own_nu.normal_()
-    init_layout = "a gradient allocation and the moments in one block where the package's init puts them"
-    layouts.append((init_layout, (own_grad.data_ptr(), own_mu.data_ptr(), own_nu.data_ptr()), 0))
-    family = {}
-    for layout, ptrs3, piece in layouts:
-        rows, top = {}, (0.0, None)
-        for name, code, levels in INPLACE3_SHAPES:
-            best = (0.0, None)
-            for level in levels:
-                lds = 0 if code == 7 else lds_for_waves(level)
-
-                def launch():
-                    rc = probe.bench_probe_inplace3(code, ptrs3[0], ptrs3[1], ptrs3[2], array_bytes,
-                                                    piece, lds, level, stream.cuda_stream)
-                    if rc:
-                        raise RuntimeError(f'bench_probe_inplace3(shape {code}) returned {rc}')
-                gbs = 6 * array_bytes / (timed(launch) * 1e-3) / 1e9
-                if gbs > best[0]:
-                    best = (gbs, level)
-            rows[name] = {'GB/s': round(best[0], 1), 'frac_of_peak': round(best[0] / HBM_PEAK_GBS, 4),
-                          'workgroups_per_cu': best[1]}
-            if best[0] > top[0]:
-                top = (best[0], name)
-        family[layout] = {'shapes': rows, 'best_shape': top[1], 'best_GB/s': round(top[0], 1),
-                          'best_frac_of_peak': round(top[0] / HBM_PEAK_GBS, 4)}
-    # The operator itself (float32 forward_ in place, library defaults) on the same placements
-    from torchopt_amd import _lib
-    lib = _lib.load()
-    operator = {}
-    for layout, ptrs3, piece in layouts:
-        if piece:
-            continue
-        views = [torch.empty(0)] * 3
-        if layout == 'three separate arrays':
-            views = arrays[:3]
-        elif layout == init_layout:
-            views = [own_grad, own_mu, own_nu]
-        else:
-            views = [wide[(p - wide.data_ptr()) // 4:(p - wide.data_ptr()) // 4 + n_elems]
-                     for p in ptrs3]
-
-        def launch():
-            rc = lib.toa_adam_forward_inplace(_lib.TOA_F32, ptrs3[0], ptrs3[1], ptrs3[2], n_elems,
-                                              B1, B2, EPS, 0.0, 1000, stream.cuda_stream)
-            if rc:
-                raise RuntimeError(lib.toa_adam_error_string(rc).decode())
-        views[0].normal_()
-        views[1].normal_(0, 0.1)
-        views[2].normal_(0, 0.01).abs_()
-        gbs = 6 * array_bytes / (timed(launch) * 1e-3) / 1e9
-        operator[layout] = {'GB/s': round(gbs, 1), 'frac_of_peak': round(gbs / HBM_PEAK_GBS, 4),
-                            'of_the_probe_best_here': round(gbs / family[layout]['best_GB/s'], 4)}
-    # The same pass (staged shape, three separate arrays) over other data: the rate depends on the
-    # bits that cross the memory interface, so a ceiling holds for the data it was taken on.
-    by_data = {}
-    for label, fill in (('zeros', lambda t: t.zero_()),
-                        ('uniform in [1, 2): one sign, one exponent', lambda t: t.uniform_(1.0, 2.0)),
-                        ('normal (0, 1), as the operator\'s gradients', lambda t: t.normal_())):
-        for t in arrays:
-            fill(t)
-
-        def launch():
-            rc = probe.bench_probe_inplace3(1, a0, a1, a2, array_bytes, 0, lds_for_waves(18), 0,
-                                            stream.cuda_stream)
-            if rc:
-                raise RuntimeError(f'bench_probe_inplace3 returned {rc}')
-        by_data[label] = round(6 * array_bytes / (timed(launch) * 1e-3) / 1e9, 1)
-    return {'metric': 'hbm_streaming_ceiling', 'unit': 'GB/s', 'peak': HBM_PEAK_GBS,
-            'array_bytes': array_bytes, 'launches_timed': reps,
-            'device': torch.cuda.get_device_name(0), 'ceilings': out,
-            'three_arrays_read_and_written_back': family,
-            'operator_forward_inplace_f32_on_the_same_placements': operator,
-            'staged_shape_by_data_GB/s': by_data}
-
-
-def run_ceiling_backward(n=1 << 26, reps=20):
-    """The out-of-place backward ops in float64 on n elements (config 3's shape) beside
-    arithmetic-free passes of the same pattern -- 1 array read and 2 written (backward_mu), 2 and
-    2 (backward_nu), 3 and 2 (backward_updates), 6 and 3 (backward_all with both outside
-    gradients) -- over the same arrays, every residency level for the probe, library defaults for
-    the operator.  Three rounds, alternating, so that neither side always runs on a warmer
-    machine."""
-    import ctypes
-
-    import torch
-
-    from torchopt_amd import _lib
-
-    if not os.path.exists(PROBE_LIB):
-        build_probe()
-    probe = ctypes.CDLL(PROBE_LIB)
-    probe.bench_probe_stream.restype = ctypes.c_int
-    probe.bench_probe_stream.argtypes = [ctypes.c_int, ctypes.c_int,
-                                         ctypes.POINTER(ctypes.c_void_p), ctypes.c_size_t,
-                                         ctypes.c_uint, ctypes.c_void_p]
-    lib = _lib.load()
-    stream = torch.cuda.current_stream()
-    s = stream.cuda_stream
-    code, count, eps_root = _lib.TOA_F64, 3, 1e-8
-    array_bytes = 8 * n
-    g, mu, nu, d_mu, d_nu, d_u = (a.cuda() for a in host_state(3, 0, n, 'f64', extra=3))
-    new_mu, new_nu, new_u = (torch.empty_like(g) for _ in range(3))
-    rc = lib.toa_adam_forward_all(code, g.data_ptr(), mu.data_ptr(), nu.data_ptr(), n, B1, B2, EPS,
-                                  eps_root, count, new_mu.data_ptr(), new_nu.data_ptr(),
-                                  new_u.data_ptr(), s)
-    assert rc == 0
-    del mu, nu, new_nu
-    outs = [torch.empty_like(g) for _ in range(3)]
-    o = [t.data_ptr() for t in outs]
-    preheat(torch)
-
-    def timed(launch):
-        for _ in range(6):
-            launch()
-        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        ev0.record(stream)
-        for _ in range(reps):
-            launch()
-        ev1.record(stream)
-        torch.cuda.synchronize()
-        return ev0.elapsed_time(ev1) / reps
-
-    def must(rc):
-        if rc:
-            raise RuntimeError(f'launch failed: {rc}')
-
-    patterns = {
-        'backward_mu': (1, 2, [d_mu], outs[:2], lambda: must(lib.toa_adam_backward_mu(
-            code, d_mu.data_ptr(), n, B1, o[0], o[1], s))),
-        'backward_nu': (2, 2, [d_nu, g], outs[:2], lambda: must(lib.toa_adam_backward_nu(
-            code, d_nu.data_ptr(), g.data_ptr(), n, B2, o[0], o[1], s))),
-        'backward_updates': (3, 2, [d_u, new_u, new_mu], outs[:2],
-                             lambda: must(lib.toa_adam_backward_updates(
-                                 code, d_u.data_ptr(), new_u.data_ptr(), new_mu.data_ptr(), n, B1,
-                                 B2, eps_root, count, o[0], o[1], s))),
-        'backward_all': (6, 3, [d_u, new_u, new_mu, g, d_mu, d_nu], outs,
-                         lambda: must(lib.toa_adam_backward_all(
-                             code, d_u.data_ptr(), new_u.data_ptr(), new_mu.data_ptr(),
-                             g.data_ptr(), d_mu.data_ptr(), d_nu.data_ptr(), n, B1, B2, eps_root,
-                             count, o[0], o[1], o[2], s))),
-    }
-    result = {}
-    for name, (reads, writes, ins, outs_, op_launch) in patterns.items():
-        ptrs = (ctypes.c_void_p * (reads + writes))(*[t.data_ptr() for t in ins + list(outs_)])
-        alg = (reads + writes) * array_bytes
-        op_gbs, probe_by_level = [], {}
-        for rnd in range(3):
-            if rnd % 2 == 0:
-                op_gbs.append(alg / (timed(op_launch) * 1e-3) / 1e9)
-            for waves in RESIDENCY_LEVELS[:9]:
-                def launch():
-                    must(probe.bench_probe_stream(reads, writes, ptrs, array_bytes,
-                                                  lds_for_waves(waves), s))
-                probe_by_level.setdefault(waves, []).append(alg / (timed(launch) * 1e-3) / 1e9)
-            if rnd % 2 == 1:
-                op_gbs.append(alg / (timed(op_launch) * 1e-3) / 1e9)
-        levels = {w: sorted(v)[len(v) // 2] for w, v in probe_by_level.items()}
-        best_level = max(levels, key=levels.get)
-        op_med = sorted(op_gbs)[len(op_gbs) // 2]
-        result[name] = {
-            'pattern': f'{reads}R{writes}W', 'algorithmic_bytes': alg,
-            'operator_GB/s': round(op_med, 1), 'operator_frac_of_peak': round(op_med / HBM_PEAK_GBS, 4),
-            'probe_best_GB/s': round(levels[best_level], 1), 'probe_best_waves_per_cu': best_level,
-            'probe_frac_of_peak': round(levels[best_level] / HBM_PEAK_GBS, 4),
-            'operator_of_probe_best': round(op_med / levels[best_level], 4),
-            'probe_GB/s_by_waves_per_cu': {str(w): round(x, 1) for w, x in levels.items()},
-            'output_address_mod_16KiB': [p % 16384 for p in o[:writes]],
-        }
-    return {'metric': 'backward_ops_against_their_pattern_ceiling', 'unit': 'GB/s',
-            'peak': HBM_PEAK_GBS, 'dtype': 'f64', 'elements': n,
-            'device': torch.cuda.get_device_name(0), 'ops': result}
-
-
-def run_placements(reps=10, n=1 << 28, ladder=None):
-    """The operator (float32 forward_ in place, 2^28 elements, library defaults) over placements of
-    its three arrays inside ONE allocation: mu at 1 GiB + a, nu at 2 GiB + b for a <= b (so the
-    arrays stay disjoint) from a ladder of distances between 0 and 4 MiB.  The rate depends on how
-    the three read and three write streams fall on DRAM channels and banks; this is the table of
-    that dependence."""
-    import torch
-
-    from torchopt_amd import _lib
-
-    lib = _lib.load()
-    stream = torch.cuda.current_stream()
-    if ladder is None:  # KiB
-        ladder = (0, 1, 2, 3, 4, 5, 6, 7, 8, 12, 16, 24, 32, 64, 128, 256, 512, 1024, 2048, 4096)
-    arena = torch.empty(3 * n + 2 * max(ladder) * 256, device='cuda')
-    preheat(torch)
-    grid, cells = {}, []
-    for a_kib in ladder:
-        row = {}
-        for b_kib in ladder:
-            if b_kib < a_kib:
-                continue
-            u = arena[0:n]
-            mu = arena[n + a_kib * 256:2 * n + a_kib * 256]
-            nu = arena[2 * n + b_kib * 256:3 * n + b_kib * 256]
-            u.normal_()
-            mu.normal_(0, 0.1)
-            nu.normal_(0, 0.01).abs_()
-            ptrs = (u.data_ptr(), mu.data_ptr(), nu.data_ptr())
-
-            def launch():
-                rc = lib.toa_adam_forward_inplace(_lib.TOA_F32, *ptrs, n, B1, B2, EPS, 0.0, 1000,
-                                                  stream.cuda_stream)
-                if rc:
-                    raise RuntimeError(lib.toa_adam_error_string(rc).decode())
-            for _ in range(2):
-                launch()
-            ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            ev0.record(stream)
-            for _ in range(reps):
-                launch()
-            ev1.record(stream)
-            torch.cuda.synchronize()
-            gbs = 24 * n / (ev0.elapsed_time(ev1) / reps) / 1e6
-            row[f'nu +{b_kib} KiB'] = round(gbs)
-            cells.append(gbs)
-        grid[f'mu +{a_kib} KiB'] = row
-    cells.sort()
-    return {'metric': 'forward_inplace_f32_by_placement', 'unit': 'GB/s', 'peak': HBM_PEAK_GBS,
-            'elements': n, 'placements': len(cells), 'launches_timed': reps,
-            'min': round(cells[0], 1), 'median': round(cells[len(cells) // 2], 1),
-            'max': round(cells[-1], 1),
-            'min_frac': round(cells[0] / HBM_PEAK_GBS, 4),
-            'median_frac': round(cells[len(cells) // 2] / HBM_PEAK_GBS, 4),
-            'max_frac': round(cells[-1] / HBM_PEAK_GBS, 4),
-            'device': torch.cuda.get_device_name(0), 'GB/s_by_placement': grid}
-
-
-def run_state_phases(reps=12, n=1 << 28, step_kib=2, span_kib=32):
-    """The operator (float32 forward_ in place, 2^28 elements, library defaults) on three SEPARATE
-    PyTorch allocations -- what a training loop hands it -- with mu and nu shifted inside their own
-    allocations by every pair of phases from 0 to `span_kib` in steps of `step_kib`; the gradient
-    stays where the allocator put it (a 2 MiB boundary).  After every row the unshifted placement
-    is timed again, so a drift of the machine over the run shows.  This is the measurement behind
-    the phase at which the package allocates state (toa_adam_state_shift)."""
-    import torch
-
-    from torchopt_amd import _lib
-
-    lib = _lib.load()
-    stream = torch.cuda.current_stream()
-    pad = span_kib * 256
-    u = torch.empty(n, device='cuda')
-    mu_block = torch.empty(n + pad, device='cuda')
-    nu_block = torch.empty(n + pad, device='cuda')
-    preheat(torch)
-
-    def timed(a_kib, b_kib):
-        mu = mu_block[a_kib * 256:a_kib * 256 + n]
-        nu = nu_block[b_kib * 256:b_kib * 256 + n]
-        u.normal_()
-        mu.normal_(0, 0.1)
-        nu.normal_(0, 0.01).abs_()
-        ptrs = (u.data_ptr(), mu.data_ptr(), nu.data_ptr())
-
-        def launch():
-            rc = lib.toa_adam_forward_inplace(_lib.TOA_F32, *ptrs, n, B1, B2, EPS, 0.0, 1000,
-                                              stream.cuda_stream)
-            if rc:
-                raise RuntimeError(lib.toa_adam_error_string(rc).decode())
-        for _ in range(3):
-            launch()
-        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        ev0.record(stream)
-        for _ in range(reps):
-            launch()
-        ev1.record(stream)
-        torch.cuda.synchronize()
-        return 24 * n / (ev0.elapsed_time(ev1) / reps) / 1e6
-
-    phases = list(range(0, span_kib, step_kib))
-    grid, unshifted = {}, []
-    for a in phases:
-        grid[f'mu +{a} KiB'] = {f'nu +{b} KiB': round(timed(a, b)) for b in phases}
-        unshifted.append(round(timed(0, 0)))
-    shift_mu, shift_nu = (lib.toa_adam_state_shift(0, k) // 1024 for k in (0, 1))
-    return {'metric': 'forward_inplace_f32_by_state_phase', 'unit': 'GB/s', 'peak': HBM_PEAK_GBS,
-            'elements': n, 'launches_timed': reps, 'device': torch.cuda.get_device_name(0),
-            'address_mod_16KiB': {'updates': u.data_ptr() % 16384,
-                                  'mu_block': mu_block.data_ptr() % 16384,
-                                  'nu_block': nu_block.data_ptr() % 16384},
-            'library_phases_kib': {'mu': shift_mu, 'nu': shift_nu},
-            'at_library_phases': grid[f'mu +{shift_mu} KiB'][f'nu +{shift_nu} KiB'],
-            'unshifted_after_each_row': unshifted, 'GB/s_by_phase': grid}
-
-
-def run_state_distances(reps=12, n=1 << 28, distances_mib=None):
-    """The operator (float32 forward_ in place, 2^28 elements, library defaults) with the gradient
-    in a PyTorch allocation of its own and BOTH moments in one block, each 8 KiB off the 16 KiB
-    address phase, the second `n * 4 bytes + d` after the first for a ladder of distances d.  This
-    is the measurement behind the distance at which the package's init places the two moments of
-    a leaf (torchopt_amd/placement.py).  Beside it: each moment in a block of its own at the
-    phase, and at the allocator's placement."""
-    import torch
-
-    from torchopt_amd import _lib
-
-    lib = _lib.load()
-    stream = torch.cuda.current_stream()
-    if distances_mib is None:
-        distances_mib = (0, 0.25, 0.5, 1, 1.5, 2, 2.5, 3, 4, 5, 6, 7, 8, 10, 12, 14, 16, 20, 24, 32)
-    mib = 1 << 18  # float32 elements
-    phase = (8 << 10) // 4
-    u_block = torch.empty(n + 4 * phase, device='cuda')
-    u = u_block[:n]
-    block = torch.empty(2 * n + int(max(distances_mib) * mib) + 4 * phase, device='cuda')
-    own_mu = torch.empty(n + 2 * phase, device='cuda')
-    own_nu = torch.empty(n + 2 * phase, device='cuda')
-    preheat(torch)
-
-    def timed(mu, nu, launches=reps, u=u):
-        u.normal_()
-        mu.normal_(0, 0.1)
-        nu.normal_(0, 0.01).abs_()
-        ptrs = (u.data_ptr(), mu.data_ptr(), nu.data_ptr())
-
-        def launch():
-            rc = lib.toa_adam_forward_inplace(_lib.TOA_F32, *ptrs, n, B1, B2, EPS, 0.0, 1000,
-                                              stream.cuda_stream)
-            if rc:
-                raise RuntimeError(lib.toa_adam_error_string(rc).decode())
-        for _ in range(3):
-            launch()
-        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        ev0.record(stream)
-        for _ in range(launches):
-            launch()
-        ev1.record(stream)
-        torch.cuda.synchronize()
-        return round(24 * n / (ev0.elapsed_time(ev1) / launches) / 1e6)
-
-    def in_block(d):
-        at = n + int(d * mib) + phase
-        return block[phase:phase + n], block[at:at + n]
-
-    timed(*in_block(8), launches=60)  # past the operator's start-up transient
-    rounds = [{f'{d} MiB': timed(*in_block(d)) for d in distances_mib} for _ in range(2)]
-    # The two moments at one phase against 8 KiB apart (what the package's init does), 8 MiB
-    # beyond the array size apart, with the gradient's own phase shifted: an allocator puts large
-    # blocks on 2 MiB boundaries, but where the physical pages lie is not the caller's to see.
-    by_gradient_phase = {}
-    for name, (a_kib, b_kib) in (('both moments 8 KiB off', (8, 8)),
-                                 ('first moment 8 KiB off, second at 0', (8, 0)),
-                                 ('first moment at 0, second 8 KiB off', (0, 8)),
-                                 ('both moments at 0', (0, 0))):
-        mu = block[a_kib * 256:a_kib * 256 + n]
-        at = n + 8 * mib + b_kib * 256
-        nu = block[at:at + n]
-        by_gradient_phase[name] = {f'gradient +{g} KiB': timed(mu, nu, u=u_block[g * 256:g * 256 + n])
-                                   for g in (0, 4, 8, 12)}
-    return {'metric': 'forward_inplace_f32_by_moment_distance', 'unit': 'GB/s',
-            'peak': HBM_PEAK_GBS, 'elements': n, 'launches_timed': reps,
-            'device': torch.cuda.get_device_name(0),
-            'gradient_minus_block_mib': (u.data_ptr() - block.data_ptr()) / 2 ** 20,
-            'GB/s_by_distance_beyond_the_array_size': rounds,
-            'GB/s_by_phases_of_the_moments_and_of_the_gradient': by_gradient_phase,
-            'blocks_of_their_own_at_their_phases': timed(own_mu[phase:phase + n], own_nu[:n]),
-            'allocator_placement': timed(own_mu[:n], own_nu[:n])}
-
-
 # ----------------------------------------------------------------------------- CPU baseline
 
 
@@ -1662,24 +1166,6 @@ def main(argv=None):
                     help='after the timed region also run 5 plain device copies of 1 GiB, so a '
                          'rocprofv3 --pmc run holds a kernel of known traffic to scale '
                          'FETCH_SIZE / WRITE_SIZE by')
-    ap.add_argument('--ceiling', action='store_true',
-                    help='measure the streaming ceilings of this machine (probe kernels with '
-                         'the operator\'s launch shape) instead of the operator')
-    ap.add_argument('--ceiling-backward', action='store_true',
-                    help='time the float64 backward ops on 2^26 elements beside arithmetic-free '
-                         'passes of the same read / write pattern')
-    ap.add_argument('--placements', action='store_true',
-                    help='time the operator over 210 placements of its three arrays inside one '
-                         'allocation instead of the benchmark (the rate depends on the '
-                         'distances between the arrays)')
-    ap.add_argument('--state-phases', action='store_true',
-                    help='time the operator on three separate allocations with mu and nu shifted '
-                         'inside theirs by every pair of phases below 32 KiB (steps of 2 KiB): '
-                         'the measurement behind the phase at which the package allocates state')
-    ap.add_argument('--state-distances', action='store_true',
-                    help='time the operator with both moments in one block over a ladder of '
-                         'distances between them: the measurement behind the distance at which '
-                         "the package's init places the two moments of a leaf")
     args = ap.parse_args(argv)
 
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
@@ -1687,22 +1173,6 @@ def main(argv=None):
               'GPUs; each would run the same kernel on its shard). Run with --gpus 1.',
               file=sys.stderr)
         return 2
-
-    if args.ceiling:
-        print(json.dumps(run_ceiling()), flush=True)
-        return 0
-    if args.ceiling_backward:
-        print(json.dumps(run_ceiling_backward()), flush=True)
-        return 0
-    if args.placements:
-        print(json.dumps(run_placements()), flush=True)
-        return 0
-    if args.state_phases:
-        print(json.dumps(run_state_phases()), flush=True)
-        return 0
-    if args.state_distances:
-        print(json.dumps(run_state_distances()), flush=True)
-        return 0
 
     host_cores()  # before torch (and with it the OpenMP runtime) loads
 

@@ -2,6 +2,8 @@
 
 Markers
   gpu   needs a real MI355X; everything unmarked runs on CPU only.
+  perf  speed gates (tests/test_perf_gates.py): need an MI355X too, but are kept out of `-m gpu`
+        so that the GPU suite is a pure correctness signal; skipped where there is no GPU.
 
 Only the test suite, the smoke check and the benchmark's CPU-baseline leg may import
 `oracle`; the product package `torchopt_amd` never does.
@@ -24,6 +26,8 @@ GOLDEN_DIR = os.path.join(REPO, 'tests', 'golden')
 
 def pytest_configure(config):
     config.addinivalue_line('markers', 'gpu: test needs a real AMD GPU (MI355X)')
+    config.addinivalue_line('markers', 'perf: speed gate (needs an MI355X); never selected by -m gpu, '
+                                       'skipped where there is no GPU')
 
 
 def load_golden(tag: str):

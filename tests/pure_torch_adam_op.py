@@ -2,10 +2,11 @@
 
 The reference keeps such a module as the import fallback for a build without its C++ extension
 (/root/reference/torchopt/accelerated_op/_src/adam_op.py:28-130, picked at
-/root/reference/torchopt/accelerated_op/adam_op.py:27-30).  Here it is NOT a fallback: the
-package refuses to import without its HIP library, and nothing routes through this file.  It
-exists for what the reference's fallback is also good for -- a statement of the mathematics that
-runs on any device PyTorch serves, to read and to check the native op against.
+/root/reference/torchopt/accelerated_op/adam_op.py:27-30).  Here it is a test aid, kept with the
+tests and outside the package: `torchopt_amd` refuses to import without its HIP library and has
+nothing to fall back on.  It exists for what the reference's fallback is also good for -- a
+statement of the mathematics that runs on any device PyTorch serves, to read and to check the
+native op against (tests/test_src_statement.py).
 
 Same names, argument order and return shapes as the native functions.  Results agree with the
 native op closely, not bit for bit: PyTorch divides by the bias correction where the native op

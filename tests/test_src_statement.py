@@ -1,4 +1,4 @@
-"""The plain-PyTorch statement of the operator (`torchopt_amd/accelerated_op/_src/adam_op.py`)
+"""The plain-PyTorch statement of the operator (`tests/pure_torch_adam_op.py`)
 against the CPU oracle on CPU tensors, and -- on a GPU -- against the native op.  Agreement is to
 a tolerance, not bit for bit: PyTorch divides by the bias correction where the native op
 multiplies by its reciprocal, and forms (1 - b) in double where the native op forms it in the
@@ -17,11 +17,11 @@ import torch
 from oracle import adam_oracle as O
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SRC = os.path.join(HERE, '..', 'torchopt_amd', 'accelerated_op', '_src', 'adam_op.py')
+SRC = os.path.join(HERE, 'pure_torch_adam_op.py')
 
 
 def load_statement():
-    # by path: importing the package needs the HIP library, this file does not
+    # by path: it is a test aid beside this file, not a module of the package
     spec = importlib.util.spec_from_file_location('toa_src_adam_op', SRC)
     mod = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mod)
