@@ -14,7 +14,8 @@ from torchopt_amd.alias import adam, adamw, apply_updates, chain
 from torchopt_amd.func import FuncOptimizer
 from torchopt_amd.meta import MetaAdam, MetaAdamW
 from torchopt_amd.optim import Adam, AdamW, FusedAdam, FusedAdamW
-from torchopt_amd.placement import state_empty_like, state_zeros_like, state_zeros_like_tree
+from torchopt_amd.placement import (placed_like_tree, state_empty_like, state_zeros_like,
+                                    state_zeros_like_tree, unshared)
 
 # `import torchopt_amd._C.adam_op` should work like `from torchopt_amd._C import adam_op`
 from torchopt_amd import _C  # noqa: E402
@@ -24,4 +25,5 @@ _sys.modules.setdefault('torchopt_amd._C.adam_op', _C.adam_op)
 __version__ = '0.1.0'
 
 __all__ = ['Adam', 'AdamOp', 'AdamW', 'FuncOptimizer', 'FusedAdam', 'FusedAdamW', 'MetaAdam', 'MetaAdamW', 'MultiAdamOp', 'accelerated_op',
-           'accelerated_op_available', 'adam', 'adamw', 'apply_updates', 'chain', 'state_empty_like', 'state_zeros_like', 'state_zeros_like_tree']
+           'accelerated_op_available', 'adam', 'adamw', 'apply_updates', 'chain', 'placed_like_tree',
+           'state_empty_like', 'state_zeros_like', 'state_zeros_like_tree', 'unshared']

@@ -40,7 +40,7 @@ import torch
 
 from torchopt_amd.accelerated_op.adam_op import adam_op
 from torchopt_amd.base import accelerated_only
-from torchopt_amd.placement import state_zeros_like_tree
+from torchopt_amd.placement import placed_like_tree, state_zeros_like_tree
 from torchopt_amd.transform.scale_by_adam import (INT64_MAX, ScaleByAdamState, _host_value,
                                                  _remember)
 
@@ -147,7 +147,18 @@ class FusedAdam:
         return tuple(self.state_groups)
 
     def load_state_dict(self, state_dict: Sequence) -> None:
-        self.state_groups[:] = list(state_dict)
+        """Takes the state of `state_dict()` back (as /root/reference/torchopt/optim/base.py:130-135
+        does).  Large moments that do not lie where this package's own init would have put them
+        -- state that went through `torch.save` / `torch.load`, or came from another process --
+        are copied to that placement once, here, so that the steps after a restart stream as
+        fast as the steps before it; values are untouched."""
+        groups = []
+        for s in state_dict:
+            if s is not None:
+                mu, nu = placed_like_tree(s.mu, s.nu)
+                s = s._replace(mu=tuple(mu), nu=tuple(nu))
+            groups.append(s)
+        self.state_groups[:] = groups
         self._steps = [None if s is None else [_host_value(c) for c in s.count]
                        for s in self.state_groups]
         self._stale = [False] * len(self.state_groups)

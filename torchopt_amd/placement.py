@@ -18,9 +18,21 @@ separate blocks (2 MiB on a 16 MiB leaf), and a leaf's two moments lie a whole e
 between 4 and 12, plus those 8 KiB, apart modulo 16 MiB (8 MiB where that costs little): the
 distances the step streams fastest at, and clear of the multiples of 16 MiB at which arrays meet
 in the same DRAM banks.
+
+What a caller can observe of this, beside the speed: the moments of such a tree are views into a
+shared storage (non-zero ``storage_offset()``), so (a) ``torch.save`` of the whole state writes
+the block once -- sharing is preserved in the file -- but saving ONE moment leaf on its own writes
+the whole block (``unshared(t)`` gives a leaf a storage of its own first); (b) dropping or
+replacing one leaf's state frees nothing while a sibling is alive; (c) state that comes back from
+``torch.load`` (or from anywhere else) lies where the loader put it: `FusedAdam.load_state_dict`
+and `placed_like_tree` move it to the preferred placement again, one copy per leaf.  Setting the
+environment variable ``TORCHOPT_AMD_STATE_PLACEMENT=0`` (read at every allocation) switches all
+of it off: every moment is then a plain ``zeros_like`` allocation, as in the reference.
 """
 
 from __future__ import annotations
+
+import os
 
 import torch
 
@@ -31,10 +43,15 @@ from torchopt_amd import _lib
 MIN_BYTES = 1 << 20
 
 
+def placement_enabled() -> bool:
+    """False when TORCHOPT_AMD_STATE_PLACEMENT=0: state then comes from plain ``zeros_like``."""
+    return os.environ.get('TORCHOPT_AMD_STATE_PLACEMENT', '1') != '0'
+
+
 def _placed(t: torch.Tensor, zero: bool, requires_grad: bool, moment: int) -> torch.Tensor:
     size = t.numel() * t.element_size()
     if (not t.is_cuda or size < MIN_BYTES or not t.is_contiguous()
-            or t.layout != torch.strided):
+            or t.layout != torch.strided or not placement_enabled()):
         make = torch.zeros_like if zero else torch.empty_like
         return make(t, requires_grad=requires_grad)
     lib = _lib.load()
@@ -85,7 +102,42 @@ def _second_moment_offset(end: int, largest: int, period: int) -> int:
 
 def _eligible(t) -> bool:
     return (t is not None and t.is_cuda and t.layout == torch.strided and t.is_contiguous()
-            and t.numel() * t.element_size() >= MIN_BYTES)
+            and t.numel() * t.element_size() >= MIN_BYTES and placement_enabled())
+
+
+def is_placed(t: torch.Tensor, moment: int) -> bool:
+    """Does `t` start at the preferred address phase of a first (0) or second (1) moment?"""
+    return _lib.load().toa_adam_state_shift(t.data_ptr(), moment) == 0
+
+
+def unshared(t: torch.Tensor) -> torch.Tensor:
+    """`t` itself if its storage holds nothing else, a copy with a storage of its own otherwise:
+    what to hand to ``torch.save`` when ONE state leaf is to be written (a view into a tree's
+    block would take the whole block along)."""
+    if t.untyped_storage().nbytes() <= t.numel() * t.element_size() + 512:
+        return t
+    return t.detach().clone().requires_grad_(t.requires_grad)
+
+
+def placed_like_tree(mu_leaves, nu_leaves):
+    """The moments `mu_leaves`, `nu_leaves` of a flattened tree (``None`` leaves stay ``None``)
+    at the placement `state_zeros_like_tree` would have given them: leaves that are eligible (GPU,
+    contiguous, 1 MiB or more) and not already at their phases are copied into a fresh block,
+    the others are returned as they are.  Values, shapes, dtypes and ``requires_grad`` are kept.
+    For state that arrives from ``torch.load`` or another process."""
+    mu_leaves, nu_leaves = list(mu_leaves), list(nu_leaves)
+    move = [k for k, (m, v) in enumerate(zip(mu_leaves, nu_leaves))
+            if _eligible(m) and v is not None and not (is_placed(m, 0) and is_placed(v, 1))]
+    if not move:
+        return mu_leaves, nu_leaves
+    fresh_mu, fresh_nu = state_zeros_like_tree([mu_leaves[k] for k in move])
+    with torch.no_grad():
+        for k, m, v in zip(move, fresh_mu, fresh_nu):
+            m.copy_(mu_leaves[k])
+            v.copy_(nu_leaves[k])
+            mu_leaves[k] = m.requires_grad_(mu_leaves[k].requires_grad)
+            nu_leaves[k] = v.requires_grad_(nu_leaves[k].requires_grad)
+    return mu_leaves, nu_leaves
 
 
 def state_zeros_like_tree(leaves, *, requires_grad: bool = False):
