@@ -387,15 +387,19 @@ bool launch_tuned(const Op &op, const TensorPtrs<T, Op> &tp, size_t whole, unsig
                         (hipEventDestroy(sample.begin), false));
     if (!timed) (void)hipGetLastError();
     // record, launch, record: one step under the mutex, so no other launch of the library lands
-    // between the two events on this stream
+    // between the two events on this stream.  An event that fails costs the sample, never the
+    // launch: its error is cleared, so that the caller reports the launch's own status alone.
     bool recorded = timed && hipEventRecord(sample.begin, (hipStream_t)stream) == hipSuccess;
+    if (timed && !recorded) (void)hipGetLastError();
     launch_full_staged<T, Op>(sample.order, op, tp, whole, lds, stream);
     const hipError_t launch_rc = hipPeekAtLastError();
-    recorded = recorded && hipEventRecord(sample.end, (hipStream_t)stream) == hipSuccess;
+    if (recorded && hipEventRecord(sample.end, (hipStream_t)stream) != hipSuccess) {
+        recorded = false;
+        if (launch_rc == hipSuccess) (void)hipGetLastError();
+    }
     if (recorded && launch_rc == hipSuccess) {
         site->pending.push_back(sample);
     } else if (timed) {
-        if (launch_rc == hipSuccess) (void)hipGetLastError();  // an event's error, not the launch's
         (void)hipEventDestroy(sample.begin);
         (void)hipEventDestroy(sample.end);
     }
