@@ -210,9 +210,22 @@ def python_level_differentiable_step(torch, shapes, eps_root, count, wall_ms):
     def loss_alone():  # the part of both that is not Adam
         torch.autograd.grad(sum((g * g).sum() for g in grads), grads)
 
+    from torchopt_amd import MultiAdamOp
+
     base = wall_ms(loss_alone)
-    return {'python_update_plus_backward_ms': round(wall_ms(fused) - base, 5),
-            'python_per_leaf_tensor_expressions_ms': round(wall_ms(per_leaf_expressions) - base, 5)}
+    out = {'python_update_plus_backward_ms': round(wall_ms(fused) - base, 5),
+           'python_update_alone_ms': round(wall_ms(
+               lambda: transform.update(grads, state, inplace=False)), 5),
+           'python_loss_and_its_backward_alone_ms': round(base, 5)}
+    # the same tree-level autograd node written in Python (the route `torch.compile` traces)
+    MultiAdamOp.use_native_node = False
+    try:
+        out['python_update_plus_backward_ms_with_the_node_in_python'] = round(
+            wall_ms(fused) - base, 5)
+    finally:
+        MultiAdamOp.use_native_node = True
+    out['python_per_leaf_tensor_expressions_ms'] = round(wall_ms(per_leaf_expressions) - base, 5)
+    return out
 
 
 def time_backward_ops(torch, lib, cfg_id, code, dtype, tag, n, esize, eps_root, count, stream,

@@ -102,7 +102,7 @@ TOA_API int toa_adam_set_schedule(int schedule);
  * launches of a site go round the four orders (same bits every time), timed with events on the
  * caller's stream that are polled, never waited for; rounds alternate their direction and the
  * first two do not count, so a drift of the machine's rate cancels.  The fastest order is kept if
- * it beats order 0 by more than 0.15 %, order 0 otherwise.  On most placements order 0 wins; on
+ * it beats order 0 by more than 0.4 % (four samples an order cannot tell smaller differences from noise), order 0 otherwise.  On most placements order 0 wins; on
  * some another gains 1-2 %.  Up to 64 call sites are remembered.  Nothing is tuned under stream
  * capture, with an order or a residency level forced, or with a schedule other than 0.
  *   toa_adam_set_tuning         0 = every site runs order 0; 1 (default; the environment variable

@@ -221,7 +221,7 @@ const char OpTag<Op>::tag = 0;
 // ---------------------------------------------------------------------------
 constexpr int kTuneOrders = 4;
 constexpr int kTuneRounds = 6, kTuneSkippedRounds = 2;
-constexpr double kTuneMargin = 0.0015;
+constexpr double kTuneMargin = 0.004;
 constexpr size_t kTuneSites = 64;
 constexpr size_t kTuneFromBytes = (size_t)64 << 20;  // per array: launches of 60 us and more
 
