@@ -274,14 +274,20 @@ def time_backward_ops(torch, lib, cfg_id, code, dtype, tag, n, esize, eps_root, 
     return res
 
 
-def timed_region(torch, step, stream, warmup, steps):
+def timed_region(torch, step, stream, warmup, steps, before_warmup=None, before_timed=None):
     """`warmup` untimed steps, then exactly `steps` steps between two device synchronisations:
-    (wall-clock ms per step, stream ms per step from events around the same steps)."""
+    (wall-clock ms per step, stream ms per step from events around the same steps).  The two
+    hooks run on the host just before the warm-up steps and, after the first synchronisation,
+    just before the clock starts (they may enqueue work on OTHER streams)."""
+    if before_warmup is not None:
+        before_warmup()
     for _ in range(warmup):
         step()
     ev0 = torch.cuda.Event(enable_timing=True)
     ev1 = torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
+    if before_timed is not None:
+        before_timed()
     t0 = time.perf_counter()
     ev0.record(stream)
     for _ in range(steps):
@@ -329,7 +335,7 @@ class ClockProbe:
 
     SPINS = 20000  # ~60 us at 2.4 GHz: long against the counters' granularity, short in a stream
 
-    def __init__(self, torch, lib, slots=16):
+    def __init__(self, torch, lib, slots=16):  # noqa: D107
         self.torch, self.lib = torch, lib
         self.buf = torch.zeros(slots, 3, dtype=torch.int64, device='cuda')
         self.names = []
@@ -344,6 +350,11 @@ class ClockProbe:
             raise RuntimeError(self.lib.toa_adam_error_string(rc).decode())
         self.names.append((name, spins or self.SPINS))
 
+    def chain(self, name, stream, count, spins):
+        """`count` probes one after the other on `stream`: a time series of the shader clock."""
+        for k in range(count):
+            self.sample(f'{name}[{k}]', stream, spins)
+
     def read(self):
         host = self.buf.cpu().tolist()
         out = {}
@@ -351,6 +362,14 @@ class ClockProbe:
             out[name] = {'spins': spins, 'shader_clock_ticks': core, 'constant_100MHz_ticks': wall,
                          'shader_MHz': round(100.0 * core / wall, 1) if wall else None}
         return out
+
+    def series(self, name):
+        """(MHz of every probe of chain `name`, mean milliseconds a probe took)."""
+        got = [v for k, v in self.read().items() if k.startswith(name + '[') and v['shader_MHz']]
+        if not got:
+            return [], None
+        return ([round(v['shader_MHz']) for v in got],
+                round(sum(v['constant_100MHz_ticks'] for v in got) / len(got) / 1e5, 3))
 
 
 def in_situ(torch, step, stream, alg_bytes, iterations=50, busy_ms=5.0):
@@ -704,12 +723,29 @@ def run_gpu(cfg_id, steps, warmup, operator_preheat=None, state='init'):
     single_wide = ('shapes' not in cfg and not cfg.get('fresh_gradients')
                    and not alg_small(total * esize))
     if single_wide:
+        # beside these first launches a chain of clock probes runs on a second stream (one wave,
+        # ~0.5 ms a probe): the shader clock through the operator's start-up transient
+        series = ClockProbe(torch, lib, slots=128)
+        side = torch.cuda.Stream()
+        per_probe_spins = 30000
+        est_ms = bytes_per_elem * total / 6.8e9  # one step at 6.8 TB/s
         was = lib.toa_adam_set_tuning(0)
-        cold = timed_region(torch, step, stream, warmup, steps)
+        cold = timed_region(
+            torch, step, stream, warmup, steps,
+            before_warmup=lambda: series.chain('warmup', side, min(40, int(2 * est_ms * warmup) + 1),
+                                               per_probe_spins),
+            before_timed=lambda: series.chain('timed', side, min(80, int(2 * est_ms * steps) + 1),
+                                              per_probe_spins))
         lib.toa_adam_set_tuning(was)
+        torch.cuda.synchronize()
+        mhz_w, ms_w = series.series('warmup')
+        mhz_t, ms_t = series.series('timed')
         beside['cold_start'] = leg(*cold, note=(
             f'{warmup} + {steps} steps straight after upload and the PyTorch-kernel preheat: no '
-            'launch of the operator before them, load-order tuning off (order 0 throughout)'))
+            'launch of the operator before them, load-order tuning off (order 0 throughout)'),
+            shader_MHz_beside_the_warmup_steps=mhz_w, shader_MHz_beside_the_timed_steps=mhz_t,
+            ms_per_clock_probe=ms_t or ms_w)
+        del series, side
     if op_launches and single_wide:
         for _ in range(op_launches):
             step()
@@ -764,15 +800,11 @@ def run_gpu(cfg_id, steps, warmup, operator_preheat=None, state='init'):
     spread = {}
     if wall_ms > 0.05:
         reps = min(steps, 20)
-        side = None
+        beside_probes = None
         if bandwidth_bound:
-            first = probes.read().get('before_the_timed_region')
-            if first and first['shader_clock_ticks'] and first['shader_MHz']:
-                ticks_per_spin = first['shader_clock_ticks'] / first['spins']
-                want_us = 0.6 * reps * kern_ms * 1e3
-                spins = int(min(want_us * first['shader_MHz'] / ticks_per_spin, 1 << 27))
-                side = torch.cuda.Stream()
-                probes.sample('beside_the_per_step_pass', side, spins=max(spins, 1000))
+            beside_probes = ClockProbe(torch, lib, slots=64)
+            side = torch.cuda.Stream()
+            beside_probes.chain('beside', side, min(60, int(2 * reps * kern_ms) + 2), 30000)
         pairs = []
         for _ in range(reps):
             a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -786,13 +818,16 @@ def run_gpu(cfg_id, steps, warmup, operator_preheat=None, state='init'):
         spread = {'step_ms_min': round(each[0], 5), 'step_ms_median': round(each[len(each) // 2], 5),
                   'step_ms_max': round(each[-1], 5)}
         if bandwidth_bound:
+            mhz, probe_ms = beside_probes.series('beside')
             beside['clock'] = {
                 'probes': probes.read(),
+                'shader_MHz_beside_the_per_step_pass': mhz, 'ms_per_clock_probe': probe_ms,
                 'probe': 'toa_adam_clock_probe: one lane, a fixed spin of dependent integer '
                          'multiply-adds; shader-clock ticks against ticks of the constant 100 MHz '
                          'counter.  before / after: on the timed stream, either side of the timed '
-                         'region; beside: on a second stream while 20 further steps of the same '
-                         'work run',
+                         'region (the GPU otherwise idle: the boost clock); beside: a chain of '
+                         'probes on a second stream while 20 further steps of the same work run '
+                         '(those that start after the steps have ended read the boost clock again)',
                 'driver_while_steps_are_queued': busy_state}
 
     # ---- the same W + K steps with the moments where the ALLOCATOR puts them (what a caller

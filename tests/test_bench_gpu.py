@@ -24,7 +24,24 @@ def test_bench_config_runs(cfg, capsys):
     assert line['config']['workload'] == bench.CONFIGS[cfg]['name']
     roof = line['roofline']
     assert roof['bound'] == 'hbm' and roof['peak'] == 8000.0 and roof['unit'] == 'GB/s'
-    assert roof['achieved'] > 0 and roof['frac'] > 0
+    assert roof['achieved'] > 0 and roof['frac'] > 0 and roof['frac_by_wall_clock'] > 0
+    beside = line['beside_the_headline']
+    if cfg in (2, 3):  # large single tensors: every leg beside the headline
+        assert {'cold_start', 'clock', 'state_where_the_allocator_puts_it',
+                'one_launch_per_iteration_between_other_work'} <= set(beside)
+        cold = beside['cold_start']
+        assert cold['frac'] > 0 and len(cold['shader_MHz_beside_the_timed_steps']) >= 1
+        assert beside['state_where_the_allocator_puts_it']['address_mod_16KiB'] == {
+            'updates': 0, 'mu': 0, 'nu': 0}
+        assert line['config']['load_order_kept_for_this_call_site'] in (-1, 0, 1, 2, 3)
+    if cfg >= 2:  # bandwidth-bound: clock evidence and the one-launch-per-iteration leg
+        probes = beside['clock']['probes']
+        assert 300 < probes['before_the_timed_region']['shader_MHz'] < 4000
+        assert 300 < probes['after_the_timed_region']['shader_MHz'] < 4000
+        assert beside['clock']['shader_MHz_beside_the_per_step_pass']
+        situ = beside['one_launch_per_iteration_between_other_work']
+        assert situ['iterations'] == 50 and situ['other_work_ms_per_iteration'] >= 5.0
+        assert 0 < situ['operator_ms_min'] <= situ['operator_ms_median'] <= situ['operator_ms_max']
     torch.cuda.empty_cache()
 
 
