@@ -18,7 +18,7 @@ TOA_F32 = 0
 TOA_F64 = 1
 TOA_F16 = 2
 TOA_BF16 = 3
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _vp = ctypes.c_void_p
 _vpp = ctypes.POINTER(ctypes.c_void_p)

@@ -1019,7 +1019,7 @@ int backward_all_multi(size_t num, const void *const *dnew_updates,
 
 extern "C" {
 
-int toa_adam_abi_version(void) { return 4; }
+int toa_adam_abi_version(void) { return 5; }
 
 // Preferred placement of state arrays: the two moments of a tensor 8 KiB apart modulo 16 KiB.
 size_t toa_adam_state_slack(void) { return kStatePeriod; }
