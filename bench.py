@@ -58,9 +58,9 @@ BYTES_PER_ELEM = {  # op -> number of arrays streamed (multiply by the element s
 # figures belong to the kernels as they were when the profile was taken; re-record them whenever
 # adam_kernels.hpp or the launch shape changes.
 RECORDED_TRAFFIC = {
-    2: (6442418075, 'profiles/forward_inplace_f32_config2_pmc_traffic.md'),
-    4: (8516220369, 'profiles/forward_inplace_multi_f32_config4_kernel_trace_and_traffic.md'),
-    5: (9935416838, 'profiles/fused_step_multi_f32_config5_kernel_trace_and_traffic.md'),
+    2: (6442408757, 'profiles/forward_inplace_f32_config2_pmc_traffic.md'),
+    4: (8516262926, 'profiles/forward_inplace_multi_f32_config4_kernel_trace_and_traffic.md'),
+    5: (9935431788, 'profiles/fused_step_multi_f32_config5_kernel_trace_and_traffic.md'),
 }
 
 B1, B2, EPS = 0.9, 0.999, 1e-8
@@ -732,9 +732,11 @@ def run_gpu(cfg_id, steps, warmup, operator_preheat=None, state='init'):
         was = lib.toa_adam_set_tuning(0)
         cold = timed_region(
             torch, step, stream, warmup, steps,
-            before_warmup=lambda: series.chain('warmup', side, min(40, int(2 * est_ms * warmup) + 1),
+            # (the chains end before the steps they accompany do: the region's synchronisation
+            # must wait for the steps, not for the probes)
+            before_warmup=lambda: series.chain('warmup', side, min(40, int(1.4 * est_ms * warmup)),
                                                per_probe_spins),
-            before_timed=lambda: series.chain('timed', side, min(80, int(2 * est_ms * steps) + 1),
+            before_timed=lambda: series.chain('timed', side, min(80, int(1.4 * est_ms * steps)),
                                               per_probe_spins))
         lib.toa_adam_set_tuning(was)
         torch.cuda.synchronize()
