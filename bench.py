@@ -713,7 +713,7 @@ def run_gpu(cfg_id, steps, warmup, operator_preheat=None, state='init'):
     # warm-up steps, and the line says how often and on what:
     #   * float32 / float64 single tensors: on the timed arrays themselves, as the first steps of
     #     a training run would (the library also settles its choice of load order for this call
-    #     site during its first 24 launches); what the same W + K steps read WITHOUT any of that
+    #     site during its first 30 launches); what the same W + K steps read WITHOUT any of that
     #     is measured first and reported as `cold_start`;
     #   * the 16-bit single tensors and the lists: on scratch state of the same shape (the 16-bit
     #     step's speed depends on its data, which a step fed its own output drifts away from);

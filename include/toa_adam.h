@@ -98,19 +98,21 @@ TOA_API int toa_adam_set_schedule(int schedule);
  * previous setting.  No counterpart in the reference.
  *
  * The library's choice is made per call site -- the in-place step on one set of three arrays of
- * one length, 64 MiB or more each -- by measurement on the caller's own launches: the first 24
- * launches of a site go round the four orders (same bits every time), timed with events on the
+ * one length, 64 MiB or more each -- by measurement on the caller's own launches: the first 30
+ * launches of a site go round the four orders and the plain schedule (all loads, then all stores;
+ * same bits every time), timed with events on the
  * caller's stream that are polled, never waited for; rounds alternate their direction and the
- * first two do not count, so a drift of the machine's rate cancels.  The fastest order is kept if
+ * first two do not count, so a drift of the machine's rate cancels.  The fastest variant is kept if
  * it beats order 0 by more than 0.4 % (four samples an order cannot tell smaller differences from noise), order 0 otherwise.  On most placements order 0 wins; on
  * some another gains 1-2 %.  Up to 64 call sites are remembered.  Nothing is tuned under stream
  * capture, with an order or a residency level forced, or with a schedule other than 0.
  *   toa_adam_set_tuning         0 = every site runs order 0; 1 (default; the environment variable
  *                               TOA_ADAM_TUNING=0 starts with 0) = as above.  Returns the previous
  *                               setting.
- *   toa_adam_tuned_load_order   the order kept for that call site of toa_adam_forward_inplace, or
- *                               -1 while it is unknown or still being explored (the _devcount
- *                               form of the step keeps sites of its own). */
+ *   toa_adam_tuned_load_order   what was kept for that call site of toa_adam_forward_inplace: 0-3
+ *                               an order of the staged program, 4 the plain schedule, -1 while
+ *                               it is unknown or still being explored (the _devcount form of
+ *                               the step keeps sites of its own). */
 TOA_API int toa_adam_set_load_order(int order);
 TOA_API int toa_adam_set_tuning(int on);
 TOA_API int toa_adam_tuned_load_order(int dtype, const void *updates, const void *mu,

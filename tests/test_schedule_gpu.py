@@ -152,8 +152,8 @@ def test_every_load_order_of_the_staged_step_matches_the_oracle(tag):
 
 @pytest.mark.parametrize('tag', ['f32', 'f64'])
 def test_the_load_order_is_chosen_per_call_site_and_changes_no_bit(tag):
-    """A call site of 64 MiB per array is explored over its first 24 launches (four orders, six
-    rounds) and then keeps one order; forty steps on it give the bits of forty steps with tuning
+    """A call site of 64 MiB per array is explored over its first 30 launches (four load orders and the
+    plain schedule, six rounds) and then keeps one of them; forty steps on it give the bits of forty steps with tuning
     off (order 0 throughout) -- and, for the first of them, the oracle's.  With tuning off, under
     a forced order or below the size limit no site is recorded."""
     lib = _lib.load()
@@ -191,10 +191,10 @@ def test_the_load_order_is_chosen_per_call_site_and_changes_no_bit(tag):
         rc = lib.toa_adam_forward_inplace(code, *[a.data_ptr() for a in tuned], n, B1, B2, 1e-8,
                                           1e-8, k + 1, stream)
         assert rc == 0
-        if k in (5, 23):
-            assert site(tuned) == -1 or k == 23  # exploring: nothing is decided before 24 launches
+        if k in (5, 29):
+            assert site(tuned) == -1 or k == 29  # exploring: nothing is decided before 30 launches
     torch.cuda.synchronize()
-    assert site(tuned) in (0, 1, 2, 3)  # every sample is back: decided
+    assert site(tuned) in (0, 1, 2, 3, 4)  # every sample is back: decided
     for a, b, name in zip(tuned, plain, ('updates', 'mu', 'nu')):
         assert torch.equal(a.view(torch.int32), b.view(torch.int32)), f'{tag} tuned != untuned {name}'
     # no site for a forced order, a forced level, or arrays below the limit

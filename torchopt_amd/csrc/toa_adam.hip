@@ -210,16 +210,20 @@ const char OpTag<Op>::tag = 0;
 // arrays lie, and with it which of the four load orders of the staged program streams fastest:
 // on most placements the first (g, mu, nu) does, on some another gains 1-2 %.  The results are
 // the same bits in every order, so the library can try them on the caller's own launches: the
-// first kTuneRounds x 4 launches of a call site (one op on one set of arrays of one length) go
-// round the four orders, timed with events on the caller's stream; rounds alternate their
+// first kTuneRounds x 5 launches of a call site (one op on one set of arrays of one length) go
+// round the four orders and the plain schedule (all loads, then all stores at its own residency
+// level: on a few placements -- both moments 4 KiB off the gradient's phase is one -- it beats
+// every staged order by 1-2 %), timed with events on the caller's stream; rounds alternate their
 // direction and the first two do not count, so a drift in the machine's rate (clocks settling
 // under a new load) cancels instead of favouring whatever ran last.  Once every sample has come
-// back -- events are polled, never waited for -- the order with the lowest mean time is kept for
+// back -- events are polled, never waited for -- the variant with the lowest mean time is kept for
 // the call site if it beats the default order by more than kTuneMargin, the default otherwise.
 // Nothing is tuned under stream capture, with an order or residency level forced, or with
 // tuning switched off; up to kTuneSites call sites are remembered, least recently used first out.
 // ---------------------------------------------------------------------------
-constexpr int kTuneOrders = 4;
+constexpr int kTuneOrders = 4;    // load orders of the staged program
+constexpr int kTuneVariants = 5;  // ... and the plain schedule (all loads, then all stores)
+constexpr int kTunePlain = 4;
 constexpr int kTuneRounds = 6, kTuneSkippedRounds = 2;
 constexpr double kTuneMargin = 0.004;
 constexpr size_t kTuneSites = 64;
@@ -243,10 +247,10 @@ struct TuneSite {
     size_t n = 0;
     int device = 0;
     uint64_t stamp = 0;
-    int decided = -1;  // the order kept, or -1 while the site is being explored
+    int decided = -1;  // the variant kept (0-3 an order, 4 plain), or -1 while being explored
     int launches = 0;  // exploring launches issued so far
-    double sum[kTuneOrders] = {0, 0, 0, 0};
-    int count[kTuneOrders] = {0, 0, 0, 0};
+    double sum[kTuneVariants] = {0, 0, 0, 0, 0};
+    int count[kTuneVariants] = {0, 0, 0, 0, 0};
     struct Sample {
         int order;
         bool counted;
@@ -290,16 +294,16 @@ void tune_collect(TuneSite &site) {
         (void)hipEventDestroy(s.end);
     }
     site.pending.resize(kept);
-    if (site.launches < kTuneRounds * kTuneOrders || !site.pending.empty()) return;
+    if (site.launches < kTuneRounds * kTuneVariants || !site.pending.empty()) return;
     int best = 0;
     bool complete = true;
-    double mean[kTuneOrders];
-    for (int o = 0; o < kTuneOrders; ++o) {
+    double mean[kTuneVariants];
+    for (int o = 0; o < kTuneVariants; ++o) {
         complete = complete && site.count[o] == kTuneRounds - kTuneSkippedRounds;
         mean[o] = site.count[o] ? site.sum[o] / site.count[o] : 0.0;
     }
     if (complete)
-        for (int o = 1; o < kTuneOrders; ++o)
+        for (int o = 1; o < kTuneVariants; ++o)
             if (mean[o] < mean[best]) best = o;
     site.decided = (complete && mean[best] < mean[0] * (1.0 - kTuneMargin)) ? best : 0;
 }
@@ -370,16 +374,25 @@ bool launch_tuned(const Op &op, const TensorPtrs<T, Op> &tp, size_t whole, unsig
     std::unique_lock<std::mutex> lock(g_tune_mutex);
     TuneSite *site = tune_find(&OpTag<Op>::tag, p, whole, device, true);
     if (site->decided < 0) tune_collect(*site);
-    if (site->decided >= 0 || site->launches >= kTuneRounds * kTuneOrders) {
+    // one variant of the five: a load order of the staged program, or the plain schedule
+    auto launch_variant = [&](int variant) {
+        if (variant == kTunePlain)
+            hipLaunchKernelGGL((full_tiles_kernel<T, Op, kUnroll, kNonTemporal>),
+                               dim3((unsigned)whole), dim3(kBlock), lds_reservation<Op>(false, whole),
+                               (hipStream_t)stream, op, tp);
+        else
+            launch_full_staged<T, Op>(variant, op, tp, whole, lds, stream);
+    };
+    if (site->decided >= 0 || site->launches >= kTuneRounds * kTuneVariants) {
         // settled, or every exploring launch is out and its samples are still on their way
-        const int order = site->decided >= 0 ? site->decided : 0;
+        const int variant = site->decided >= 0 ? site->decided : 0;
         lock.unlock();
-        launch_full_staged<T, Op>(order, op, tp, whole, lds, stream);
+        launch_variant(variant);
         return true;
     }
-    const int round = site->launches / kTuneOrders, at = site->launches % kTuneOrders;
+    const int round = site->launches / kTuneVariants, at = site->launches % kTuneVariants;
     TuneSite::Sample sample;
-    sample.order = round % 2 == 0 ? at : kTuneOrders - 1 - at;
+    sample.order = round % 2 == 0 ? at : kTuneVariants - 1 - at;
     sample.counted = round >= kTuneSkippedRounds;
     ++site->launches;
     const bool timed = hipEventCreate(&sample.begin) == hipSuccess &&
@@ -391,7 +404,7 @@ bool launch_tuned(const Op &op, const TensorPtrs<T, Op> &tp, size_t whole, unsig
     // launch: its error is cleared, so that the caller reports the launch's own status alone.
     bool recorded = timed && hipEventRecord(sample.begin, (hipStream_t)stream) == hipSuccess;
     if (timed && !recorded) (void)hipGetLastError();
-    launch_full_staged<T, Op>(sample.order, op, tp, whole, lds, stream);
+    launch_variant(sample.order);
     const hipError_t launch_rc = hipPeekAtLastError();
     if (recorded && hipEventRecord(sample.end, (hipStream_t)stream) != hipSuccess) {
         recorded = false;
