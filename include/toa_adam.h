@@ -94,8 +94,8 @@ TOA_API int toa_adam_set_schedule(int schedule);
  *   0  g | mu | store mu', nu | store nu', store u'      2  mu | g | store mu', nu | ...
  *   1  g | nu | store nu', mu | store mu', store u'      3  nu | g | store nu', mu | ...
  *  -1  (default) the library's choice.
- * bfloat16, lists and the other ops have one order; the setting is ignored there.  Returns the
- * previous setting.  No counterpart in the reference.
+ * The 16-bit types, lists and the other ops have one order; the setting is ignored there.
+ * Returns the previous setting.  No counterpart in the reference.
  *
  * The library's choice is made per call site -- the in-place step on one set of three arrays of
  * one length, 64 MiB or more each -- by measurement on the caller's own launches: the first 30

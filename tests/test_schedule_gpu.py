@@ -108,7 +108,7 @@ def test_staged_schedule_at_every_residency_level(levels):
 def test_every_load_order_of_the_staged_step_matches_the_oracle(tag):
     """Which moment the staged program handles first, and whether it loads it before the
     gradient, moves the rate with the placement of the arrays and nothing else: all four orders
-    (bfloat16 has one, whatever is asked for), at the three residency levels around the default,
+    (the 16-bit types have one, whatever is asked for), at the three residency levels around the default,
     give the oracle's bits -- through the host-counted and the device-counted entry point."""
     lib = _lib.load()
     n = BIG[tag]

@@ -228,8 +228,60 @@ struct Pair16 {
     }
     __device__ Pair16(int i) { *this = rounded((float)i, (float)i); }
     __device__ Pair16(Float2 f) { *this = rounded(f.lo, f.hi); }  // the one rounding of a result
-    __device__ R16<F> half(int h) const { return R16<F>(h ? hi : lo); }
+    __device__ float low() const { return lo; }
+    __device__ float high() const { return hi; }
 };
+
+// float16 pairs compute in the hardware's own packed half arithmetic.  An operation between two
+// float16 values, run in float and rounded back (what c10::Half does), IS the correctly rounded
+// float16 operation: a product of two 11-bit significands is exact in float's 24, and a sum or
+// difference rounded first to 24 bits and then to 11 rounds as if rounded once (double rounding is
+// innocuous when the wider format has at least 2 x 11 + 2 bits).  So v_pk_mul_f16 / v_pk_add_f16
+// give the reference's bits for two elements per instruction with no conversion in between --
+// never fused: the build contracts nothing.  The root, the sum with eps and the quotient of the
+// step direction stay in float, as for one value.
+template <>
+struct Pair16<HalfFormat> {
+    typedef _Float16 Halves __attribute__((ext_vector_type(2)));
+    Halves v;
+    Pair16() = default;
+    __device__ static Pair16 from_bits(uint32_t p) {
+        Pair16 r;
+        r.v = __builtin_bit_cast(Halves, p);
+        return r;
+    }
+    __device__ static Pair16 rounded(float a, float b) { return from_bits(HalfFormat::encode2(a, b)); }
+    __device__ uint32_t bits() const { return __builtin_bit_cast(uint32_t, v); }
+    __device__ explicit Pair16(R16<HalfFormat> s) {
+        // through integer arithmetic: picking a 16-bit field out of the op as a half vector makes
+        // the compiler keep the op in memory (promoted to LDS, which costs residency)
+        const uint32_t w = s.bits;
+        v = __builtin_bit_cast(Halves, w | (w << 16));
+    }
+    __device__ Pair16(int i) {
+        const _Float16 h = static_cast<_Float16>(static_cast<float>(i));
+        v = Halves{h, h};
+    }
+    __device__ Pair16(Float2 f) { *this = rounded(f.lo, f.hi); }  // the one rounding of a result
+    __device__ float low() const { return static_cast<float>(v[0]); }
+    __device__ float high() const { return static_cast<float>(v[1]); }
+};
+// sums, differences and products of float16 pairs: the packed half instructions
+#define TOA_HALF_PAIR_BINOP(OP)                                                                  \
+    __device__ inline Pair16<HalfFormat> operator OP(Pair16<HalfFormat> a,                       \
+                                                     Pair16<HalfFormat> b) {                     \
+        Pair16<HalfFormat> r;                                                                    \
+        r.v = a.v OP b.v;                                                                        \
+        return r;                                                                                \
+    }
+TOA_HALF_PAIR_BINOP(+)
+TOA_HALF_PAIR_BINOP(-)
+TOA_HALF_PAIR_BINOP(*)
+#undef TOA_HALF_PAIR_BINOP
+// a quotient of float16 values goes through float's correctly rounded division
+__device__ inline Pair16<HalfFormat> operator/(Pair16<HalfFormat> a, Pair16<HalfFormat> b) {
+    return Pair16<HalfFormat>::rounded(a.low() / b.low(), a.high() / b.high());
+}
 #define TOA_PAIR_BINOP(OP)                                                                       \
     template <class F>                                                                           \
     __device__ inline Pair16<F> operator OP(Pair16<F> a, Pair16<F> b) {                          \
@@ -239,13 +291,16 @@ struct Pair16 {
     __device__ inline Pair16<F> operator OP(int a, Pair16<F> b) {                                \
         return Pair16<F>(a) OP b;                                                                \
     }                                                                                            \
+    __device__ inline Pair16<HalfFormat> operator OP(int a, Pair16<HalfFormat> b) {              \
+        return Pair16<HalfFormat>(a) OP b;                                                       \
+    }                                                                                            \
     template <class F>                                                                           \
     __device__ inline Float2 operator OP(Pair16<F> a, Float2 b) {                                \
-        return {a.lo OP b.lo, a.hi OP b.hi};                                                     \
+        return {a.low() OP b.lo, a.high() OP b.hi};                                              \
     }                                                                                            \
     template <class F>                                                                           \
     __device__ inline Float2 operator OP(Float2 a, Pair16<F> b) {                                \
-        return {a.lo OP b.lo, a.hi OP b.hi};                                                     \
+        return {a.lo OP b.low(), a.hi OP b.high()};                                              \
     }
 TOA_PAIR_BINOP(+)
 TOA_PAIR_BINOP(-)
@@ -337,7 +392,7 @@ __device__ __forceinline__ float toa_sqrt(R16<F> x) { return sqrtf((float)x); }
 // as for one 16-bit value: the root is taken in float and NOT rounded back
 template <class F>
 __device__ __forceinline__ Float2 toa_sqrt(Pair16<F> x) {
-    return {sqrtf(x.lo), sqrtf(x.hi)};
+    return {sqrtf(x.low()), sqrtf(x.high())};
 }
 
 // The step direction mu_hat / (sqrt(nu_hat + eps_root) + eps) as the reference writes it
@@ -432,7 +487,7 @@ __device__ __forceinline__ Pair16<F> adam_direction_quick(Pair16<F> mh, Pair16<F
                                                           uint32_t &bad) {
     using L = QuickLimits<F>;
     const Pair16<F> x = vh + eps_root;
-    const float e = eps.lo;  // both halves hold the same hyper-parameter
+    const float e = eps.low();  // both halves hold the same hyper-parameter
     // eps = 0 is served too: the radicand must then be positive (a zero one would divide by zero)
     const bool eps_fits = ((e >= 5.42101086e-20f) & (e <= 9.22337204e18f)) | (e == 0.0f);
     const int radicand_classes = e == 0.0f ? 0x100 : 0x160;
@@ -449,8 +504,8 @@ __device__ __forceinline__ Pair16<F> adam_direction_quick(Pair16<F> mh, Pair16<F
         return radicand & range & clear;
     };
     float q_lo, q_hi;
-    const bool ok_lo = one(x.lo, mh.lo, q_lo) & eps_fits;
-    const bool ok_hi = one(x.hi, mh.hi, q_hi) & eps_fits;
+    const bool ok_lo = one(x.low(), mh.low(), q_lo) & eps_fits;
+    const bool ok_hi = one(x.high(), mh.high(), q_hi) & eps_fits;
     bad = (ok_lo ? 0u : 1u) | (ok_hi ? 0u : 2u);
     return Pair16<F>::rounded(q_lo, q_hi);
 }
@@ -657,10 +712,10 @@ struct alignas(8) AdamSteps {
     __device__ __forceinline__ void staged_steps(const IO &io) const {
         using V = typename Vec<T>::type;
         constexpr int VN = Vec<T>::N;
-        if constexpr (__is_same(T, bfloat_t)) {
-            // bfloat16: two elements per step (see Pair16), the quick route for both.  (float16
-            // gains nothing from pairs here -- its roundings have no one-instruction form -- and
-            // takes the element-wise branch below.)
+        if constexpr (sizeof(T) == 2) {
+            // the 16-bit types: two elements per step (see Pair16: bfloat16 rounds a pair with
+            // one instruction, float16 computes in packed half arithmetic), the quick route for
+            // both elements
             using P = typename PairOf<T>::type;
             typedef uint32_t Words __attribute__((ext_vector_type(4)));
             const Words g = __builtin_bit_cast(Words, io.load(0));
@@ -788,9 +843,9 @@ struct ForwardInplace : AdamSteps<T> {
     __device__ static constexpr int out_slot(int j) { return j == 0 ? 1 : (j == 1 ? 2 : 0); }
     static constexpr bool kSpeculative = HasQuickDirection<T>::value;
     static constexpr bool kPairs = true;
-    // The staged program exists in four load orders (bfloat16, which computes in pairs, in one):
-    // which order streams fastest depends on where the three arrays lie, see staged_steps.
-    static constexpr int kLoadOrders = __is_same(T, bfloat_t) ? 1 : 4;
+    // The staged program exists in four load orders (the 16-bit types, which compute in pairs, in
+    // one): which order streams fastest depends on where the three arrays lie, see staged_steps.
+    static constexpr int kLoadOrders = sizeof(T) == 2 ? 1 : 4;
     template <class IO>
     __device__ __forceinline__ void staged(const IO &io) const {
         this->template staged_steps<ForwardInplace, 0>(io);

@@ -1087,7 +1087,6 @@ int toa_adam_tuned_load_order(int dtype, const void *updates, const void *mu, co
     switch (dtype) {
         case TOA_F32: return look(&OpTag<ForwardInplace<float>>::tag, Tile<float, kUnroll>::ELEMS);
         case TOA_F64: return look(&OpTag<ForwardInplace<double>>::tag, Tile<double, kUnroll>::ELEMS);
-        case TOA_F16: return look(&OpTag<ForwardInplace<half_t>>::tag, Tile<half_t, kUnroll>::ELEMS);
         default: return -1;
     }
 }
