@@ -1179,6 +1179,67 @@ struct alignas(8) FusedStep {
     template <class IO>
     __device__ __forceinline__ void staged(const IO &io) const {
         using V = typename Vec<T>::type;
+        if constexpr (sizeof(T) == 2) {
+            // The 16-bit types (which take no weight decay): two elements per step, as the
+            // in-place step computes them (Pair16), the quick route for the direction.
+            // load g | load mu | store mu', load nu | store nu', load p | store p' [, store u']
+            using P = typename PairOf<T>::type;
+            typedef uint32_t Words __attribute__((ext_vector_type(4)));
+            constexpr int VN = Vec<T>::N;
+            const AdamSteps<T> adam{b1, b2, c1, c2, eps, eps_root};
+            Words g = __builtin_bit_cast(Words, io.load(0));
+            io.wait();
+            if (maximize) g ^= 0x80008000u;  // -g: the sign bit of both halves
+            const Words m = __builtin_bit_cast(Words, io.load(1));
+            io.wait();
+            P gp[4], ap[4], bp[4];
+            Words a, b, c;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                gp[e] = P::from_bits(g[e]);
+                ap[e] = adam.template first<P>(gp[e], P::from_bits(m[e]));
+                a[e] = ap[e].bits();
+            }
+            io.store(1, __builtin_bit_cast(V, a));
+            const Words v = __builtin_bit_cast(Words, io.load(2));
+            io.wait();
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                bp[e] = adam.template second<P>(gp[e], P::from_bits(v[e]));
+                b[e] = bp[e].bits();
+            }
+            io.store(2, __builtin_bit_cast(V, b));
+            const Words p = __builtin_bit_cast(Words, io.load(3));
+            uint32_t redo = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                P r;
+                redo |= adam.template third_quick_pair<P>(ap[e], bp[e], r) << (2 * e);
+                c[e] = r.bits();
+            }
+            V dir = __builtin_bit_cast(V, c);
+            if (redo != 0) {  // rare: an element the quick route could not settle
+                const V av = __builtin_bit_cast(V, a), bv = __builtin_bit_cast(V, b);
+#pragma unroll
+                for (int e = 0; e < VN; ++e)
+                    if (redo & (1u << e))
+                        Vec<T>::set(dir, e,
+                                    adam.template third<T>(Vec<T>::get(av, e), Vec<T>::get(bv, e)));
+            }
+            io.wait();
+            const Words d = __builtin_bit_cast(Words, dir);
+            Words p1, step;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                // the update times float(-lr), rounded once; then params plus that, rounded once
+                const P st(P::from_bits(d[e]) * Float2{neg_lr, neg_lr});
+                step[e] = st.bits();
+                p1[e] = (P::from_bits(p[e]) + st).bits();
+            }
+            io.store(3, __builtin_bit_cast(V, p1));
+            if constexpr (WRITE_UPDATES) io.store(0, __builtin_bit_cast(V, step));
+            return;
+        }
         const bool early_p = decay == kDecayIntoGradient;
         V g = io.load(0);
         V p;
