@@ -330,6 +330,92 @@ def test_native_node_contract():
     assert adam_op.step_multi([], [], [], B1, B2, EPS, 0.0, 1) == ([], [], [])
 
 
+def test_native_node_behaves_like_any_autograd_node():
+    """The node is written against autograd's Node interface directly, so what a Function gets
+    for free is checked here: saved tensors released after a backward without retain_graph (and
+    the usual error on a second one), identical gradients from repeated backwards with
+    retain_graph, the version check on saved tensors, saved-tensor hooks, a layout-converted
+    input, and no reference cycle between the node and the outputs it saves."""
+    import gc
+
+    from torchopt_amd._C import adam_op
+
+    def fresh():
+        torch.manual_seed(3)
+        g = [torch.randn(64, 3, device='cuda', requires_grad=True),
+             torch.randn(17, device='cuda', requires_grad=True)]
+        mu = [torch.randn_like(x).mul_(0.1).requires_grad_(True) for x in g]
+        nu = [torch.rand_like(x).mul_(0.01).requires_grad_(True) for x in g]
+        return g, mu, nu
+
+    def loss_of(out):
+        return sum((t * t).sum() for lst in out for t in lst)
+
+    g, mu, nu = fresh()
+    out = adam_op.step_multi(g, mu, nu, B1, B2, EPS, 1e-8, 2)
+    assert out[0][0].grad_fn.name() == 'AdamStepBackward'
+    assert all(t.grad_fn is out[0][0].grad_fn for lst in out for t in lst)
+    loss = loss_of(out)
+    first = torch.autograd.grad(loss, g + mu + nu, retain_graph=True)
+    second = torch.autograd.grad(loss, g + mu + nu)
+    for a, b in zip(first, second):
+        assert torch.equal(a, b)
+    with pytest.raises(RuntimeError, match='second time'):
+        torch.autograd.grad(loss, g + mu + nu)
+
+    # a saved tensor modified in place between forward and backward is caught
+    g, mu, nu = fresh()
+    out = adam_op.step_multi(g, mu, nu, B1, B2, EPS, 1e-8, 2)
+    loss = loss_of(out)
+    with torch.no_grad():
+        out[0][1].add_(1.0)  # new_mu of the second leaf, saved for backward
+    with pytest.raises(RuntimeError, match='modified by an inplace operation'):
+        loss.backward()
+
+    # saved-tensor hooks see the 3 tensors per leaf the reference's Functions save
+    g, mu, nu = fresh()
+    packed = []
+
+    def pack(t):
+        packed.append(t.shape)
+        return t
+
+    with torch.autograd.graph.saved_tensors_hooks(pack, lambda t: t):
+        out = adam_op.step_multi(g, mu, nu, B1, B2, EPS, 1e-8, 2)
+    assert len(packed) == 3 * len(g)
+    want = torch.autograd.grad(loss_of(out), g + mu + nu)
+    for a, b in zip(first, want):
+        assert torch.equal(a, b)
+
+    # an expanded gradient (what sum().backward() hands on): converted inside, its gradient
+    # comes back in the input's own shape
+    base = torch.randn(1, device='cuda', requires_grad=True)
+    ge = [base.expand(64, 3), g[1]]
+    out = adam_op.step_multi(ge, mu, nu, B1, B2, EPS, 1e-8, 2)
+    (d_base,) = torch.autograd.grad(loss_of(out), [base])
+    dense = base.detach().expand(64, 3).contiguous().requires_grad_(True)
+    out2 = adam_op.step_multi([dense, g[1]], mu, nu, B1, B2, EPS, 1e-8, 2)
+    (d_dense,) = torch.autograd.grad(loss_of(out2), [dense])
+    torch.testing.assert_close(d_base, d_dense.sum().reshape(1), rtol=1e-5, atol=0)
+
+    # dropping the outputs frees their memory at once: the node holds its saved outputs
+    # without a cycle through their grad_fn
+    del out, out2, loss, want, first, second
+    gc.collect()
+    gc.disable()
+    try:
+        big = [torch.randn(1 << 20, device='cuda', requires_grad=True)]
+        zeros = [torch.zeros(1 << 20, device='cuda')]
+        torch.cuda.synchronize()
+        before = torch.cuda.memory_allocated()
+        held = adam_op.step_multi(big, zeros, zeros, B1, B2, EPS, 1e-8, 1)
+        assert torch.cuda.memory_allocated() >= before + 3 * (1 << 22)  # the three outputs
+        del held
+        assert torch.cuda.memory_allocated() == before
+    finally:
+        gc.enable()
+
+
 def test_meta_step_through_the_transformation():
     """A MAML-style inner step: params' = params - lr * adam(grad); the outer loss
     differentiates through the update, the moments and the step."""

@@ -127,7 +127,7 @@ class MultiAdamOp:
     (`forward_all_multi`) and backward (`backward_all_multi`) are one multi-tensor pass each, so
     a tree of any size costs two launches per step instead of six per leaf, and each direction
     reads its operands once.  Values and gradients are bit-identical to the per-leaf `AdamOp`.
-    The node lives in the extension module (`adam_op.step_multi`, a C++ autograd function: no
+    The node lives in the extension module (`adam_op.step_multi`, a C++ autograd node: no
     Python runs between autograd's engine and the launches); `StepOp` below is the same node
     written in Python, the route taken while `torch.compile` traces.
 

@@ -24,7 +24,10 @@
 #include <c10/hip/HIPStream.h>
 #include <hip/hip_runtime_api.h>
 #include <pybind11/stl.h>
-#include <torch/csrc/autograd/custom_function.h>
+#include <ATen/FuncTorchTLS.h>
+#include <torch/csrc/autograd/function.h>
+#include <torch/csrc/autograd/functions/utils.h>
+#include <torch/csrc/autograd/saved_variable.h>
 #include <torch/extension.h>
 
 #include <array>
@@ -732,52 +735,64 @@ std::tuple<TensorList, TensorList, TensorList> backwardAllMulti(
 // Living in C++ it costs the host no Python between autograd's engine and the launch: the
 // same node written in Python spends 0.2 ms per step on a ten-leaf tree (list slicing, per-leaf
 // pybind conversions), twenty times what its two launches take on the device.
-class AdamStepNode : public torch::autograd::Function<AdamStepNode> {
-  public:
+//
+// The node derives from torch::autograd::Node itself, as PyTorch's own derivative nodes do,
+// not from torch::autograd::Function: that wrapper's per-call work (an input record and an
+// output record per tensor, sets of dirty and non-differentiable tensors, conversions of the
+// argument pack and of the result) costs more host time on thirty inputs and thirty outputs
+// than the node's own forward.  What Function would have provided is done here by hand: the
+// edges to the inputs' gradient functions, the outputs' history, saved variables (so version
+// checks and saved-tensor hooks behave as for any node), the lock around apply and the release
+// of the saved tensors after a backward without retain_graph.  Compiled autograd does not know
+// the node (no compiled_args); torch.compile traces the Python twin instead.
+struct AdamStepBackward : public torch::autograd::Node {
     using variable_list = torch::autograd::variable_list;
-    using Context = torch::autograd::AutogradContext;
 
-    static variable_list forward(Context *ctx, at::TensorList updates, at::TensorList mu,
-                                 at::TensorList nu, double b1, double b2, double eps,
-                                 double eps_root, std::vector<int64_t> counts) {
-        const size_t k = mu.size();
-        auto [new_mu, new_nu, new_updates] = forwardAllMultiImpl(
-            updates.vec(), mu.vec(), nu.vec(), b1, b2, eps, eps_root, countsOf(counts, k));
-        variable_list keep;
-        keep.reserve(3 * k);
-        keep.insert(keep.end(), new_updates.begin(), new_updates.end());
-        keep.insert(keep.end(), new_mu.begin(), new_mu.end());
-        keep.insert(keep.end(), updates.begin(), updates.end());
-        ctx->save_for_backward(std::move(keep));
-        ctx->saved_data["b1"] = b1;
-        ctx->saved_data["b2"] = b2;
-        ctx->saved_data["eps_root"] = eps_root;
-        ctx->saved_data["counts"] = std::move(counts);
-        ctx->set_materialize_grads(false);  // a missing gradient must stay missing
-        variable_list out;
-        out.reserve(3 * k);
-        for (TensorList *l : {&new_mu, &new_nu, &new_updates})
-            for (Tensor &t : *l) out.push_back(std::move(t));
-        return out;
+    size_t k = 0;
+    // new_updates, new_mu (outputs of this node) and updates (an input), k of each
+    std::vector<torch::autograd::SavedVariable> saved;
+    bool released = false;
+    double b1 = 0, b2 = 0, eps_root = 0;
+    std::vector<int64_t> counts;
+
+    std::string name() const override { return "AdamStepBackward"; }
+
+    void release_variables() override {
+        std::lock_guard<std::mutex> lock(mutex_);
+        saved.clear();
+        released = true;
     }
 
-    static variable_list backward(Context *ctx, variable_list grads) {
-        const variable_list saved = ctx->get_saved_variables();
-        const size_t k = saved.size() / 3;
+    static Counts countsOf(const std::vector<int64_t> &values, size_t num) {
+        Counts c;
+        if (values.size() == 1) {
+            c.all = (uint64_t)values[0];
+        } else {
+            TORCH_CHECK(values.size() == num, "adamStep: expected ", num, " counts, got ",
+                        values.size());
+            c.each.assign(values.begin(), values.end());
+        }
+        return c;
+    }
+
+    // grads: for new_mu, new_nu, new_updates of every leaf (undefined where none arrived: the
+    // engine does not materialize zeros for a plain Node).  Returns d(updates), d(mu), d(nu).
+    variable_list apply(variable_list &&grads) override {
+        std::lock_guard<std::mutex> lock(mutex_);
+        TORCH_CHECK(!released, torch::autograd::ERR_BACKWARD_TWICE);
         TORCH_CHECK(grads.size() == 3 * k, "adamStep: expected ", 3 * k, " gradients, got ",
                     grads.size());
-        const double b1 = ctx->saved_data["b1"].toDouble(), b2 = ctx->saved_data["b2"].toDouble(),
-                     eps_root = ctx->saved_data["eps_root"].toDouble();
-        const std::vector<int64_t> counts = ctx->saved_data["counts"].toIntVector();
-        auto part = [&](const variable_list &v, size_t j) {
-            return TensorList(v.begin() + j * k, v.begin() + (j + 1) * k);
-        };
-        const TensorList new_updates = part(saved, 0), new_mu = part(saved, 1),
-                         updates = part(saved, 2);
-        const TensorList g_mu = part(grads, 0), g_nu = part(grads, 1), g_u = part(grads, 2);
+        const std::shared_ptr<Node> self = shared_from_this();
+        TensorList new_updates, new_mu, updates;
+        new_updates.reserve(k);
+        new_mu.reserve(k);
+        updates.reserve(k);
+        for (size_t i = 0; i < k; ++i) new_updates.push_back(saved[i].unpack(self));
+        for (size_t i = 0; i < k; ++i) new_mu.push_back(saved[k + i].unpack(self));
+        for (size_t i = 0; i < k; ++i) updates.push_back(saved[2 * k + i].unpack());
+        const Tensor *g_mu = grads.data(), *g_nu = grads.data() + k, *g_u = grads.data() + 2 * k;
 
-        // d(updates), d(mu), d(nu) per leaf, then nothing for the five non-tensor arguments
-        variable_list result(3 * k + 5);
+        variable_list result(3 * k);
         Tensor *dupdates = result.data(), *dmu = result.data() + k, *dnu = result.data() + 2 * k;
 
         std::vector<size_t> live, via_mu, via_nu;
@@ -789,12 +804,14 @@ class AdamStepNode : public torch::autograd::Function<AdamStepNode> {
                 if (g_nu[i].defined()) via_nu.push_back(i);
             }
         }
-        auto pick = [](const TensorList &from, const std::vector<size_t> &idx) {
-            if (idx.size() == from.size()) return from;
+        auto pick = [this](const Tensor *from, const std::vector<size_t> &idx) {
             TensorList out;
             out.reserve(idx.size());
             for (size_t i : idx) out.push_back(from[i]);
             return out;
+        };
+        auto pick_list = [this, &pick](const TensorList &from, const std::vector<size_t> &idx) {
+            return idx.size() == k ? from : pick(from.data(), idx);
         };
         auto counts_of = [&](const std::vector<size_t> &idx) {
             if (counts.size() <= 1 || idx.size() == k) return countsOf(counts, k);
@@ -808,7 +825,7 @@ class AdamStepNode : public torch::autograd::Function<AdamStepNode> {
             // skips the addition, as autograd would.  Some: members without one get -0.0, the
             // exact identity of IEEE addition (x + -0.0 is x for every x, signed zeros
             // included), so they too come out as if nothing had been added.
-            auto outside = [&](const TensorList &gs) -> c10::optional<TensorList> {
+            auto outside = [&](const Tensor *gs) -> c10::optional<TensorList> {
                 bool any = false;
                 for (size_t i : live) any = any || gs[i].defined();
                 if (!any) return c10::nullopt;
@@ -819,8 +836,9 @@ class AdamStepNode : public torch::autograd::Function<AdamStepNode> {
                 return out;
             };
             auto [du, dm, dn] = backwardAllMultiImpl(
-                pick(g_u, live), outside(g_mu), outside(g_nu), pick(new_updates, live),
-                pick(new_mu, live), pick(updates, live), b1, b2, eps_root, counts_of(live));
+                pick(g_u, live), outside(g_mu), outside(g_nu), pick_list(new_updates, live),
+                pick_list(new_mu, live), pick_list(updates, live), b1, b2, eps_root,
+                counts_of(live));
             for (size_t j = 0; j < live.size(); ++j) {
                 dupdates[live[j]] = std::move(du[j]);
                 dmu[live[j]] = std::move(dm[j]);
@@ -828,7 +846,7 @@ class AdamStepNode : public torch::autograd::Function<AdamStepNode> {
             }
         }
         if (!via_mu.empty()) {
-            const TensorList donors = pick(updates, via_mu);
+            const TensorList donors = pick_list(updates, via_mu);
             auto [du, dm] = backwardMuMulti(pick(g_mu, via_mu), donors, donors, b1);
             for (size_t j = 0; j < via_mu.size(); ++j) {
                 dupdates[via_mu[j]] = std::move(du[j]);
@@ -836,7 +854,7 @@ class AdamStepNode : public torch::autograd::Function<AdamStepNode> {
             }
         }
         if (!via_nu.empty()) {
-            const TensorList donors = pick(updates, via_nu);
+            const TensorList donors = pick_list(updates, via_nu);
             auto [du, dn] = backwardNuMulti(pick(g_nu, via_nu), donors, donors, b2);
             for (size_t j = 0; j < via_nu.size(); ++j) {
                 const size_t i = via_nu[j];
@@ -848,23 +866,53 @@ class AdamStepNode : public torch::autograd::Function<AdamStepNode> {
         // Gradients nobody asked for (torch.autograd.grad with `inputs`, leaves that do not
         // require grad) are dropped here rather than checked and routed by the engine.
         for (size_t i = 0; i < 3 * k; ++i)
-            if (result[i].defined() && !ctx->needs_input_grad(i)) result[i] = Tensor();
+            if (result[i].defined() && !task_should_compute_output(i)) result[i] = Tensor();
         return result;
     }
-
-  private:
-    static Counts countsOf(const std::vector<int64_t> &values, size_t num) {
-        Counts c;
-        if (values.size() == 1) {
-            c.all = (uint64_t)values[0];
-        } else {
-            TORCH_CHECK(values.size() == num, "adamStep: expected ", num, " counts, got ",
-                        values.size());
-            c.each.assign(values.begin(), values.end());
-        }
-        return c;
-    }
 };
+
+// The forward of the node: new_mu, new_nu, new_updates of every leaf, in that order, with their
+// history set when any input requires a gradient (and gradients are being recorded).
+torch::autograd::variable_list adamStep(const TensorList &updates, const TensorList &mu,
+                                        const TensorList &nu, double b1, double b2, double eps,
+                                        double eps_root, std::vector<int64_t> counts) {
+    const auto &functorch_tls = at::functorch::functorchTLSAccessor();
+    // functorch transforms wrap custom nodes in Python; this one they would see through
+    if (functorch_tls) functorch_tls->checkSupportsCppAutogradFunction();
+    const size_t k = mu.size();
+    std::shared_ptr<AdamStepBackward> node;
+    if (torch::autograd::compute_requires_grad(updates, mu, nu)) {
+        node = std::shared_ptr<AdamStepBackward>(new AdamStepBackward(),
+                                                 torch::autograd::deleteNode);
+        node->set_next_edges(torch::autograd::collect_next_edges(updates, mu, nu));
+    }
+    std::tuple<TensorList, TensorList, TensorList> fresh;
+    {
+        // layout conversions of the inputs in there must not be recorded: the gradients this
+        // node returns are for the inputs as they came
+        at::AutoGradMode no_grad(false);
+        fresh = forwardAllMultiImpl(updates, mu, nu, b1, b2, eps, eps_root,
+                                    AdamStepBackward::countsOf(counts, k));
+    }
+    auto &[new_mu, new_nu, new_updates] = fresh;
+    torch::autograd::variable_list out;
+    out.reserve(3 * k);
+    for (TensorList *l : {&new_mu, &new_nu, &new_updates})
+        for (Tensor &t : *l) out.push_back(std::move(t));
+    if (node) {
+        for (const Tensor &t : out) torch::autograd::set_history(t, node);
+        node->k = k;
+        node->b1 = b1;
+        node->b2 = b2;
+        node->eps_root = eps_root;
+        node->counts = std::move(counts);
+        node->saved.reserve(3 * k);
+        for (size_t i = 0; i < k; ++i) node->saved.emplace_back(out[2 * k + i], /*is_output=*/true);
+        for (size_t i = 0; i < k; ++i) node->saved.emplace_back(out[i], /*is_output=*/true);
+        for (size_t i = 0; i < k; ++i) node->saved.emplace_back(updates[i], /*is_output=*/false);
+    }
+    return out;
+}
 
 // (new_mu, new_nu, new_updates) as lists, differentiable with respect to every tensor of the
 // three input lists.  `counts` as for the other list functions.
@@ -883,8 +931,7 @@ py::tuple stepMulti(const py::object &updates_o, const py::object &mu_o, const p
         values.assign(c.each.begin(), c.each.end());
     for (int64_t v : values)
         if (v < 0) throw py::type_error("counts beyond INT64_MAX are not served here");
-    const auto out = AdamStepNode::apply(at::TensorList(updates), at::TensorList(mu),
-                                         at::TensorList(nu), b1, b2, eps, eps_root, values);
+    const auto out = adamStep(updates, mu, nu, b1, b2, eps, eps_root, std::move(values));
     py::list lists[3];
     for (int j = 0; j < 3; ++j)
         for (size_t i = 0; i < k; ++i) lists[j].append(py::cast(out[j * k + i]));
