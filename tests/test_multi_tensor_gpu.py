@@ -120,6 +120,28 @@ def test_many_ragged_tensors_cross_table_capacity(dtype):
     run_all_multi(dtype, sizes, 77, 1e-8, 3)
 
 
+def test_shared_output_allocation_is_bounded():
+    """Small leaves' outputs share one allocation per call, up to 64 MiB: 200 leaves of 0.75 MiB
+    (150 MiB per output list) get results equal to the per-leaf op, outputs that overlap neither
+    one another nor the inputs, and no storage larger than the bound."""
+    n, num = 196_608, 200  # 0.75 MiB of float32 per leaf
+    gen = torch.Generator(device='cuda').manual_seed(11)
+    g = [torch.randn(n, device='cuda', generator=gen) for _ in range(num)]
+    mu = [0.1 * torch.randn(n, device='cuda', generator=gen) for _ in range(num)]
+    nu = [0.01 * torch.rand(n, device='cuda', generator=gen) for _ in range(num)]
+    new_mu, new_nu, new_u = adam_op.forward_all_multi(g, mu, nu, B1, B2, EPS, 1e-8, 3)
+    outs = new_mu + new_nu + new_u
+    assert max(t.untyped_storage().nbytes() for t in outs) <= 64 << 20
+    assert min(t.untyped_storage().nbytes() for t in outs) == 4 * n  # the rest: one each
+    assert all(t.data_ptr() % 256 == 0 for t in outs)
+    spans = sorted((t.data_ptr(), t.data_ptr() + 4 * n) for t in outs + g + mu + nu)
+    assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:]))
+    for k in (0, 27, 28, 29, 199):  # both sides of where the shared allocation ends
+        m1, v1, u1 = adam_op.forward_all(g[k], mu[k], nu[k], B1, B2, EPS, 1e-8, 3)
+        assert torch.equal(new_mu[k], m1) and torch.equal(new_nu[k], v1)
+        assert torch.equal(new_u[k], u1)
+
+
 def test_per_tensor_counts():
     """The API lets every leaf carry its own step count; tensors are grouped per count."""
     sizes = [1000, 17, 5000, 256, 3, 70_000, 999, 1]

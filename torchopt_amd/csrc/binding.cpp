@@ -441,8 +441,11 @@ Counts parseCounts(const py::object &counts, size_t num) {
 // bandwidth -- then costs one trip to the allocator instead of one per leaf and list (2-3 us
 // each).  The leaves do not overlap; what they share is the storage's lifetime (it lives as long
 // as any of them) and torch.save of a single leaf writing the whole storage.  Larger leaves get
-// an allocation each.
+// an allocation each, and so do the leaves that would take the shared allocation beyond 64 MiB:
+// what one surviving leaf can keep alive stays bounded, and past that size the step is no longer
+// bound by host time.
 constexpr size_t kPooledLeafBytes = (size_t)1 << 20;
+constexpr size_t kPoolMaxBytes = (size_t)64 << 20;
 
 std::vector<TensorList> emptyLikeSets(const TensorList &donors, size_t sets) {
     std::vector<TensorList> out(sets, TensorList(donors.size()));
@@ -456,9 +459,11 @@ std::vector<TensorList> emptyLikeSets(const TensorList &donors, size_t sets) {
             !d.is_non_overlapping_and_dense() || d.layout() != at::kStrided)
             continue;
         if (pooled != 0 && d.device() != donors[first].device()) continue;
+        const size_t padded = (need + 255) / 256 * 256;
+        if ((bytes + padded) * sets > kPoolMaxBytes) continue;
         if (pooled++ == 0) first = k;
         at[k] = bytes;
-        bytes += (need + 255) / 256 * 256;
+        bytes += padded;
     }
     if (pooled * sets >= 2) {
         const Tensor pool =
