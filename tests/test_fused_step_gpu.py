@@ -309,6 +309,51 @@ def test_16_bit_single_tensor_against_oracle(fmt, maximize, write_updates):
 
 
 @pytest.mark.parametrize('fmt', ['f16', 'bf16'])
+@pytest.mark.parametrize('operand', [0, 1, 2, 3], ids=['params', 'updates', 'mu', 'nu'])
+@pytest.mark.parametrize('maximize', [False, True])
+@pytest.mark.parametrize('lr', [0.05, 1e-3])
+def test_16_bit_every_bit_pattern_of_one_operand(fmt, operand, maximize, lr):
+    """All 65 536 values of the type (every denormal, infinity and NaN) in one operand, the
+    others random, through the element-wise kernel (65 536 elements) and the whole-tile kernel
+    (the same 128 times over): every conversion, rounding and sign case, the sign flip of
+    `maximize` included.  (This is the test that caught float16 steps rounded once where the CPU
+    rounds twice: parameter 0x09ae, direction 0x85d2, lr 0.05.)"""
+    for repeat in (1, 128):
+        n = (1 << 16) * repeat
+        h, d = rand4_16(fmt, n, 500 + operand)
+        every = torch.arange(n, dtype=torch.int32).to(torch.int16).view(TDT[fmt])
+        d[operand] = every.cuda()
+        h[operand] = bits16(every, fmt)
+        print(f'fused_step_ {fmt} every pattern in operand {operand} x {repeat} '
+              f'maximize={maximize} lr={lr}', flush=True)
+        adam_op.fused_step_(d[0], d[1], d[2], d[3], B1, B2, 1e-3, 1e-4, 3, lr,
+                            maximize=maximize, write_updates=True)
+        with np.errstate(all='ignore'):
+            O.fused_step(h[0], h[1], h[2], h[3], B1, B2, 1e-3, 1e-4, 3, lr, maximize, True)
+        for j, what in enumerate(('params', 'updates', 'mu', 'nu')):
+            assert_bit_equal(bits16(d[j], fmt), h[j], f'{fmt} all {operand} x {repeat} {what}')
+
+
+@pytest.mark.parametrize('fmt', ['f16', 'bf16'])
+@pytest.mark.parametrize('lr', [0.05, 1e-4, 1e-5, 2.5e-6])
+def test_16_bit_steps_down_to_the_denormal_range(fmt, lr):
+    """Small learning rates put float16 steps below 6.1e-5, the type's denormal range (with
+    lr = 1e-4 nine steps in ten are denormal); the float multiplication by -lr and the rounding
+    to 16 bits must stay two roundings there as everywhere, as on the CPU (a handful of
+    elements per run tell the difference).  Whole tiles and the element-wise kernel of short
+    and ragged tensors."""
+    for n in (1, 5, 777, (1 << 18), (1 << 18) + 13):
+        h, d = rand4_16(fmt, n, 4242 + n)
+        print(f'fused_step_ {fmt} n={n} lr={lr}', flush=True)
+        adam_op.fused_step_(d[0], d[1], d[2], d[3], B1, B2, 1e-3, 1e-4, 3, lr,
+                            maximize=False, write_updates=True)
+        with np.errstate(all='ignore'):
+            O.fused_step(h[0], h[1], h[2], h[3], B1, B2, 1e-3, 1e-4, 3, lr, False, True)
+        for j, what in enumerate(('params', 'updates', 'mu', 'nu')):
+            assert_bit_equal(bits16(d[j], fmt), h[j], f'{fmt} n={n} lr={lr} {what}')
+
+
+@pytest.mark.parametrize('fmt', ['f16', 'bf16'])
 def test_16_bit_step_equals_the_unfused_chain_on_the_gpu(fmt):
     """forward_ in place, then PyTorch's own GPU kernels for mul_(-lr) and add_."""
     n, lr, count = (1 << 21) + 5, 0.05, 9

@@ -161,6 +161,20 @@ struct R16 {
     }
     __host__ __device__ operator float() const { return F::decode(bits); }
 };
+// A float result that is about to be rounded to 16 bits, kept apart from that rounding.  The
+// reference rounds twice there -- the float operation to 24 bits, then the conversion to 16 -- and
+// the compiler would merge a float16 operand's widening, the float operation and the conversion
+// into ONE mixed-precision instruction (v_fma_mixlo_f16) that rounds once.  Between two 16-bit
+// operands that is the same value (a product is exact in float, a sum's double rounding is
+// innocuous); with a float operand of 24 significant bits (the step's -lr) it is not: 1490 x
+// 2^-24 times float(-0.05) is 74.5000011 units of 2^-24, which the float product rounds to the
+// tie 74.5 and the conversion to 74, where one rounding gives 75.
+__host__ __device__ inline float rounded_to_float(float x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("" : "+v"(x));
+#endif
+    return x;
+}
 #define TOA_R16_BINOP(OP)                                                                        \
     template <class F>                                                                           \
     __host__ __device__ inline R16<F> operator OP(R16<F> a, R16<F> b) {                          \
@@ -171,9 +185,13 @@ struct R16 {
         return R16<F>(a) OP b;                                                                   \
     }                                                                                            \
     template <class F>                                                                           \
-    __host__ __device__ inline float operator OP(R16<F> a, float b) { return (float)a OP b; }    \
+    __host__ __device__ inline float operator OP(R16<F> a, float b) {                            \
+        return rounded_to_float((float)a OP b);                                                  \
+    }                                                                                            \
     template <class F>                                                                           \
-    __host__ __device__ inline float operator OP(float a, R16<F> b) { return a OP(float) b; }    \
+    __host__ __device__ inline float operator OP(float a, R16<F> b) {                            \
+        return rounded_to_float(a OP(float) b);                                                  \
+    }                                                                                            \
     template <class F>                                                                           \
     __host__ __device__ inline double operator OP(R16<F> a, double b) {                          \
         return (double)(float)a OP b;                                                            \
@@ -250,7 +268,10 @@ struct Pair16<HalfFormat> {
         r.v = __builtin_bit_cast(Halves, p);
         return r;
     }
-    __device__ static Pair16 rounded(float a, float b) { return from_bits(HalfFormat::encode2(a, b)); }
+    __device__ static Pair16 rounded(float a, float b) {
+        // the floats are results of float operations: see rounded_to_float
+        return from_bits(HalfFormat::encode2(rounded_to_float(a), rounded_to_float(b)));
+    }
     __device__ uint32_t bits() const { return __builtin_bit_cast(uint32_t, v); }
     __device__ explicit Pair16(R16<HalfFormat> s) {
         // through integer arithmetic: picking a 16-bit field out of the op as a half vector makes
@@ -1104,7 +1125,7 @@ __device__ __forceinline__ double toa_fma(double a, double b, double c) { return
 // of these overloads is rounded when it is assigned to the 16-bit type.
 template <class F>
 __device__ __forceinline__ float toa_fma(float a, R16<F> b, R16<F> c) {
-    return __builtin_fmaf(a, (float)b, (float)c);
+    return rounded_to_float(__builtin_fmaf(a, (float)b, (float)c));
 }
 // The type the step's two scalars (-lr and the weight decay) are held in: the element type for
 // float32 / float64, float for the 16-bit types.
