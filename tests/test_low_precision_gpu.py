@@ -158,6 +158,79 @@ def test_quick_route_equals_exact_route_for_every_pair(tag, hyper):
     torch.cuda.empty_cache()
 
 
+def _as_one_nan(t):
+    nan = torch.tensor(0x7fff, dtype=torch.int16, device=t.device)
+    return torch.where(t.isnan(), nan, t.view(torch.int16))
+
+
+def _first_moment_in_float(mu, g, b1):
+    """b1*mu + (1-b1)*g the way c10::Half computes it -- every operation in float, each result
+    rounded to float16 -- with PyTorch's own kernels, one operation and one conversion per
+    kernel, so no instruction can merge an operation with its rounding."""
+    one_minus = float(torch.tensor(1.0, dtype=torch.float16) - torch.tensor(b1, dtype=torch.float16))
+    a = (mu.float() * b1).half()
+    b = (g.float() * one_minus).half()
+    return (a.float() + b.float()).half()
+
+
+def _first_moment(op, mu, g, b1):
+    """new_mu from the element-wise kernel (forward_mu, whose float16 operations the compiler
+    may merge with their roundings) or from the kernels that compute float16 in pairs
+    (forward_ in place: packed half instructions)."""
+    if op == 'forward_mu':
+        return adam_op.forward_mu(g, mu, b1)
+    new_mu = mu.clone()
+    adam_op.forward_(g.clone(), new_mu, torch.ones_like(mu), b1, 0.999, 1e-3, 0.0, 1)
+    return new_mu
+
+
+@pytest.mark.parametrize('op', ['forward_mu', 'forward_'])
+def test_half_sums_equal_float_sums_rounded_for_every_pair(op):
+    """float16 pairs are added with v_pk_add_f16, and single values by whatever the compiler
+    makes of widen-add-convert.  That both are the float addition rounded to float16 (what the
+    reference computes) for EVERY pair of operands: the first moment with b1 = 0.5 is
+    0.5*mu + 0.5*g, whose two halvings are exact for all but the smallest values, over all
+    2^32 (mu, g) pairs, against the same expression evaluated in float by separate PyTorch
+    kernels."""
+    every = torch.arange(65536, dtype=torch.int32, device='cuda').to(torch.int16)
+    rows = 1024
+    mu = every.repeat(rows).view(torch.float16)
+    for chunk in range(65536 // rows):
+        g = every[chunk * rows:(chunk + 1) * rows].repeat_interleave(65536).view(torch.float16)
+        got = _as_one_nan(_first_moment(op, mu, g, 0.5))
+        want = _as_one_nan(_first_moment_in_float(mu, g, 0.5))
+        if not torch.equal(got, want):
+            bad = (got != want).nonzero()[0].item()
+            raise AssertionError(
+                f'mu {mu.view(torch.int16)[bad].item() & 0xffff:#06x} g '
+                f'{g.view(torch.int16)[bad].item() & 0xffff:#06x}: got '
+                f'{got[bad].item() & 0xffff:#06x} want {want[bad].item() & 0xffff:#06x}')
+        del g, got, want
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize('op', ['forward_mu', 'forward_'])
+def test_half_products_equal_float_products_rounded_for_every_pair(op):
+    """... and v_pk_mul_f16 (or the compiler's widen-multiply-convert) the float multiplication
+    rounded to float16: b1*mu for float16 values of b1 in [0, 1) (every 5th, all of them around
+    the powers of two, every denormal) times every mu, with a zero gradient."""
+    every = torch.arange(65536, dtype=torch.int32, device='cuda').to(torch.int16)
+    mu = every.view(torch.float16)
+    g = torch.zeros(65536, dtype=torch.float16, device='cuda')
+    patterns = sorted(set(range(0, 0x3c00, 5))
+                      | {p + d for p in range(0x0400, 0x3c00, 0x0400) for d in range(-3, 4)}
+                      | set(range(0, 0x0410)))  # the denormal values of b1, all of them
+    for pattern in patterns:
+        b1 = float(torch.tensor(pattern, dtype=torch.int16).view(torch.float16))
+        got = _as_one_nan(_first_moment(op, mu, g, b1))
+        want = _as_one_nan(_first_moment_in_float(mu, g, b1))
+        if not torch.equal(got, want):
+            bad = (got != want).nonzero()[0].item()
+            raise AssertionError(f'b1 {pattern:#06x} mu {bad:#06x}: got '
+                                 f'{got[bad].item() & 0xffff:#06x} want '
+                                 f'{want[bad].item() & 0xffff:#06x}')
+
+
 @pytest.mark.parametrize('tag', ['f16', 'bf16'])
 def test_misaligned_views(tag):
     n = 30_001
