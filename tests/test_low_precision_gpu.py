@@ -164,19 +164,21 @@ def _as_one_nan(t):
 
 
 def _first_moment_in_float(mu, g, b1):
-    """b1*mu + (1-b1)*g the way c10::Half computes it -- every operation in float, each result
-    rounded to float16 -- with PyTorch's own kernels, one operation and one conversion per
-    kernel, so no instruction can merge an operation with its rounding."""
-    one_minus = float(torch.tensor(1.0, dtype=torch.float16) - torch.tensor(b1, dtype=torch.float16))
-    a = (mu.float() * b1).half()
-    b = (g.float() * one_minus).half()
-    return (a.float() + b.float()).half()
+    """b1*mu + (1-b1)*g the way c10::Half / c10::BFloat16 compute it -- every operation in
+    float, each result rounded to the 16-bit type -- with PyTorch's own kernels, one operation
+    and one conversion per kernel, so no instruction can merge an operation with its rounding."""
+    dt = mu.dtype
+    one_minus = float(torch.tensor(1.0, dtype=dt) - torch.tensor(b1, dtype=dt))
+    a = (mu.float() * b1).to(dt)
+    b = (g.float() * one_minus).to(dt)
+    return (a.float() + b.float()).to(dt)
 
 
 def _first_moment(op, mu, g, b1):
     """new_mu from the element-wise kernel (forward_mu, whose float16 operations the compiler
-    may merge with their roundings) or from the kernels that compute float16 in pairs
-    (forward_ in place: packed half instructions)."""
+    may merge with their roundings) or from the kernels that compute in pairs (forward_ in
+    place: packed half instructions for float16, one rounding instruction per pair for
+    bfloat16)."""
     if op == 'forward_mu':
         return adam_op.forward_mu(g, mu, b1)
     new_mu = mu.clone()
@@ -185,18 +187,20 @@ def _first_moment(op, mu, g, b1):
 
 
 @pytest.mark.parametrize('op', ['forward_mu', 'forward_'])
-def test_half_sums_equal_float_sums_rounded_for_every_pair(op):
+@pytest.mark.parametrize('tag', ['f16', 'bf16'])
+def test_sums_equal_float_sums_rounded_for_every_pair(tag, op):
     """float16 pairs are added with v_pk_add_f16, and single values by whatever the compiler
     makes of widen-add-convert.  That both are the float addition rounded to float16 (what the
     reference computes) for EVERY pair of operands: the first moment with b1 = 0.5 is
     0.5*mu + 0.5*g, whose two halvings are exact for all but the smallest values, over all
     2^32 (mu, g) pairs, against the same expression evaluated in float by separate PyTorch
-    kernels."""
+    kernels.  bfloat16, which adds in float and rounds with one instruction, likewise."""
+    dt = TORCH[tag]
     every = torch.arange(65536, dtype=torch.int32, device='cuda').to(torch.int16)
     rows = 1024
-    mu = every.repeat(rows).view(torch.float16)
+    mu = every.repeat(rows).view(dt)
     for chunk in range(65536 // rows):
-        g = every[chunk * rows:(chunk + 1) * rows].repeat_interleave(65536).view(torch.float16)
+        g = every[chunk * rows:(chunk + 1) * rows].repeat_interleave(65536).view(dt)
         got = _as_one_nan(_first_moment(op, mu, g, 0.5))
         want = _as_one_nan(_first_moment_in_float(mu, g, 0.5))
         if not torch.equal(got, want):
@@ -210,18 +214,22 @@ def test_half_sums_equal_float_sums_rounded_for_every_pair(op):
 
 
 @pytest.mark.parametrize('op', ['forward_mu', 'forward_'])
-def test_half_products_equal_float_products_rounded_for_every_pair(op):
+@pytest.mark.parametrize('tag', ['f16', 'bf16'])
+def test_products_equal_float_products_rounded_for_every_pair(tag, op):
     """... and v_pk_mul_f16 (or the compiler's widen-multiply-convert) the float multiplication
-    rounded to float16: b1*mu for float16 values of b1 in [0, 1) (every 5th, all of them around
-    the powers of two, every denormal) times every mu, with a zero gradient."""
+    rounded to 16 bits: b1*mu for values of b1 in [0, 1) (every 5th bit pattern, all of them
+    around the powers of two, every denormal) times every mu, with a zero gradient."""
+    dt = TORCH[tag]
     every = torch.arange(65536, dtype=torch.int32, device='cuda').to(torch.int16)
-    mu = every.view(torch.float16)
-    g = torch.zeros(65536, dtype=torch.float16, device='cuda')
-    patterns = sorted(set(range(0, 0x3c00, 5))
-                      | {p + d for p in range(0x0400, 0x3c00, 0x0400) for d in range(-3, 4)}
-                      | set(range(0, 0x0410)))  # the denormal values of b1, all of them
+    mu = every.view(dt)
+    g = torch.zeros(65536, dtype=dt, device='cuda')
+    one, binade = (0x3c00, 0x0400) if tag == 'f16' else (0x3f80, 0x0080)
+    patterns = sorted(p for p in set(range(0, one, 5))
+                      | {p + d for p in range(binade, one, binade) for d in range(-3, 4)}
+                      | set(range(0, binade + 16))  # the denormal values of b1, all of them
+                      if p < one)
     for pattern in patterns:
-        b1 = float(torch.tensor(pattern, dtype=torch.int16).view(torch.float16))
+        b1 = float(torch.tensor(pattern, dtype=torch.int16).view(dt))
         got = _as_one_nan(_first_moment(op, mu, g, b1))
         want = _as_one_nan(_first_moment_in_float(mu, g, b1))
         if not torch.equal(got, want):
