@@ -221,6 +221,30 @@ def test_sizes_against_oracle(tag, via):
 
 
 @pytest.mark.parametrize('tag', ['f32', 'f64'])
+def test_operands_over_the_whole_exponent_range(tag):
+    """Operands drawn uniformly over the finite BIT PATTERNS of the type -- every exponent equally
+    likely, denormals and values next to overflow included -- so that the division, the root and
+    the long product of backward_updates meet underflow, overflow and gradual underflow at
+    random; whole-tile kernel and ragged tail."""
+    route = ROUTES['module'](tag)
+    n = (1 << 22) + 37
+    rng = np.random.default_rng(20)
+    it, ft = (np.uint32, np.float32) if tag == 'f32' else (np.uint64, np.float64)
+    top = int(np.array(np.inf, ft).view(it))  # patterns below it: the finite non-negative values
+
+    def draw(nonneg=False):
+        bits = rng.integers(0, top, size=n, dtype=it)
+        if not nonneg:
+            bits |= rng.integers(0, 2, size=n, dtype=it) << it(8 * bits.itemsize - 1)
+        return bits.view(ft)
+
+    inp = {'updates': draw(), 'mu': draw(), 'nu': draw(nonneg=True), 'dmu': draw(),
+           'dnu': draw(), 'dupdates': draw()}
+    for hyper in ((0.9, 0.999, 1e-8, 0.0, 1), (0.9, 0.999, 1e-8, 1e-8, 4)):
+        check_all_seven(route, inp, hyper, f'{tag}/whole exponent range {hyper}')
+
+
+@pytest.mark.parametrize('tag', ['f32', 'f64'])
 def test_zero_mu_branch_and_specials_in_backward_updates(tag):
     dtype = NP[tag]
     inp = rand(dtype, 5000, 3)

@@ -72,6 +72,34 @@ def test_weight_decay_against_oracle(dtype, decoupled):
             assert_bit_equal(host(t), want, f'n={n} {what}')
 
 
+@pytest.mark.parametrize('dtype', [np.float32, np.float64], ids=['f32', 'f64'])
+@pytest.mark.parametrize('decay', [None, 'l2', 'decoupled'])
+def test_operands_over_the_whole_exponent_range(dtype, decay):
+    """Operands drawn uniformly over the finite bit patterns of the type (every exponent equally
+    likely, denormals and near-overflow values included): the step's fused multiply-adds,
+    division and root under underflow and overflow; whole-tile kernel and ragged tail."""
+    n = (1 << 22) + 37
+    rng = np.random.default_rng(21)
+    it = np.uint32 if dtype is np.float32 else np.uint64
+    top = int(np.array(np.inf, dtype).view(it))
+
+    def draw(nonneg=False):
+        bits = rng.integers(0, top, size=n, dtype=it)
+        if not nonneg:
+            bits |= rng.integers(0, 2, size=n, dtype=it) << it(8 * bits.itemsize - 1)
+        return bits.view(dtype)
+
+    p, g, m, v = draw(), draw(), draw(), draw(nonneg=True)
+    wd, decoupled = (0.0, False) if decay is None else (0.05, decay == 'decoupled')
+    gp, gg, gm, gv = dev(p), dev(g), dev(m), dev(v)
+    adam_op.fused_step_(gp, gg, gm, gv, B1, B2, EPS, 1e-8, 4, 0.01, maximize=True,
+                        write_updates=True, weight_decay=wd, decoupled=decoupled)
+    with np.errstate(all='ignore'):
+        O.fused_step(p, g, m, v, B1, B2, EPS, 1e-8, 4, 0.01, True, True, wd, decoupled)
+    for t, want, what in ((gp, p, 'params'), (gg, g, 'updates'), (gm, m, 'mu'), (gv, v, 'nu')):
+        assert_bit_equal(host(t), want, f'whole exponent range, decay {decay}: {what}')
+
+
 @pytest.mark.parametrize('decay', ['l2', 'decoupled'])
 def test_weight_decay_equals_the_unfused_chain_on_the_gpu(decay):
     """With PyTorch's own GPU kernels for the neighbours (add_ with alpha, mul_, add_)."""
