@@ -340,9 +340,19 @@ def test_one_pass_forward_and_backward_against_oracle_chain(tag):
     dtype = NP[tag]
     lib = _lib.load()
     stream = torch.cuda.current_stream().cuda_stream
-    for k, n in enumerate([1, 5, 257, 4099, 300_001]):
+    np.seterr(all='ignore')  # the last case overflows on purpose
+    for k, n in enumerate([1, 5, 257, 4099, 300_001, (1 << 22) + 37]):
         b1, b2, eps, er, c = HYPERS[k % 3]
         inp = rand(dtype, n, 900 + n)
+        if n > (1 << 22):  # the staged whole-tile kernels, on operands of every exponent
+            rng = np.random.default_rng(22)
+            it = np.uint32 if tag == 'f32' else np.uint64
+            top = int(np.array(np.inf, dtype).view(it))
+            for key in inp:
+                bits = rng.integers(0, top, size=n, dtype=it)
+                if key != 'nu':
+                    bits |= rng.integers(0, 2, size=n, dtype=it) << it(8 * bits.itemsize - 1)
+                inp[key] = bits.view(dtype)
         g = {key: dev(a) for key, a in inp.items()}
         e_mu, e_nu = O.forward_mu(inp['updates'], inp['mu'], b1), O.forward_nu(inp['updates'],
                                                                               inp['nu'], b2)
@@ -373,7 +383,9 @@ def test_one_pass_forward_and_backward_against_oracle_chain(tag):
                 outs[1].data_ptr(), outs[2].data_ptr(), stream)
             assert rc == 0
             for a, b in zip(outs, got):
-                assert torch.equal(a, b), f'{label}: C ABI and module disagree'
+                bits = torch.int32 if tag == 'f32' else torch.int64  # NaNs included
+                assert torch.equal(a.view(bits), b.view(bits)), \
+                    f'{label}: C ABI and module disagree'
 
 
 def test_empty_tensors():
