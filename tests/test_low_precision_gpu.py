@@ -283,6 +283,40 @@ def test_multi_tensor_and_autograd(tag):
 
 
 @pytest.mark.parametrize('tag', ['f16', 'bf16'])
+@pytest.mark.parametrize('operand', ['updates', 'mu', 'nu', 'dmu', 'dnu', 'dupdates'])
+def test_one_pass_ops_equal_the_seven_for_every_bit_pattern(tag, operand):
+    """forward_all / backward_all (one pass per direction) against the seven ops they fuse, with
+    every value of the type in one operand: the element-wise kernels (65 536 elements) and the
+    whole-tile ones (128 times that).  The seven are pinned to the oracle above; here GPU
+    results are compared with GPU results, NaNs as one value."""
+    b1, b2, eps, er, c = 0.9, 0.999, 1e-3, 1e-4, 3
+    for repeat in (1, 128):
+        n = 65536 * repeat
+        inp = draw(tag, n, 1200 + len(operand))
+        g = {k: dev(a, tag) for k, a in inp.items()}
+        every = torch.arange(n, dtype=torch.int32, device='cuda').to(torch.int16)
+        g[operand] = every.view(TORCH[tag])
+        new_mu = adam_op.forward_mu(g['updates'], g['mu'], b1)
+        new_nu = adam_op.forward_nu(g['updates'], g['nu'], b2)
+        new_u = adam_op.forward_updates(new_mu, new_nu, b1, b2, eps, er, c)
+        got = adam_op.forward_all(g['updates'], g['mu'], g['nu'], b1, b2, eps, er, c)
+        for a, b, what in zip(got, (new_mu, new_nu, new_u), ('new_mu', 'new_nu', 'new_updates')):
+            assert torch.equal(_as_one_nan(a), _as_one_nan(b)), f'{tag} x{repeat} {what}'
+        bm, bv = adam_op.backward_updates(g['dupdates'], new_u, new_mu, new_nu, b1, b2, er, c)
+        for has_m, has_v in [(False, False), (True, False), (False, True), (True, True)]:
+            tot_m = g['dmu'] + bm if has_m else bm
+            tot_v = g['dnu'] + bv if has_v else bv
+            du1, dmu = adam_op.backward_mu(tot_m, g['updates'], g['mu'], b1)
+            du2, dnu = adam_op.backward_nu(tot_v, g['updates'], g['nu'], b2)
+            got = adam_op.backward_all(g['dupdates'], g['dmu'] if has_m else None,
+                                       g['dnu'] if has_v else None, new_u, new_mu, g['updates'],
+                                       b1, b2, er, c)
+            for a, b, what in zip(got, (du1 + du2, dmu, dnu), ('dupdates', 'dmu', 'dnu')):
+                assert torch.equal(_as_one_nan(a), _as_one_nan(b)), \
+                    f'{tag} x{repeat} dm={has_m} dv={has_v} {what}'
+
+
+@pytest.mark.parametrize('tag', ['f16', 'bf16'])
 @pytest.mark.parametrize('eps', [-1e-3, -0.25, -4.0, float('nan')])
 def test_negative_eps_takes_the_exact_chain(tag, eps):
     """The quick route's error bound assumes root + eps does not cancel.  The raw ops accept a
