@@ -123,7 +123,7 @@ TOA_API int toa_adam_tuned_load_order(int dtype, const void *updates, const void
  * length, run as ONE launch over a device-resident table, a
  * "plan": one 96-byte record per tensor, written by small kernels that carry the records in
  * their arguments and cached per (device, stream, list) in memory the library allocates (at most
- * 4 plans per stream, 64 per process), with a coarse index from tiles to records in the launch's
+ * 16 plans per stream, 128 per process), with a coarse index from tiles to records in the launch's
  * own arguments (and, for lists of more than 1664 tensors, a finer one beside the records).  A call whose list is cached costs one launch and no other device work, and a
  * call whose arguments repeat the previous call's byte for byte (same arrays, same sizes, one step
  * count for all) skips the per-tensor host work as well: a few microseconds whatever the length.

@@ -92,55 +92,56 @@ void test_hit_and_lru() {
     Device dev;
     Cache cache(FakeBackend{&dev});
     bool fresh = false;
+    const int P = (int)toa::kPlanSlotsPerStream;
     std::vector<void *> mem;
-    for (int k = 0; k < 4; ++k) {
+    for (int k = 0; k < P; ++k) {
         Cache::Slot *s = cache.acquire(0, S(0), key_of(k), 1000, &fresh);
         EXPECT(s != nullptr && fresh);
         serve(cache, dev, s, fresh, S(0), key_of(k));
         mem.push_back(s->mem);
     }
-    EXPECT(cache.slots() == 4 && dev.allocs == 4);
+    EXPECT((int)cache.slots() == P && (int)dev.allocs == P);
     // hits: same memory, nothing to write
-    for (int k = 0; k < 4; ++k) {
+    for (int k = 0; k < P; ++k) {
         Cache::Slot *s = cache.acquire(0, S(0), key_of(k), 1000, &fresh);
         EXPECT(s != nullptr && !fresh && s->mem == mem[k]);
     }
-    // touch 0, then a fifth list evicts the least recently used: list 1
+    // touch 0, then one list more than the stream may keep evicts the least recently used: list 1
     cache.acquire(0, S(0), key_of(0), 1000, &fresh);
-    Cache::Slot *s = cache.acquire(0, S(0), key_of(9), 1000, &fresh);
+    Cache::Slot *s = cache.acquire(0, S(0), key_of(1000), 1000, &fresh);
     EXPECT(s != nullptr && fresh && s->mem == mem[1]);  // rewritten in place, same stream
-    serve(cache, dev, s, fresh, S(0), key_of(9));
-    EXPECT(cache.slots() == 4 && dev.allocs == 4 && dev.blocking_frees == 0);
+    serve(cache, dev, s, fresh, S(0), key_of(1000));
+    EXPECT((int)cache.slots() == P && (int)dev.allocs == P && dev.blocking_frees == 0);
     s = cache.acquire(0, S(0), key_of(1), 1000, &fresh);
     EXPECT(fresh);  // list 1 is gone
     // another stream gets slots of its own
     s = cache.acquire(0, S(1), key_of(0), 1000, &fresh);
-    EXPECT(s != nullptr && fresh && cache.slots() == 5);
+    EXPECT(s != nullptr && fresh && (int)cache.slots() == P + 1);
     // and so does another device
     s = cache.acquire(1, S(0), key_of(0), 1000, &fresh);
-    EXPECT(s != nullptr && fresh && cache.slots() == 6);
+    EXPECT(s != nullptr && fresh && (int)cache.slots() == P + 2);
 }
 
 void test_grow_parks_memory_until_its_readers_are_done() {
     Device dev;
     Cache cache(FakeBackend{&dev});
     bool fresh = false;
-    for (int k = 0; k < 4; ++k) {
+    for (int k = 0; k < (int)toa::kPlanSlotsPerStream; ++k) {
         Cache::Slot *s = cache.acquire(0, S(0), key_of(k), 1000, &fresh);
         serve(cache, dev, s, fresh, S(0), key_of(k));
     }
     const size_t live_before = dev.live.size();
-    // a longer fifth list: the evicted slot's memory is too small and still being read
-    Cache::Slot *s = cache.acquire(0, S(0), key_of(7), 100000, &fresh);
+    // one list more, and a longer one: the evicted slot's memory is too small and still being read
+    Cache::Slot *s = cache.acquire(0, S(0), key_of(1007), 100000, &fresh);
     EXPECT(s != nullptr && fresh && s->capacity >= 100000);
     EXPECT(dev.blocking_frees == 0);                 // nothing waited, nothing freed
     EXPECT(dev.live.size() == live_before + 1);      // the old block is parked, not gone
     EXPECT(cache.parked() == 1);
-    serve(cache, dev, s, fresh, S(0), key_of(7));
+    serve(cache, dev, s, fresh, S(0), key_of(1007));
     // while the stream has not drained the parked block is not handed out again
-    s = cache.acquire(0, S(0), key_of(8), 100000, &fresh);
+    s = cache.acquire(0, S(0), key_of(1008), 100000, &fresh);
     EXPECT(s != nullptr && fresh && cache.parked() == 2 && dev.blocking_frees == 0);
-    serve(cache, dev, s, fresh, S(0), key_of(8));
+    serve(cache, dev, s, fresh, S(0), key_of(1008));
     drain(dev, S(0));
     // now a small new list may reuse a parked block instead of allocating
     const size_t allocs = dev.allocs;
@@ -160,12 +161,12 @@ void test_full_table_takes_over_the_oldest_slot_through_a_blocking_free() {
         serve(cache, dev, s, fresh, S(i), key_of(1));
     }
     EXPECT(cache.slots() == toa::kPlanSlotsTotal);
-    // stream 0 is still running its launch when stream 100 needs a slot
-    Cache::Slot *s = cache.acquire(0, S(100), key_of(1), 1000, &fresh);
+    // stream 0 is still running its launch when a new stream needs a slot
+    Cache::Slot *s = cache.acquire(0, S(5000), key_of(1), 1000, &fresh);
     EXPECT(s != nullptr && fresh);           // never "no plan for good"
-    EXPECT(s->stream == S(100));
+    EXPECT(s->stream == S(5000));
     EXPECT(dev.blocking_frees == 1);         // stream 0's block went through the blocking free
-    serve(cache, dev, s, fresh, S(100), key_of(1));  // checks: no foreign reader of this memory
+    serve(cache, dev, s, fresh, S(5000), key_of(1));  // checks: no foreign reader of this memory
     EXPECT(cache.slots() == toa::kPlanSlotsTotal);
     // stream 0 lost its plan and gets a new one by taking over the next oldest (stream 1)
     s = cache.acquire(0, S(0), key_of(1), 1000, &fresh);
@@ -189,15 +190,15 @@ void test_remembered_calls() {
     EXPECT(cache.find_call(1, S(0), call) == nullptr);   // another device: no
     EXPECT(cache.find_call(0, S(0), key_of(43, 64)) == nullptr);
     // eviction forgets the call
-    for (int k = 2; k < 6; ++k) {
+    for (int k = 2; k < 2 + (int)toa::kPlanSlotsPerStream; ++k) {
         Cache::Slot *t = cache.acquire(0, S(0), key_of(k), 1000, &fresh);
         serve(cache, dev, t, fresh, S(0), key_of(k));
     }
     EXPECT(cache.find_call(0, S(0), call) == nullptr);
     // a failed write leaves neither key nor call behind
-    s = cache.acquire(0, S(0), key_of(9), 1000, &fresh);
+    s = cache.acquire(0, S(0), key_of(200), 1000, &fresh);
     cache.invalidate(s);
-    cache.acquire(0, S(0), key_of(9), 1000, &fresh);
+    cache.acquire(0, S(0), key_of(200), 1000, &fresh);
     EXPECT(fresh);
 }
 
@@ -223,7 +224,7 @@ void test_threads_share_a_stream() {
     std::map<void *, int> being_filled;  // block -> thread that is between fill and launch
     auto worker = [&](int id) {
         for (int round = 0; round < 2000; ++round) {
-            const Bytes key = key_of(16 * id + round % 7, 8 + (round % 3) * 4096);
+            const Bytes key = key_of(16 * id + round % 7, 8 + (round % 3) * 4096);  // 28 lists
             std::lock_guard<std::mutex> lock(cache.mutex());
             bool fresh = false;
             Cache::Slot *s = cache.acquire(0, S(0), key, key.size() * 8, &fresh);

@@ -85,7 +85,7 @@ def test_cached_plan_then_another_list_then_the_first_again():
     step_and_check(g1, h1, 5, 'list 1 with one array elsewhere')
     # more lists than a stream keeps plans for: the oldest is rewritten
     others = []
-    for k in range(6):
+    for k in range(18):  # a stream keeps 16
         s = ragged_sizes(130 + k, 20 + k)
         others.append((to_dev(make_lists(np.float32, s, 30 + k)), make_lists(np.float32, s, 30 + k)))
     for k, (g, h) in enumerate(others):

@@ -33,8 +33,8 @@
 
 namespace toa {
 
-constexpr size_t kPlanSlotsPerStream = 4;  // cached plans a stream may hold
-constexpr size_t kPlanSlotsTotal = 64;     // and the process as a whole
+constexpr size_t kPlanSlotsPerStream = 16;  // cached plans a stream may hold
+constexpr size_t kPlanSlotsTotal = 128;     // and the process as a whole
 
 // Backend:
 //   void *alloc(size_t bytes)                 device memory on the current device, nullptr on failure

@@ -681,9 +681,10 @@ int launch_multi(MakeOp make_op, size_t num_tensors,
             unsigned char *at = call.data();
             std::memcpy(at, head, sizeof(head));
             at += sizeof(head);
-            std::memcpy(at, n, row);
-            at += row;
+            // pointers first: two lists of one model differ there, not in their sizes, so a
+            // comparison with another list's remembered call ends at its first bytes
             for (int i = 0; i < Op::NPTR; ++i, at += row) std::memcpy(at, lists[i], row);
+            std::memcpy(at, n, row);
             int device = 0;
             if (hipGetDevice(&device) == hipSuccess) {
                 // lookup and launch are one step under the cache's mutex (plan_cache.hpp)
