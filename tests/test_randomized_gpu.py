@@ -107,6 +107,98 @@ def test_random_cases(seed):
             assert_bit_equal(full[off + n:], raw[k][off + n:], label + ' tail guard')
 
 
+_TOP = {'f32': (np.uint32, 0x7f800000), 'f64': (np.uint64, 0x7ff0000000000000),
+        'f16': (np.uint16, 0x7c00), 'bf16': (np.uint16, 0x7f80)}
+
+
+def draw(rng, tag, n, kind, nonneg=False):
+    """'bits': uniform over the finite bit patterns of the type (every exponent equally likely),
+    now and then with an infinity or a NaN; 'sparse': half the elements zero; else normal."""
+    if kind == 'bits':
+        it, top = _TOP[tag]
+        b = rng.integers(0, top + (3 if rng.random() < 0.3 else 0), size=n,
+                         dtype=np.uint64).astype(it)
+        if not nonneg:
+            sign = rng.integers(0, 2, size=n, dtype=np.uint64) << np.uint64(8 * b.itemsize - 1)
+            b |= sign.astype(it)
+        return b if tag == 'bf16' else b.view({'f32': np.float32, 'f64': np.float64,
+                                               'f16': np.float16}[tag])
+    x = 10.0 ** rng.uniform(-4, 2) * rng.standard_normal(n)
+    if kind == 'sparse':
+        x[rng.random(n) < 0.5] = 0.0
+    return to_fmt(np.abs(x) if nonneg else x, tag)
+
+
+@pytest.mark.parametrize('seed', range(int(os.environ.get('TOA_RANDOM_SEEDS', '4'))))
+def test_random_cases_of_the_optimizer_step_and_of_lists(seed):
+    """The fused optimizer step (single tensors and lists, every type, with `maximize`, with and
+    without the written-back update, weight decay for float32 / float64) and the in-place step
+    over ragged lists with per-tensor step numbers, on normal, half-zero and bit-pattern-uniform
+    operands, learning rates that are round decimal numbers among them."""
+    rng = np.random.default_rng(977 + seed)
+    for case in range(25):
+        tag = ['f32', 'f64', 'f16', 'bf16'][int(rng.integers(4))]
+        kind = str(rng.choice(['normal', 'bits', 'sparse']))
+        b1 = float(rng.choice([0.0, 0.5, 0.9, rng.uniform(0, 0.999)]))
+        b2 = float(rng.choice([0.0, 0.99, 0.999, rng.uniform(0, 0.9999)]))
+        eps = float(rng.choice([0.0, 1e-8, 1e-3, 10.0 ** rng.uniform(-8, -1)]))
+        er = float(rng.choice([0.0, 1e-8, 1e-4]))
+        count = int(rng.choice([1, 2, 10, 1000, 10 ** 6]))
+        lr = float(rng.choice([0.05, 0.1, 0.01, 1e-3, 3e-4, 1e-5, 10.0 ** rng.uniform(-6, 0)]))
+        mx, wu = bool(rng.integers(2)), bool(rng.integers(2))
+        wd, dec = 0.0, False
+        if tag in ('f32', 'f64') and rng.random() < 0.5:
+            wd, dec = 0.05, bool(rng.integers(2))
+        which = int(rng.integers(3))
+        label = (f'seed {seed} case {case}: {tag} {kind} b1={b1} b2={b2} eps={eps} er={er} '
+                 f'count={count} lr={lr} maximize={mx} write_updates={wu} wd={wd} '
+                 f'decoupled={dec} which={which}')
+        print(label, flush=True)
+        with np.errstate(all='ignore'):
+            if which == 0:  # one tensor through the fused step, at a random element offset
+                n = int(rng.choice([rng.integers(1, 600), rng.integers(1, 70_000),
+                                    rng.integers(1, 1_500_000)]))
+                off = int(rng.integers(0, 8))
+                raw = [draw(rng, tag, n + off, kind, nonneg=(j == 3)) for j in range(4)]
+                h = [a[off:].copy() for a in raw]
+                d = [dev(a, tag)[off:] for a in raw]
+                adam_op.fused_step_(d[0], d[1], d[2], d[3], b1, b2, eps, er, count, lr,
+                                    maximize=mx, write_updates=wu, weight_decay=wd,
+                                    decoupled=dec)
+                O.fused_step(h[0], h[1], h[2], h[3], b1, b2, eps, er, count, lr, mx, wu, wd, dec)
+                for j, what in enumerate(('params', 'updates', 'mu', 'nu')):
+                    assert_bit_equal(host(d[j], tag), h[j], f'{label} {what}')
+                continue
+            num = int(rng.integers(1, 200))
+            sizes = [int(x) for x in rng.choice([0, 1, 7, 255, 256, 513, 4096, 70_001], size=num)]
+            if rng.random() < 0.3:
+                sizes[int(rng.integers(num))] = int(rng.integers(1, 1_500_000))
+            counts = [int(rng.choice([1, 2, 1000])) for _ in sizes] if rng.random() < 0.5 else count
+            cl = counts if isinstance(counts, list) else [counts] * num
+            hs = [[draw(rng, tag, m, kind, nonneg=(j == 3)) for j in range(4)] for m in sizes]
+            ds = [[dev(a, tag) for a in h] for h in hs]
+            if which == 1:  # the fused step over a ragged list
+                adam_op.fused_step_multi_([d[0] for d in ds], [d[1] for d in ds],
+                                          [d[2] for d in ds], [d[3] for d in ds], b1, b2, eps, er,
+                                          counts, lr, maximize=mx, write_updates=wu,
+                                          weight_decay=wd, decoupled=dec)
+                for k, (h, d) in enumerate(zip(hs, ds)):
+                    if sizes[k]:
+                        O.fused_step(h[0], h[1], h[2], h[3], b1, b2, eps, er, cl[k], lr, mx, wu,
+                                     wd, dec)
+                        for j in range(4):
+                            assert_bit_equal(host(d[j], tag), h[j], f'{label} tensor {k}/{j}')
+            else:  # the in-place step over a ragged list
+                adam_op.forward_multi_([d[1] for d in ds], [d[2] for d in ds],
+                                       [d[3] for d in ds], b1, b2, eps, er, counts)
+                for k, (h, d) in enumerate(zip(hs, ds)):
+                    if sizes[k]:
+                        want = O.forward_inplace(h[1].copy(), h[2].copy(), h[3].copy(), b1, b2,
+                                                 eps, er, cl[k])
+                        for j in range(3):
+                            assert_bit_equal(host(d[j + 1], tag), want[j], f'{label} {k}/{j}')
+
+
 def test_tensor_longer_than_2_to_32_elements():
     """2^32 + 777 float16 elements per array (8 GiB each): element indices and byte offsets pass
     32 bits inside one launch.  Windows at the start, across the 2^32 boundary and at the ragged
