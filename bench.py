@@ -58,9 +58,9 @@ BYTES_PER_ELEM = {  # op -> number of arrays streamed (multiply by the element s
 # figures belong to the kernels as they were when the profile was taken; re-record them whenever
 # adam_kernels.hpp or the launch shape changes.
 RECORDED_TRAFFIC = {
-    2: (6442403377, 'profiles/forward_inplace_f32_config2_pmc_traffic.md'),
-    4: (8516265767, 'profiles/forward_inplace_multi_f32_config4_kernel_trace_and_traffic.md'),
-    5: (9935446877, 'profiles/fused_step_multi_f32_config5_kernel_trace_and_traffic.md'),
+    2: (6442409480, 'profiles/forward_inplace_f32_config2_pmc_traffic.md'),
+    4: (8516253697, 'profiles/forward_inplace_multi_f32_config4_kernel_trace_and_traffic.md'),
+    5: (9935440703, 'profiles/fused_step_multi_f32_config5_kernel_trace_and_traffic.md'),
 }
 
 B1, B2, EPS = 0.9, 0.999, 1e-8
