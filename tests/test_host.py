@@ -283,3 +283,14 @@ def test_state_placement_advice():
     mu, nu = state_zeros_like_tree([torch.ones(1 << 19), None, t], requires_grad=True)
     assert mu[1] is None and nu[1] is None and mu[0].storage_offset() == 0 and nu[2].stride() == t.stride()
     assert all(x.requires_grad and not x.any() for x in (mu[0], nu[0], mu[2], nu[2]))
+
+
+def test_recorded_traffic_figures_are_the_ones_in_the_profile_summaries():
+    """bench.py quotes counter traffic recorded by rocprofv3 runs; each figure must be the one its
+    named summary under profiles/ states."""
+    import bench
+
+    for cfg, (traffic, source) in bench.RECORDED_TRAFFIC.items():
+        text = open(os.path.join(REPO, source)).read()
+        spaced = f'{traffic:,}'.replace(',', ' ')
+        assert spaced in text or str(traffic) in text, (cfg, traffic, source)
