@@ -22,7 +22,8 @@ LIB = os.path.join(REPO, 'torchopt_amd', 'libtoa_adam.so')
 
 
 @pytest.fixture(scope='module')
-def kernels(tmp_path_factory):
+def code_object(tmp_path_factory):
+    """The gfx950 code object inside the built library, unbundled into a file of its own."""
     if not all(os.path.exists(t) for t in TOOLS):
         pytest.skip('needs the LLVM tools of ROCm')
     if not os.path.exists(LIB):
@@ -33,7 +34,12 @@ def kernels(tmp_path_factory):
                    check=True)
     subprocess.run([TOOLS[1], '--unbundle', '--type=o', f'--input={fatbin}',
                     '--targets=hipv4-amdgcn-amd-amdhsa--gfx950', f'--output={code}'], check=True)
-    notes = subprocess.run([TOOLS[2], '--notes', code], check=True, capture_output=True,
+    return code
+
+
+@pytest.fixture(scope='module')
+def kernels(code_object):
+    notes = subprocess.run([TOOLS[2], '--notes', code_object], check=True, capture_output=True,
                            text=True).stdout
     # one block per kernel, opened by "  - .first_key:"; the kernel's own keys are indented by
     # four spaces (those of its arguments deeper), in alphabetical order, `.name` among them
@@ -80,3 +86,19 @@ def test_whole_tile_kernels_fit_every_residency_level(kernels):
         pytest.skip('kernel names could not be demangled')
     for name, k in whole.items():
         assert k['vgpr_count'] <= 64, f'{name}: {k["vgpr_count"]} VGPRs, 32 waves per CU need 64'
+
+
+def test_no_packed_float32_arithmetic_and_no_fused_half_arithmetic(code_object):
+    """The library is built with packed float32 code generation off (some forms of
+    v_pk_add_f32 / v_pk_mul_f32 / v_pk_fma_f32 have given wrong results on this hardware) and
+    without contraction (every product and sum rounds on its own: no fused multiply-add may
+    appear in the packed half arithmetic of the float16 kernels either)."""
+    objdump = os.path.join(LLVM, 'llvm-objdump')
+    if not os.path.exists(objdump):
+        pytest.skip('needs llvm-objdump')
+    text = subprocess.run([objdump, '-d', '--no-show-raw-insn', code_object], check=True,
+                          capture_output=True, text=True).stdout
+    assert 'v_pk_mul_f16' in text and 'v_pk_add_f16' in text  # the float16 pairs are there
+    for banned in ('v_pk_add_f32', 'v_pk_mul_f32', 'v_pk_fma_f32', 'v_pk_fma_f16',
+                   'v_pk_mad_f16'):
+        assert banned not in text, banned
