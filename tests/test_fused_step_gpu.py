@@ -216,6 +216,35 @@ def test_fused_adam_tracks_torch_optim_adam(cls, ref_cls, wd):
         torch.testing.assert_close(p, q, rtol=25e-7, atol=25e-7)
 
 
+def test_fused_adam_one_go_path_equals_the_general_path():
+    """`step()` takes every parameter in one call when all have gradients and have stepped
+    together, and sorts them into buckets otherwise.  A run that moves between the two (a
+    gradient missing on the third step, everything present again afterwards) against a run held
+    on the general path throughout: parameters, moments and step numbers bit for bit."""
+    torch.manual_seed(5)
+    shapes = [(300,), (17, 9), (4096,), (1,)]
+    base = [torch.randn(s, device='cuda') for s in shapes]
+    runs = []
+    for general_only in (False, True):
+        ps = [b.clone().requires_grad_(True) for b in base]
+        opt = FusedAdam(ps, 0.01, eps_root=1e-8)
+        gen = torch.Generator(device='cuda').manual_seed(9)
+        for step in range(6):
+            if general_only:
+                opt._uniform = [False] * len(opt._uniform)
+            for k, p in enumerate(ps):
+                p.grad = torch.randn(p.shape, device='cuda', generator=gen)
+                if step == 2 and k == 1:
+                    p.grad = None
+            opt.step()
+        (state,) = opt.state_dict()
+        runs.append((ps, state))
+    (pa, sa), (pb, sb) = runs
+    assert [int(c) for c in sa.count] == [int(c) for c in sb.count] == [6, 5, 6, 6]
+    for a, b in zip(list(pa) + list(sa.mu) + list(sa.nu), list(pb) + list(sb.mu) + list(sb.nu)):
+        assert torch.equal(a, b)
+
+
 def test_fused_adam_reads_gradients_in_any_layout():
     """`p.grad` may be channels-last, expanded or a strided slice while the parameter is
     contiguous: the step only reads it, so it is brought to the parameter's memory order."""

@@ -34,6 +34,8 @@ refuses to run under capture.
 
 from __future__ import annotations
 
+from itertools import repeat
+from operator import is_
 from typing import Callable, Iterable, Sequence
 
 import torch
@@ -103,6 +105,7 @@ class FusedAdam:
         self._decays: list[list[bool]] = []       # whether weight decay applies, per parameter
         self._steps: list[list[int] | None] = []  # host-side step numbers per parameter
         self._stale: list[bool] = []              # device count tensors lag the host numbers
+        self._uniform: list[bool] = []            # the group's parameters form one bucket
         self.add_param_group(params)
 
     def add_param_group(self, params: Iterable[torch.Tensor]) -> None:
@@ -127,6 +130,9 @@ class FusedAdam:
                                      f'and float64 parameters only, got {p.dtype}')
         self._steps.append(None)
         self._stale.append(False)
+        # one bucket for the whole group: a single (device, dtype) and a single decay flag
+        self._uniform.append(len(group) > 0 and len(set(self._kinds[-1])) == 1
+                             and len(set(self._decays[-1])) == 1)
 
     def zero_grad(self, set_to_none: bool = False) -> None:
         for group in self.param_groups:
@@ -290,6 +296,22 @@ class FusedAdam:
                 self.state_groups[i] = self._init_state(i)
             state, steps = self.state_groups[i], self._steps[i]
             grads = [p.grad for p in group]
+            if (self._uniform[i] and not scheduled and steps.count(steps[0]) == len(steps)
+                    and not any(map(is_, grads, repeat(None)))):
+                # the usual step in one go: every parameter has a gradient, the group is one
+                # bucket (one device and type, one decay flag) and has stepped together so far
+                c = steps[0]
+                if c != INT64_MAX:
+                    c += 1
+                    steps[:] = [c] * len(steps)
+                self._stale[i] = True
+                adam_op.fused_step_multi_(
+                    list(group), grads, list(state.mu), list(state.nu), self.b1, self.b2,
+                    self.eps, self.eps_root, c, self.lr, maximize=self.maximize,
+                    write_updates=False,
+                    weight_decay=self.weight_decay if self._decays[i][0] else 0.0,
+                    decoupled=self._decoupled)
+                continue
             live = [k for k, g in enumerate(grads) if g is not None]
             if not live:
                 continue
