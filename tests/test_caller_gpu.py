@@ -118,6 +118,37 @@ def test_flat_variant_matches_tree_variant():
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize('kind', [dict, collections.OrderedDict])
+@pytest.mark.parametrize('inplace', [True, False])
+def test_dicts_of_tensors_step_like_tuples_whatever_their_key_order(kind, inplace):
+    """A plain dict of tensors (`dict(module.named_parameters())`) is flattened without the
+    general tree walk; it must step exactly as the tuple of its values does, keep its type and
+    keys, and line gradients up with the state BY NAME when their dict was built in another
+    order (the reference's pytree library sorts dict keys, so order never matters there)."""
+    torch.manual_seed(8)
+    names = ['w2', 'b2', 'w1', 'b1', 'emb']
+    shapes = [(7, 5), (7,), (5, 3), (5,), (300,)]
+    params = kind((n, torch.randn(s, device='cuda')) for n, s in zip(names, shapes))
+    t = scale_by_accelerated_adam(B1, B2, EPS, 1e-8)
+    as_dict, as_tuple = t.init(params), t.init(tuple(params.values()))
+    assert type(as_dict.mu) is kind and list(as_dict.mu) == names and list(as_dict.count) == names
+    for step in range(3):
+        grads = [torch.randn(s, device='cuda') for s in shapes]
+        order = list(range(len(names))) if step != 1 else [3, 0, 4, 2, 1]  # shuffled once
+        gd = kind((names[k], grads[k].clone()) for k in order)
+        ud, as_dict = t.update(gd, as_dict, inplace=inplace)
+        ut, as_tuple = t.update(tuple(g.clone() for g in grads), as_tuple, inplace=inplace)
+        assert type(ud) is kind and sorted(ud) == sorted(names)
+        for k, n in enumerate(names):
+            assert torch.equal(ud[n], ut[k]), (step, n)
+            assert torch.equal(as_dict.mu[n], as_tuple.mu[k])
+            assert torch.equal(as_dict.nu[n], as_tuple.nu[k])
+            assert int(as_dict.count[n]) == int(as_tuple.count[k]) == step + 1
+    bad = kind((n + '_', g) for n, g in zip(names, grads))
+    with pytest.raises(ValueError, match='different keys'):
+        t.update(bad, as_dict, inplace=inplace)
+
+
 def test_count_state_restored_from_elsewhere_is_read_once():
     """Counts that did not come from this transformation (a loaded checkpoint) carry no host
     mirror: they are read from the device, and the step uses their value."""

@@ -518,6 +518,29 @@ TensorList toTensorList(const py::object &o, const char *what) {
     return out;
 }
 
+// True when `o` is a non-empty list or tuple whose members are all tensors of one device and one
+// dtype: what a caller must know before it hands a whole tree to one list call, asked in C
+// instead of a Python loop over the leaves.
+bool oneKind(const py::object &o) {
+    PyObject *seq = o.ptr();
+    const bool is_list = PyList_Check(seq);
+    if (!is_list && !PyTuple_Check(seq)) return false;
+    const Py_ssize_t num = is_list ? PyList_GET_SIZE(seq) : PyTuple_GET_SIZE(seq);
+    if (num == 0) return false;
+    const Tensor *first = nullptr;
+    for (Py_ssize_t k = 0; k < num; ++k) {
+        PyObject *item = is_list ? PyList_GET_ITEM(seq, k) : PyTuple_GET_ITEM(seq, k);
+        if (!THPVariable_Check(item)) return false;
+        const Tensor &t = THPVariable_Unpack(item);
+        if (!t.defined()) return false;
+        if (first == nullptr)
+            first = &t;
+        else if (t.scalar_type() != first->scalar_type() || t.device() != first->device())
+            return false;
+    }
+    return true;
+}
+
 py::tuple forwardMultiInplace(const py::object &updates_o, const py::object &mu_o,
                               const py::object &nu_o, double b1, double b2, double eps,
                               double eps_root, const py::object &counts) {
@@ -1139,6 +1162,10 @@ PYBIND11_MODULE(_C, mod) {
     m.def("backward_all_multi", &backwardAllMulti, "backward_all over lists", "dnew_updates"_a,
           "dnew_mu"_a, "dnew_nu"_a, "new_updates"_a, "new_mu"_a, "updates"_a, "b1"_a, "b2"_a,
           "eps_root"_a, "counts"_a);
+
+    m.def("one_kind", &oneKind,
+          "whether a list or tuple holds only tensors, all of one device and one dtype",
+          "tensors"_a);
 
     m.def("step_multi", &stepMulti,
           "the differentiable step of a whole list as one autograd node -> "
