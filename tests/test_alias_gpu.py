@@ -246,3 +246,34 @@ def test_adamw_mask_decays_only_the_chosen_leaves(inplace):
         optim_ref.step()
     for p, q in zip(model.parameters(), ref.parameters()):
         torch.testing.assert_close(p, q, **TOL)
+
+
+@pytest.mark.parametrize('inplace', [True, False])
+@pytest.mark.parametrize('make', [lambda: topt.adam(0.01, weight_decay=0.1, maximize=True),
+                                  lambda: topt.adamw(0.01, weight_decay=0.1),
+                                  lambda: topt.adam(lambda c: 0.01 / (1 + c))],
+                         ids=['adam', 'adamw', 'schedule'])
+def test_dict_trees_are_matched_by_name_through_the_whole_chain(make, inplace):
+    """Parameters, gradients and state as flat dicts whose insertion orders differ: every
+    transformation of the chain and `apply_updates` pair leaves by name (the reference's pytree
+    library sorts dict keys), so the run equals the same run on tuples."""
+    torch.manual_seed(4)
+    names = ['c', 'a', 'd', 'b']
+    shapes = [(5, 3), (7,), (2, 2, 2), (300,)]
+    values = [torch.randn(s, device='cuda', dtype=torch.float64) for s in shapes]
+    pd = {n: v.clone() for n, v in zip(names, values)}
+    pt = tuple(v.clone() for v in values)
+    od, ot = make(), make()
+    sd, st = od.init(pd), ot.init(pt)
+    for step in range(3):
+        grads = [torch.randn(s, device='cuda', dtype=torch.float64) for s in shapes]
+        order = [2, 0, 3, 1] if step % 2 else [0, 1, 2, 3]
+        gd = {names[k]: grads[k].clone() for k in order}
+        ud, sd = od.update(gd, sd, params=pd, inplace=inplace)
+        ut, st = ot.update(tuple(g.clone() for g in grads), st, params=pt, inplace=inplace)
+        pd = topt.apply_updates(pd, ud, inplace=inplace)
+        pt = topt.apply_updates(pt, ut, inplace=inplace)
+        assert sorted(pd) == sorted(names)
+        for k, n in enumerate(names):
+            assert torch.equal(ud[n], ut[k]), (step, n, 'update')
+            assert torch.equal(pd[n], pt[k]), (step, n, 'parameter')

@@ -16,16 +16,19 @@ place so gradients flow, and with one fused list call per transformation in plac
 the transformations and keeps one state per transformation; `apply_updates`
 (/root/reference/torchopt/update.py:50-81) adds updates to parameters.
 
-Trees are plain containers flattened with ``torch.utils._pytree`` (``None`` is a leaf).
+Trees are plain containers (``None`` is a leaf), flattened by `torchopt_amd._tree`: flat lists,
+tuples and dicts of tensors directly, anything else with ``torch.utils._pytree``.
 """
 
 from __future__ import annotations
 
+from itertools import repeat
+from operator import is_
 from typing import Any, Callable, NamedTuple
 
 import torch
-from torch.utils import _pytree as pytree
 
+from torchopt_amd._tree import flatten, leaves_like, rebuild
 from torchopt_amd.base import GradientTransformation, accelerated_only
 from torchopt_amd.transform.scale_by_adam import _inc_counts, _remember, scale_by_accelerated_adam
 
@@ -45,16 +48,18 @@ class ScaleByScheduleState(NamedTuple):
 
 def _map_leaves(fn: Callable, tree: Any, *rest: Any) -> Any:
     """``fn`` over corresponding leaves; a ``None`` in the first tree stays ``None``."""
-    leaves, spec = pytree.tree_flatten(tree)
-    others = [pytree.tree_flatten(r)[0] for r in rest]
+    leaves, spec = flatten(tree)
+    others = [leaves_like(r, spec) for r in rest]
     out = [None if x is None else fn(x, *(o[k] for o in others)) for k, x in enumerate(leaves)]
-    return pytree.tree_unflatten(out, spec)
+    return rebuild(out, tree, spec)
 
 
 def _tensors(tree: Any, *rest: Any):
     """Parallel lists of the non-``None`` leaves of `tree` and their partners in `rest`."""
-    leaves = pytree.tree_flatten(tree)[0]
-    others = [pytree.tree_flatten(r)[0] for r in rest]
+    leaves, spec = flatten(tree)
+    others = [leaves_like(r, spec) for r in rest]
+    if not any(map(is_, leaves, repeat(None))):
+        return leaves, others
     keep = [k for k, x in enumerate(leaves) if x is not None]
     return [leaves[k] for k in keep], [[o[k] for k in keep] for o in others]
 
@@ -134,11 +139,11 @@ def _add_decayed_weights(weight_decay: float, mask: Any = None) -> GradientTrans
         if mask is None:
             chosen = None
         else:
-            chosen = pytree.tree_flatten(mask(params) if callable(mask) else mask)[0]
+            chosen = leaves_like(mask(params) if callable(mask) else mask, flatten(updates)[1])
         if inplace:
             gs, (ps,) = _tensors(updates, params)
             if chosen is not None:
-                keep = [k for k, x in enumerate(pytree.tree_flatten(updates)[0]) if x is not None]
+                keep = [k for k, x in enumerate(flatten(updates)[0]) if x is not None]
                 picked = [j for j, k in enumerate(keep) if chosen[k]]
                 gs, ps = [gs[j] for j in picked], [ps[j] for j in picked]
             if gs:
@@ -147,11 +152,11 @@ def _add_decayed_weights(weight_decay: float, mask: Any = None) -> GradientTrans
         if chosen is None:
             return _map_leaves(lambda g, p: g.add(p, alpha=weight_decay), updates, params)
         marks = iter(chosen)
-        leaves, spec = pytree.tree_flatten(updates)
-        p_leaves = pytree.tree_flatten(params)[0]
+        leaves, spec = flatten(updates)
+        p_leaves = leaves_like(params, spec)
         out = [g if (g is None or not m) else g.add(p, alpha=weight_decay)
                for g, p, m in zip(leaves, p_leaves, marks)]
-        return pytree.tree_unflatten(out, spec)
+        return rebuild(out, updates, spec)
 
     return _stateless(update)
 
@@ -182,9 +187,9 @@ def _scale_by_neg_lr(lr) -> GradientTransformation:
             return g.mul_(step) if inplace else g.mul(step)
 
         new_updates = _map_leaves(scale, updates, state.count)
-        c_leaves, c_spec = pytree.tree_flatten(state.count)
-        new_counts, _ = _inc_counts(c_leaves, pytree.tree_flatten(updates)[0])
-        return new_updates, ScaleByScheduleState(count=pytree.tree_unflatten(new_counts, c_spec))
+        c_leaves, c_spec = flatten(state.count)
+        new_counts, _ = _inc_counts(c_leaves, leaves_like(updates, c_spec))
+        return new_updates, ScaleByScheduleState(count=rebuild(new_counts, state.count, c_spec))
 
     return GradientTransformation(init_fn, update_fn)
 
@@ -251,12 +256,12 @@ def adamw(
 
 def apply_updates(params: Any, updates: Any, *, inplace: bool = True) -> Any:
     """``params + updates`` leaf by leaf; a ``None`` update leaves its parameter as it is."""
-    p_leaves, spec = pytree.tree_flatten(params)
-    u_leaves = pytree.tree_flatten(updates)[0]
+    p_leaves, spec = flatten(params)
+    u_leaves = leaves_like(updates, spec)
     if inplace:
         pairs = [(p, u) for p, u in zip(p_leaves, u_leaves) if p is not None and u is not None]
         if pairs:
             torch._foreach_add_([p.data for p, _ in pairs], [u for _, u in pairs])
         return params
     out = [p if (p is None or u is None) else p.add(u) for p, u in zip(p_leaves, u_leaves)]
-    return pytree.tree_unflatten(out, spec)
+    return rebuild(out, params, spec)

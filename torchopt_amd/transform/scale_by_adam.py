@@ -29,14 +29,13 @@ Trees are plain Python containers (dict / list / tuple / namedtuple, flattened w
 
 from __future__ import annotations
 
-from collections import OrderedDict
 from itertools import repeat
 from operator import is_
 from typing import Any, NamedTuple, Sequence
 
 import torch
-from torch.utils import _pytree as pytree
 
+from torchopt_amd import _tree
 from torchopt_amd.accelerated_op import MultiAdamOp
 from torchopt_amd.accelerated_op.adam_op import adam_op
 from torchopt_amd.base import GradientTransformation
@@ -47,15 +46,6 @@ __all__ = ['ScaleByAdamState', 'scale_by_accelerated_adam']
 
 INT64_MAX = torch.iinfo(torch.int64).max
 _MIRROR = '_toa_host_value'
-# exact leaf types a flat list may hold to count as already flattened (checked in C, per call)
-_PLAIN_LEAVES = frozenset({torch.Tensor, torch.nn.Parameter, type(None)})
-
-
-class _DictSpec(NamedTuple):
-    """How to put a flat dict back together: its type (dict or OrderedDict) and its keys."""
-
-    kind: type
-    keys: tuple
 
 
 class ScaleByAdamState(NamedTuple):
@@ -193,24 +183,11 @@ def _scale_by_accelerated_adam(
            for flag in (False, True)}
 
     def flatten(tree):
-        # A plain list / tuple of tensors and Nones is its own flattening, and a plain dict of
-        # them (what `dict(module.named_parameters())` is) flattens to its values in insertion
-        # order, as torch.utils._pytree has it; the general walk (pure Python there) costs
-        # ~0.5 us per leaf per tree and direction, eight times per update.
-        kind = type(tree)
-        if already_flattened or (kind in (list, tuple)
-                                 and _PLAIN_LEAVES.issuperset(map(type, tree))):
+        if already_flattened:
             return list(tree), None
-        if kind in (dict, OrderedDict) and _PLAIN_LEAVES.issuperset(map(type, tree.values())):
-            return list(tree.values()), _DictSpec(kind, tuple(tree.keys()))
-        return pytree.tree_flatten(tree)
+        return _tree.flatten(tree)
 
-    def rebuild(leaves, like, spec):
-        if spec is None:
-            return leaves if type(like) is list else type(like)(leaves)
-        if type(spec) is _DictSpec:
-            return spec.kind(zip(spec.keys, leaves))
-        return pytree.tree_unflatten(leaves, spec)
+    rebuild = _tree.rebuild
 
     def init_fn(params):
         leaves, spec = flatten(params)
@@ -254,15 +231,11 @@ def _scale_by_accelerated_adam(
         mu_leaves, mu_spec = flatten(state.mu)
         nu_leaves, nu_spec = flatten(state.nu)
         c_leaves, c_spec = flatten(state.count)
-        if (type(g_spec) is _DictSpec and type(mu_spec) is _DictSpec
+        if (type(g_spec) is _tree.DictSpec and type(mu_spec) is _tree.DictSpec
                 and g_spec.keys != mu_spec.keys):
-            # the same names in another order (the reference's pytree library sorts the keys of
-            # a dict, so order never matters there): line the gradients up with the state
-            if len(g_spec.keys) != len(mu_spec.keys) or set(g_spec.keys) != set(mu_spec.keys):
-                raise ValueError('updates and optimizer state are dicts with different keys; '
-                                 'make sure `init` was called on matching parameters')
-            g_leaves = [updates[k] for k in mu_spec.keys]
-            g_spec = _DictSpec(g_spec.kind, mu_spec.keys)
+            # the same names in another order: line the gradients up with the state
+            g_leaves = _tree.leaves_like(updates, mu_spec)
+            g_spec = _tree.DictSpec(g_spec.kind, mu_spec.keys)
         n = len(g_leaves)
         if not (len(mu_leaves) == len(nu_leaves) == len(c_leaves) == n):
             raise ValueError('updates and optimizer state have different tree structures; '
