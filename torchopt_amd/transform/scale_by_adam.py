@@ -23,8 +23,10 @@ Here the whole tree goes to the multi-tensor entry points (one launch per op for
 hundred leaves), the counts are advanced with one fused launch, and their values are mirrored on
 the host so no step reads them back from the device.
 
-Trees are plain Python containers (dict / list / tuple / namedtuple, flattened with
-``torch.utils._pytree``, where ``None`` is a leaf).
+Trees are plain Python containers (dict / list / tuple / namedtuple; ``None`` is a leaf),
+flattened by `torchopt_amd._tree`: flat lists, tuples and dicts of tensors directly -- dicts
+matched by name, as the reference's key-sorting pytree library has it -- and anything nested with
+``torch.utils._pytree``.
 """
 
 from __future__ import annotations
